@@ -1,0 +1,173 @@
+"""ctypes binding of ``libgelib_hip.so`` (the C ABI declared in ``include/gelib_hip.h``).
+
+Tensors are ``torch.complex64`` on the GPU with shape ``(batch, [grid...], 2l+1, channels)``; they are
+passed as 5-D descriptors of pointer, dims and strides.  Every call is queued on torch's current HIP
+stream.  A missing library or a non-zero status raises; nothing here falls back to another implementation.
+"""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libgelib_hip.so")
+
+SYMBOLS = [
+    "gelib_hip_strerror", "gelib_hip_last_runtime_error", "gelib_hip_version", "gelib_hip_cg_matrix",
+    "gelib_hip_so3type_product",
+    "gelib_hip_so3part_cg_fwd", "gelib_hip_so3part_cg_back0", "gelib_hip_so3part_cg_back1",
+    "gelib_hip_so3part_diagcg_fwd", "gelib_hip_so3part_diagcg_back0", "gelib_hip_so3part_diagcg_back1",
+    "gelib_hip_so3vec_cg_fwd", "gelib_hip_so3vec_cg_bwd", "gelib_hip_so3vec_diagcg_fwd",
+    "gelib_hip_so3vec_diagcg_bwd", "gelib_hip_set_option", "gelib_hip_last_path",
+]
+
+
+class PartDesc(ctypes.Structure):
+    _fields_ = [("ptr", ctypes.c_void_p), ("dims", ctypes.c_int64 * 5), ("strides", ctypes.c_int64 * 5)]
+
+
+class GelibHipError(RuntimeError):
+    def __init__(self, status, message):
+        super().__init__("GElib error: %s (status %d)" % (message, status))
+        self.status = status
+
+
+_lib = None
+
+
+def lib():
+    """Load the library; raises OSError with the build hint if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise OSError("%s is missing: build it with `make -C gelib_amd/csrc` "
+                          "(or `python -c 'import __graft_entry__ as g; g.build()'`)" % LIB_PATH)
+        L = ctypes.CDLL(LIB_PATH)
+        P = ctypes.POINTER(PartDesc)
+        for name in ("gelib_hip_strerror", "gelib_hip_last_runtime_error", "gelib_hip_version"):
+            getattr(L, name).restype = ctypes.c_char_p
+        L.gelib_hip_strerror.argtypes = [ctypes.c_int]
+        L.gelib_hip_cg_matrix.argtypes = [ctypes.c_int] * 3 + [ctypes.c_void_p]
+        L.gelib_hip_so3type_product.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_int),
+                                                ctypes.POINTER(ctypes.c_int), ctypes.c_int,
+                                                ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int),
+                                                ctypes.c_int, ctypes.POINTER(ctypes.c_int64), ctypes.c_int]
+        for name in SYMBOLS[5:11]:
+            getattr(L, name).argtypes = [P, P, P, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]
+        for name in ("gelib_hip_so3vec_cg_fwd", "gelib_hip_so3vec_diagcg_fwd"):
+            getattr(L, name).argtypes = [ctypes.c_int, P, ctypes.c_int, P, ctypes.c_int, P, ctypes.c_int,
+                                         ctypes.c_void_p]
+        for name in ("gelib_hip_so3vec_cg_bwd", "gelib_hip_so3vec_diagcg_bwd"):
+            getattr(L, name).argtypes = [P, P, ctypes.c_int, P, ctypes.c_int, P, ctypes.c_int, P, ctypes.c_int,
+                                         ctypes.c_void_p]
+        L.gelib_hip_set_option.argtypes = [ctypes.c_char_p, ctypes.c_int]
+        _lib = L
+    return _lib
+
+
+def check(status):
+    if status != 0:
+        L = lib()
+        msg = L.gelib_hip_strerror(status).decode()
+        if status == 10:
+            msg += ": " + L.gelib_hip_last_runtime_error().decode()
+        raise GelibHipError(status, msg)
+
+
+def desc(t):
+    """5-D descriptor of a complex64 tensor shaped (b, [g0, [g1]], 2l+1, n)."""
+    import torch
+    if t.dtype != torch.complex64:
+        raise TypeError("SO3parts are complex64 tensors")
+    if t.dim() < 3 or t.dim() > 5:
+        raise ValueError("an SO3part view has 3 to 5 dimensions (batch, [grid], 2l+1, channels)")
+    d = PartDesc()
+    d.ptr = t.data_ptr() if t.numel() > 0 else None
+    shape = list(t.shape)
+    strides = list(t.stride())
+    k = t.dim() - 3
+    dims = [shape[0]] + shape[1:1 + k] + [1] * (2 - k) + shape[-2:]
+    strs = [strides[0]] + strides[1:1 + k] + [0] * (2 - k) + strides[-2:]
+    for i in range(5):
+        d.dims[i] = dims[i]
+        d.strides[i] = strs[i]
+    return d
+
+
+def _stream(t):
+    import torch
+    dev = t.device if t.is_cuda else None      # a host tensor is refused by the library itself (status 8)
+    return ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+
+
+def _arr(tensors):
+    if tensors is None:
+        return None
+    return (PartDesc * len(tensors))(*[desc(t) for t in tensors])
+
+
+def cg_matrix(l1, l2, l):
+    import numpy as np
+    out = np.zeros((2 * l1 + 1, 2 * l2 + 1), dtype=np.float32)
+    check(lib().gelib_hip_cg_matrix(l1, l2, l, out.ctypes.data))
+    return out
+
+
+def so3type_product(taux, tauy, maxl=-1, diag=False):
+    lx, ly = sorted(taux), sorted(tauy)
+    n = (max(lx) + max(ly) + 1) if lx and ly else 0
+    out = (ctypes.c_int64 * max(n, 1))()
+    I = ctypes.c_int
+    rc = lib().gelib_hip_so3type_product(int(diag), len(lx), (I * len(lx))(*lx), (I * len(lx))(*[taux[l] for l in lx]),
+                                         len(ly), (I * len(ly))(*ly), (I * len(ly))(*[tauy[l] for l in ly]), maxl, out, n)
+    if rc < 0:
+        check(-rc)
+    return {l: int(out[l]) for l in range(n) if out[l] > 0}
+
+
+def _part(name, dst, a, b, offs, accumulate):
+    check(getattr(lib(), name)(ctypes.byref(desc(dst)), ctypes.byref(desc(a)), ctypes.byref(desc(b)), int(offs),
+                               int(accumulate), _stream(dst)))
+
+
+def so3part_cg_fwd(r, x, y, offs=0, accumulate=True):
+    _part("gelib_hip_so3part_cg_fwd", r, x, y, offs, accumulate)
+
+
+def so3part_cg_back0(xg, g, y, offs=0, accumulate=True):
+    _part("gelib_hip_so3part_cg_back0", xg, g, y, offs, accumulate)
+
+
+def so3part_cg_back1(yg, g, x, offs=0, accumulate=True):
+    _part("gelib_hip_so3part_cg_back1", yg, g, x, offs, accumulate)
+
+
+def so3part_diagcg_fwd(r, x, y, offs=0, accumulate=True):
+    _part("gelib_hip_so3part_diagcg_fwd", r, x, y, offs, accumulate)
+
+
+def so3part_diagcg_back0(xg, g, y, offs=0, accumulate=True):
+    _part("gelib_hip_so3part_diagcg_back0", xg, g, y, offs, accumulate)
+
+
+def so3part_diagcg_back1(yg, g, x, offs=0, accumulate=True):
+    _part("gelib_hip_so3part_diagcg_back1", yg, g, x, offs, accumulate)
+
+
+def so3vec_fwd(rparts, xparts, yparts, accumulate=True, diag=False):
+    fn = lib().gelib_hip_so3vec_diagcg_fwd if diag else lib().gelib_hip_so3vec_cg_fwd
+    check(fn(len(rparts), _arr(rparts), len(xparts), _arr(xparts), len(yparts), _arr(yparts), int(accumulate),
+             _stream(rparts[0])))
+
+
+def so3vec_bwd(xgparts, ygparts, gparts, xparts, yparts, accumulate=True, diag=False):
+    """Either gradient list may be None to skip it (back0-only / back1-only)."""
+    fn = lib().gelib_hip_so3vec_diagcg_bwd if diag else lib().gelib_hip_so3vec_cg_bwd
+    check(fn(_arr(xgparts), _arr(ygparts), len(gparts), _arr(gparts), len(xparts), _arr(xparts), len(yparts),
+             _arr(yparts), int(accumulate), _stream(gparts[0])))
+
+
+def set_option(name, value):
+    check(lib().gelib_hip_set_option(name.encode(), int(value)))
+
+
+def last_path():
+    return lib().gelib_hip_last_path()

@@ -1,0 +1,466 @@
+// C ABI of libgelib_hip.so: argument validation, broadcasting, triple enumeration and kernel selection.
+//
+// The validation mirrors what the reference checks on the way to its launchers -- the dispatcher's batch/grid
+// reconciliation (core/CGproduct.hpp:44-104, core/Gpart.hpp:168-185, 416-432) and the launcher's own tests
+// (cuda/SO3part_addCGproduct.cu:189-214) -- but reports a status code instead of printing and skipping.
+#include <algorithm>
+#include <cstdio>
+#include <cstring>
+#include <string>
+#include <vector>
+
+#include "cg_common.h"
+#include "cg_unrolled.h"
+
+using namespace gelib_hip;
+
+namespace gelib_hip {
+
+namespace {
+thread_local std::string t_last_error;
+thread_local int t_last_path = kPathNone;
+int g_force_generic = 0;
+int g_check_pointers = 1;
+}  // namespace
+
+int record_hip_error(hipError_t e, const char *what) {
+  t_last_error = std::string(what) + ": " + hipGetErrorString(e);
+  (void)hipGetLastError();  // clear the sticky error so that later calls are not blamed for it
+  return GELIB_HIP_ERR_RUNTIME;
+}
+
+namespace {
+
+struct View {  // one validated descriptor
+  const gelib_part_desc *d;
+  int l;
+  int n;
+};
+
+int check_desc(const gelib_part_desc *d, View &v) {
+  if (!d) return GELIB_HIP_ERR_NULL;
+  for (int k = 0; k < 5; k++)
+    if (d->dims[k] < 0) return GELIB_HIP_ERR_ARG;
+  if (d->dims[3] % 2 != 1) return GELIB_HIP_ERR_ODD_DIM;
+  if (d->dims[3] > 2 * (4 * kMaxL) + 1 || d->dims[4] > 0x7fffffffLL) return GELIB_HIP_ERR_PARTS;
+  v.d = d;
+  v.l = (int)(d->dims[3] - 1) / 2;
+  v.n = (int)d->dims[4];
+  const bool empty = d->dims[0] == 0 || d->dims[1] == 0 || d->dims[2] == 0 || d->dims[4] == 0;
+  if (!d->ptr && !empty) return GELIB_HIP_ERR_NULL;
+  return GELIB_HIP_OK;
+}
+
+// The farthest element of the view must lie inside the allocation that holds ptr, and that allocation must be
+// device (or managed) memory: a host pointer or an over-long view would otherwise fault the GPU.
+int check_pointer(const gelib_part_desc *d) {
+  if (!g_check_pointers || !d->ptr) return GELIB_HIP_OK;
+  long long span = 0;
+  for (int k = 0; k < 5; k++) {
+    if (d->dims[k] == 0) return GELIB_HIP_OK;
+    if (d->strides[k] < 0) return GELIB_HIP_ERR_ARG;
+    span += (d->dims[k] - 1) * d->strides[k];
+  }
+  hipPointerAttribute_t attr;
+  hipError_t e = hipPointerGetAttributes(&attr, d->ptr);
+  if (e != hipSuccess) {
+    (void)hipGetLastError();
+    return GELIB_HIP_ERR_DEVICE;
+  }
+  if (attr.type != hipMemoryTypeDevice && attr.type != hipMemoryTypeManaged) return GELIB_HIP_ERR_DEVICE;
+  int dev = 0;
+  if (hipGetDevice(&dev) == hipSuccess && attr.type == hipMemoryTypeDevice && attr.device != dev) return GELIB_HIP_ERR_DEVICE;
+  hipDeviceptr_t base = nullptr;
+  size_t size = 0;
+  e = hipMemGetAddressRange(&base, &size, (hipDeviceptr_t)d->ptr);
+  if (e != hipSuccess) {
+    (void)hipGetLastError();
+    return GELIB_HIP_OK;  // range unknown (e.g. a suballocator the runtime cannot see): type check above stands
+  }
+  const char *end = (const char *)d->ptr + (span + 1) * (long long)sizeof(float2);
+  if (end > (const char *)base + size) return GELIB_HIP_ERR_DEVICE;
+  return GELIB_HIP_OK;
+}
+
+PartDev to_dev(const gelib_part_desc *d, const long long E[3], long long own[3]) {
+  PartDev p;
+  p.ptr = (float2 *)d->ptr;
+  long long s[3];
+  for (int k = 0; k < 3; k++) {
+    own[k] = (d->dims[k] == E[k]) ? E[k] : 1;
+    s[k] = (d->dims[k] == E[k] && E[k] > 1) ? d->strides[k] : 0;
+  }
+  p.sb = s[0];
+  p.sg0 = s[1];
+  p.sg1 = s[2];
+  p.sm = d->strides[3];
+  p.sc = d->strides[4];
+  return p;
+}
+
+// dims equal or 1 along each leading dimension; dimension 0 is the batch, 1..2 the grid
+int reconcile(const gelib_part_desc *const *ds, int n, long long E[3]) {
+  for (int k = 0; k < 3; k++) {
+    long long e = 1;
+    bool zero = false;
+    for (int i = 0; i < n; i++) {
+      if (ds[i]->dims[k] == 0) zero = true;
+      e = std::max(e, (long long)ds[i]->dims[k]);
+    }
+    if (zero) e = 0;
+    for (int i = 0; i < n; i++)
+      if (ds[i]->dims[k] != e && ds[i]->dims[k] != 1) return k == 0 ? GELIB_HIP_ERR_BATCH : GELIB_HIP_ERR_GRID;
+    E[k] = e;
+  }
+  return GELIB_HIP_OK;
+}
+
+// roles: r = product/gradient, x = first operand (or its gradient), y = second operand (or its gradient)
+int make_part_op(const gelib_part_desc *r, const gelib_part_desc *x, const gelib_part_desc *y, int offs, bool diag,
+                 PartOp &op) {
+  View vr, vx, vy;
+  int rc;
+  if ((rc = check_desc(r, vr))) return rc;
+  if ((rc = check_desc(x, vx))) return rc;
+  if ((rc = check_desc(y, vy))) return rc;
+  if (vx.l > kMaxL || vy.l > kMaxL) return GELIB_HIP_ERR_PARTS;
+  if (vr.l < std::abs(vx.l - vy.l) || vr.l > vx.l + vy.l) return GELIB_HIP_ERR_TRIANGLE;
+  if (diag && vx.n != vy.n) return GELIB_HIP_ERR_DIAG_CHANNELS;
+  if (offs < 0) return GELIB_HIP_ERR_ARG;
+  const long long nout = diag ? vx.n : (long long)vx.n * vy.n;
+  if (nout > 0x7fffffffLL || offs + nout > vr.n) return GELIB_HIP_ERR_CHANNELS;
+  const gelib_part_desc *ds[3] = {r, x, y};
+  if ((rc = reconcile(ds, 3, op.E))) return rc;
+  op.r = to_dev(r, op.E, op.Dr);
+  op.x = to_dev(x, op.E, op.Dx);
+  op.y = to_dev(y, op.E, op.Dy);
+  op.l1 = vx.l;
+  op.l2 = vy.l;
+  op.l = vr.l;
+  op.n1 = vx.n;
+  op.n2 = vy.n;
+  op.nout = (int)nout;
+  op.offs = offs;
+  op.diag = diag;
+  return GELIB_HIP_OK;
+}
+
+enum Kind { kFwd, kBack0, kBack1 };
+
+int part_entry(Kind kind, bool diag, const gelib_part_desc *r, const gelib_part_desc *x, const gelib_part_desc *y,
+               int offs, int accumulate, void *stream) {
+  t_last_path = kPathNone;
+  PartOp op;
+  int rc = make_part_op(r, x, y, offs, diag, op);
+  if (rc) return rc;
+  if ((rc = check_pointer(r)) || (rc = check_pointer(x)) || (rc = check_pointer(y))) return rc;
+  if (op.E[0] * op.E[1] * op.E[2] == 0 || op.nout == 0) return GELIB_HIP_OK;
+  hipStream_t s = (hipStream_t)stream;
+  if (!g_force_generic) {
+    int used = 0;
+    rc = unrolled_part(kind == kFwd ? 0 : (kind == kBack0 ? 1 : 2), op, accumulate != 0, s, &used);
+    if (rc) return rc;
+    if (used) {
+      t_last_path = kPathUnrolled;
+      return GELIB_HIP_OK;
+    }
+  }
+  t_last_path = kPathGeneric;
+  switch (kind) {
+    case kFwd: return launch_generic_fwd(op, accumulate != 0, s);
+    case kBack0: return launch_generic_back0(op, accumulate != 0, s);
+    case kBack1: return launch_generic_back1(op, accumulate != 0, s);
+  }
+  return GELIB_HIP_ERR_ARG;
+}
+
+// ---- SO3vec level ---------------------------------------------------------------------------------------------
+
+int sort_parts(int n, const gelib_part_desc *parts, int max_parts, std::vector<View> &out) {
+  if (n < 0 || n > max_parts) return GELIB_HIP_ERR_PARTS;
+  if (n > 0 && !parts) return GELIB_HIP_ERR_NULL;
+  out.resize(n);
+  for (int i = 0; i < n; i++) {
+    int rc = check_desc(&parts[i], out[i]);
+    if (rc) return rc;
+  }
+  std::sort(out.begin(), out.end(), [](const View &a, const View &b) { return a.l < b.l; });
+  for (int i = 1; i < n; i++)
+    if (out[i].l == out[i - 1].l) return GELIB_HIP_ERR_PARTS;
+  return GELIB_HIP_OK;
+}
+
+int build_vec_plan(bool diag, const std::vector<View> &R, const std::vector<View> &X, const std::vector<View> &Y,
+                   VecPlan &plan) {
+  for (auto &v : X)
+    if (v.l > kMaxL) return GELIB_HIP_ERR_PARTS;
+  for (auto &v : Y)
+    if (v.l > kMaxL) return GELIB_HIP_ERR_PARTS;
+  std::vector<const gelib_part_desc *> all;
+  for (auto &v : R) all.push_back(v.d);
+  for (auto &v : X) all.push_back(v.d);
+  for (auto &v : Y) all.push_back(v.d);
+  int rc = reconcile(all.data(), (int)all.size(), plan.E);
+  if (rc) return rc;
+  plan.diag = diag;
+  plan.triples.clear();
+  std::vector<long long> offset(2 * (2 * kMaxL) + 2, 0);
+  for (int p = 0; p < (int)X.size(); p++)
+    for (int q = 0; q < (int)Y.size(); q++) {
+      const int l1 = X[p].l, l2 = Y[q].l;
+      for (int l = std::abs(l1 - l2); l <= l1 + l2; l++) {
+        int k = -1;
+        for (int t = 0; t < (int)R.size(); t++)
+          if (R[t].l == l) k = t;
+        if (k < 0) continue;  // absent product part: skipped, offsets of other parts unaffected
+        if (diag && X[p].n != Y[q].n) return GELIB_HIP_ERR_DIAG_CHANNELS;
+        const long long nout = diag ? X[p].n : (long long)X[p].n * Y[q].n;
+        if (offset[l] + nout > R[k].n) return GELIB_HIP_ERR_CHANNELS;
+        plan.triples.push_back({p, q, k, l1, l2, l, (int)offset[l], (int)nout});
+        offset[l] += nout;
+      }
+    }
+  return GELIB_HIP_OK;
+}
+
+PartOp triple_op(const VecPlan &plan, const VecTriple &t, const std::vector<View> &R, const std::vector<View> &X,
+                 const std::vector<View> &Y) {
+  PartOp op;
+  for (int d = 0; d < 3; d++) op.E[d] = plan.E[d];
+  op.r = to_dev(R[t.ri].d, op.E, op.Dr);
+  op.x = to_dev(X[t.xi].d, op.E, op.Dx);
+  op.y = to_dev(Y[t.yi].d, op.E, op.Dy);
+  op.l1 = t.l1;
+  op.l2 = t.l2;
+  op.l = t.l;
+  op.n1 = X[t.xi].n;
+  op.n2 = Y[t.yi].n;
+  op.nout = t.nout;
+  op.offs = t.offs;
+  op.diag = plan.diag;
+  return op;
+}
+
+int vec_fwd_entry(bool diag, int nr, const gelib_part_desc *r, int nx, const gelib_part_desc *x, int ny,
+                  const gelib_part_desc *y, int accumulate, void *stream) {
+  t_last_path = kPathNone;
+  std::vector<View> R, X, Y;
+  int rc;
+  if ((rc = sort_parts(nr, r, kMaxOutParts, R)) || (rc = sort_parts(nx, x, kMaxParts, X)) ||
+      (rc = sort_parts(ny, y, kMaxParts, Y)))
+    return rc;
+  if (R.empty() || X.empty() || Y.empty()) return GELIB_HIP_OK;
+  VecPlan plan;
+  if ((rc = build_vec_plan(diag, R, X, Y, plan))) return rc;
+  for (auto &v : R)
+    if ((rc = check_pointer(v.d))) return rc;
+  for (auto &v : X)
+    if ((rc = check_pointer(v.d))) return rc;
+  for (auto &v : Y)
+    if ((rc = check_pointer(v.d))) return rc;
+  if (plan.E[0] * plan.E[1] * plan.E[2] == 0 || plan.triples.empty()) return GELIB_HIP_OK;
+  hipStream_t s = (hipStream_t)stream;
+  if (!g_force_generic) {
+    std::vector<const gelib_part_desc *> rd, xd, yd;
+    for (auto &v : R) rd.push_back(v.d);
+    for (auto &v : X) xd.push_back(v.d);
+    for (auto &v : Y) yd.push_back(v.d);
+    int used = 0;
+    rc = unrolled_vec_fwd(plan, rd, xd, yd, accumulate != 0, s, &used);
+    if (rc) return rc;
+    if (used) {
+      t_last_path = kPathUnrolled;
+      return GELIB_HIP_OK;
+    }
+  }
+  t_last_path = kPathGeneric;
+  for (auto &t : plan.triples) {
+    PartOp op = triple_op(plan, t, R, X, Y);
+    if ((rc = launch_generic_fwd(op, accumulate != 0, s))) return rc;
+  }
+  return GELIB_HIP_OK;
+}
+
+int vec_bwd_entry(bool diag, const gelib_part_desc *xg, const gelib_part_desc *yg, int ng, const gelib_part_desc *g,
+                  int nx, const gelib_part_desc *x, int ny, const gelib_part_desc *y, int accumulate, void *stream) {
+  t_last_path = kPathNone;
+  if (!xg && !yg) return GELIB_HIP_OK;
+  std::vector<View> G, X, Y, XG, YG;
+  int rc;
+  if ((rc = sort_parts(ng, g, kMaxOutParts, G)) || (rc = sort_parts(nx, x, kMaxParts, X)) ||
+      (rc = sort_parts(ny, y, kMaxParts, Y)))
+    return rc;
+  if (xg && (rc = sort_parts(nx, xg, kMaxParts, XG))) return rc;
+  if (yg && (rc = sort_parts(ny, yg, kMaxParts, YG))) return rc;
+  // gradients are shaped like their operands (l and channel count; leading dimensions may broadcast)
+  for (int i = 0; xg && i < nx; i++)
+    if (XG[i].l != X[i].l || XG[i].n != X[i].n) return GELIB_HIP_ERR_PARTS;
+  for (int i = 0; yg && i < ny; i++)
+    if (YG[i].l != Y[i].l || YG[i].n != Y[i].n) return GELIB_HIP_ERR_PARTS;
+  if (G.empty() || X.empty() || Y.empty()) return GELIB_HIP_OK;
+  VecPlan plan;
+  if ((rc = build_vec_plan(diag, G, X, Y, plan))) return rc;
+  {  // the gradients take part in the batch/grid reconciliation too
+    std::vector<const gelib_part_desc *> all;
+    for (auto &v : G) all.push_back(v.d);
+    for (auto &v : X) all.push_back(v.d);
+    for (auto &v : Y) all.push_back(v.d);
+    for (auto &v : XG) all.push_back(v.d);
+    for (auto &v : YG) all.push_back(v.d);
+    if ((rc = reconcile(all.data(), (int)all.size(), plan.E))) return rc;
+  }
+  for (auto *L : {&G, &X, &Y, &XG, &YG})
+    for (auto &v : *L)
+      if ((rc = check_pointer(v.d))) return rc;
+  if (plan.E[0] * plan.E[1] * plan.E[2] == 0) return GELIB_HIP_OK;
+  hipStream_t s = (hipStream_t)stream;
+  if (!g_force_generic && !plan.triples.empty()) {
+    std::vector<const gelib_part_desc *> gd, xd, yd, xgd, ygd;
+    for (auto &v : G) gd.push_back(v.d);
+    for (auto &v : X) xd.push_back(v.d);
+    for (auto &v : Y) yd.push_back(v.d);
+    for (auto &v : XG) xgd.push_back(v.d);
+    for (auto &v : YG) ygd.push_back(v.d);
+    int used = 0;
+    rc = unrolled_vec_bwd(plan, gd, xd, yd, xgd, ygd, accumulate != 0, s, &used);
+    if (rc) return rc;
+    if (used) {
+      t_last_path = kPathUnrolled;
+      return GELIB_HIP_OK;
+    }
+  }
+  t_last_path = kPathGeneric;
+  // shape-agnostic route: zero the destinations when overwriting, then one accumulation per triple,
+  // all back0 first and then all back1 like the reference (python/src/gelib/SO3vec.py:267-268)
+  if (!accumulate) {
+    for (auto *L : {&XG, &YG})
+      for (auto &v : *L) {
+        long long own[3];
+        PartDev pd = to_dev(v.d, plan.E, own);
+        if ((rc = launch_zero_fill(pd, own, 2 * v.l + 1, v.n, s))) return rc;
+      }
+  }
+  if (xg)
+    for (auto &t : plan.triples) {
+      PartOp op = triple_op(plan, t, G, XG, Y);
+      if ((rc = launch_generic_back0(op, true, s))) return rc;
+    }
+  if (yg)
+    for (auto &t : plan.triples) {
+      PartOp op = triple_op(plan, t, G, X, YG);
+      if ((rc = launch_generic_back1(op, true, s))) return rc;
+    }
+  return GELIB_HIP_OK;
+}
+
+}  // namespace
+}  // namespace gelib_hip
+
+extern "C" {
+
+const char *gelib_hip_strerror(int status) {
+  switch (status) {
+    case GELIB_HIP_OK: return "ok";
+    case GELIB_HIP_ERR_NULL: return "null descriptor or data pointer";
+    case GELIB_HIP_ERR_ODD_DIM: return "dimension -2 of an SO3part must be odd (2l+1)";
+    case GELIB_HIP_ERR_TRIANGLE: return "|l1-l_2| <= l <= l1+l2 not satisfied";
+    case GELIB_HIP_ERR_DIAG_CHANNELS: return "DiagCGproduct needs equal channel counts (N1==N2)";
+    case GELIB_HIP_ERR_CHANNELS: return "fragment dimension of r not large enough";
+    case GELIB_HIP_ERR_BATCH: return "batch dimensions cannot be reconciled";
+    case GELIB_HIP_ERR_GRID: return "grid dimensions cannot be reconciled";
+    case GELIB_HIP_ERR_DEVICE: return "SO3part must be on GPU (pointer is not device memory of the current device, or the view overruns its allocation)";
+    case GELIB_HIP_ERR_PARTS: return "too many parts, a repeated l, l above the supported maximum, or gradient parts that do not match their operand";
+    case GELIB_HIP_ERR_RUNTIME: return "HIP runtime error";
+    case GELIB_HIP_ERR_BROADCAST_DEST: return "cannot overwrite a broadcast destination";
+    case GELIB_HIP_ERR_ARG: return "malformed argument";
+  }
+  return "unknown status";
+}
+
+const char *gelib_hip_last_runtime_error(void) { return t_last_error.c_str(); }
+
+const char *gelib_hip_version(void) { return "gelib_hip 0.1 (gfx950)"; }
+
+int gelib_hip_cg_matrix(int l1, int l2, int l, float *out) {
+  if (!out) return GELIB_HIP_ERR_NULL;
+  if (l1 < 0 || l2 < 0 || l < std::abs(l1 - l2) || l > l1 + l2) return GELIB_HIP_ERR_TRIANGLE;
+  cg_matrix_host(l1, l2, l, out);
+  return GELIB_HIP_OK;
+}
+
+int gelib_hip_so3type_product(int diag, int nx, const int *lx, const int *cx, int ny, const int *ly, const int *cy,
+                              int maxl, int64_t *n_out, int len) {
+  if ((nx > 0 && (!lx || !cx)) || (ny > 0 && (!ly || !cy)) || !n_out) return -GELIB_HIP_ERR_NULL;
+  for (int i = 0; i < len; i++) n_out[i] = 0;
+  int count = 0;
+  for (int p = 0; p < nx; p++)
+    for (int q = 0; q < ny; q++)
+      for (int l = std::abs(lx[p] - ly[q]); l <= lx[p] + ly[q]; l++) {
+        if (maxl >= 0 && l > maxl) continue;
+        if (l >= len) return -GELIB_HIP_ERR_ARG;
+        if (n_out[l] == 0) count++;
+        n_out[l] += diag ? (int64_t)cx[p] : (int64_t)cx[p] * cy[q];
+      }
+  return count;
+}
+
+int gelib_hip_so3part_cg_fwd(const gelib_part_desc *r, const gelib_part_desc *x, const gelib_part_desc *y, int offs,
+                             int accumulate, void *stream) {
+  return part_entry(kFwd, false, r, x, y, offs, accumulate, stream);
+}
+int gelib_hip_so3part_cg_back0(const gelib_part_desc *xg, const gelib_part_desc *g, const gelib_part_desc *y,
+                               int offs, int accumulate, void *stream) {
+  return part_entry(kBack0, false, g, xg, y, offs, accumulate, stream);
+}
+int gelib_hip_so3part_cg_back1(const gelib_part_desc *yg, const gelib_part_desc *g, const gelib_part_desc *x,
+                               int offs, int accumulate, void *stream) {
+  return part_entry(kBack1, false, g, x, yg, offs, accumulate, stream);
+}
+int gelib_hip_so3part_diagcg_fwd(const gelib_part_desc *r, const gelib_part_desc *x, const gelib_part_desc *y,
+                                 int offs, int accumulate, void *stream) {
+  return part_entry(kFwd, true, r, x, y, offs, accumulate, stream);
+}
+int gelib_hip_so3part_diagcg_back0(const gelib_part_desc *xg, const gelib_part_desc *g, const gelib_part_desc *y,
+                                   int offs, int accumulate, void *stream) {
+  return part_entry(kBack0, true, g, xg, y, offs, accumulate, stream);
+}
+int gelib_hip_so3part_diagcg_back1(const gelib_part_desc *yg, const gelib_part_desc *g, const gelib_part_desc *x,
+                                   int offs, int accumulate, void *stream) {
+  return part_entry(kBack1, true, g, x, yg, offs, accumulate, stream);
+}
+
+int gelib_hip_so3vec_cg_fwd(int nr, const gelib_part_desc *r, int nx, const gelib_part_desc *x, int ny,
+                            const gelib_part_desc *y, int accumulate, void *stream) {
+  return vec_fwd_entry(false, nr, r, nx, x, ny, y, accumulate, stream);
+}
+int gelib_hip_so3vec_cg_bwd(const gelib_part_desc *xg, const gelib_part_desc *yg, int ng, const gelib_part_desc *g,
+                            int nx, const gelib_part_desc *x, int ny, const gelib_part_desc *y, int accumulate,
+                            void *stream) {
+  return vec_bwd_entry(false, xg, yg, ng, g, nx, x, ny, y, accumulate, stream);
+}
+int gelib_hip_so3vec_diagcg_fwd(int nr, const gelib_part_desc *r, int nx, const gelib_part_desc *x, int ny,
+                                const gelib_part_desc *y, int accumulate, void *stream) {
+  return vec_fwd_entry(true, nr, r, nx, x, ny, y, accumulate, stream);
+}
+int gelib_hip_so3vec_diagcg_bwd(const gelib_part_desc *xg, const gelib_part_desc *yg, int ng,
+                                const gelib_part_desc *g, int nx, const gelib_part_desc *x, int ny,
+                                const gelib_part_desc *y, int accumulate, void *stream) {
+  return vec_bwd_entry(true, xg, yg, ng, g, nx, x, ny, y, accumulate, stream);
+}
+
+int gelib_hip_set_option(const char *name, int value) {
+  if (!name) return GELIB_HIP_ERR_NULL;
+  if (!std::strcmp(name, "force_generic")) {
+    g_force_generic = value;
+    return GELIB_HIP_OK;
+  }
+  if (!std::strcmp(name, "check_pointers")) {
+    g_check_pointers = value;
+    return GELIB_HIP_OK;
+  }
+  return unrolled_set_option(name, value);
+}
+
+int gelib_hip_last_path(void) { return t_last_path; }
+
+}  // extern "C"

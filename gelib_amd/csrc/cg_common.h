@@ -1,0 +1,54 @@
+// Shared host/device declarations of libgelib_hip.so (internal; the public interface is include/gelib_hip.h).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "gelib_hip.h"
+
+namespace gelib_hip {
+
+constexpr int kMaxL = GELIB_HIP_MAX_L;
+constexpr int kMaxParts = GELIB_HIP_MAX_PARTS;
+constexpr int kMaxOutParts = GELIB_HIP_MAX_OUT_PARTS;
+constexpr int kWave = 64;
+
+// A part as the shape-agnostic kernels see it: 5-D strides in complex elements (0 = broadcast).
+struct PartDev {
+  float2 *ptr;
+  long long sb, sg0, sg1, sm, sc;
+};
+
+// One part-level operation after validation and broadcasting (host side).
+struct PartOp {
+  PartDev r, x, y;           // r = product or its gradient
+  long long E[3];            // common extents (batch, grid0, grid1)
+  long long Dr[3], Dx[3], Dy[3];  // own extents of each tensor (E[d] or 1)
+  int l1, l2, l, n1, n2, nout;
+  int offs;
+  bool diag;
+};
+
+enum PathId { kPathNone = 0, kPathGeneric = 1, kPathUnrolled = 2 };
+
+// ---- coefficient bank (cg_bank.cpp) ----
+double cg_coeff(int l1, int l2, int l, int m1, int m2);
+void cg_matrix_host(int l1, int l2, int l, float *out);
+// Device copy of one (2l1+1)x(2l2+1) table on the current device; cached for the life of the process.
+int cg_matrix_device(int l1, int l2, int l, const float **dptr);
+
+// ---- error plumbing ----
+int record_hip_error(hipError_t e, const char *what);
+#define GELIB_HIP_TRY(expr)                                   \
+  do {                                                        \
+    hipError_t _e = (expr);                                   \
+    if (_e != hipSuccess) return record_hip_error(_e, #expr); \
+  } while (0)
+
+// ---- shape-agnostic kernels (cg_generic.hip) ----
+int launch_generic_fwd(const PartOp &op, bool accumulate, hipStream_t s);
+int launch_generic_back0(const PartOp &op, bool accumulate, hipStream_t s);  // destination = op.x
+int launch_generic_back1(const PartOp &op, bool accumulate, hipStream_t s);  // destination = op.y
+int launch_zero_fill(const PartDev &d, const long long D[3], int M, int n, hipStream_t s);
+
+}  // namespace gelib_hip

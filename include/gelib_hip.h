@@ -1,0 +1,138 @@
+/*
+ * gelib_hip.h -- C ABI of the MI355X (gfx950) Clebsch-Gordan product library, libgelib_hip.so.
+ *
+ * This is the drop-in boundary for GElib's device seam: each entry point takes the place of one of
+ * the reference's GPU launchers (or of the loop of launches the reference makes at SO3vec level).
+ * Plain pointers and sizes only; no C++ or torch types.  All tensors are complex float32, stored
+ * interleaved (re,im), viewed as 5-D (batch, grid0, grid1, 2l+1, channels) exactly like the views the
+ * reference hands to its launchers (cuda/GPUtensor.hpp:31-38), with strides counted in complex
+ * elements and stride 0 meaning "broadcast along this dimension" (core/Gpart.hpp:168-185).
+ *
+ * Every call is asynchronous on the HIP stream passed in (NULL = the default stream), allocates
+ * nothing per call (the coefficient bank and the per-type triple tables are cached on first use),
+ * and returns 0 or one of the gelib_hip_status codes without printing or throwing.
+ */
+#ifndef GELIB_HIP_H
+#define GELIB_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct gelib_part_desc {
+  void *ptr;          /* device pointer to the first complex element                          */
+  int64_t dims[5];    /* (batch, grid0, grid1, 2l+1, channels); a 3-D part has grid0=grid1=1  */
+  int64_t strides[5]; /* in complex elements; 0 broadcasts the dimension                      */
+} gelib_part_desc;
+
+enum gelib_hip_status {
+  GELIB_HIP_OK = 0,
+  GELIB_HIP_ERR_NULL = 1,          /* null descriptor or data pointer                                              */
+  GELIB_HIP_ERR_ODD_DIM = 2,       /* dims[3] is not 2l+1 (SO3/SO3part.hpp:166-170)                                  */
+  GELIB_HIP_ERR_TRIANGLE = 3,      /* |l1-l2| <= l <= l1+l2 not satisfied (cuda/SO3part_addCGproduct.cu:210)         */
+  GELIB_HIP_ERR_DIAG_CHANNELS = 4, /* DiagCGproduct with n1 != n2 (SO3/SO3part.hpp:282)                              */
+  GELIB_HIP_ERR_CHANNELS = 5,      /* offs + n_out exceeds the product's channels (cuda/SO3part_addCGproduct.cu:214) */
+  GELIB_HIP_ERR_BATCH = 6,         /* batch dimensions cannot be reconciled (core/CGproduct.hpp:49)                  */
+  GELIB_HIP_ERR_GRID = 7,          /* grid dimensions cannot be reconciled (core/CGproduct.hpp:50)                   */
+  GELIB_HIP_ERR_DEVICE = 8,        /* a pointer is not device memory of the current GPU                              */
+  GELIB_HIP_ERR_PARTS = 9,         /* too many parts, a repeated l, or l above the supported maximum                 */
+  GELIB_HIP_ERR_RUNTIME = 10,      /* a HIP call failed; see gelib_hip_last_runtime_error()                          */
+  GELIB_HIP_ERR_BROADCAST_DEST = 11, /* overwrite requested into a destination that is broadcast (stride 0)          */
+  GELIB_HIP_ERR_ARG = 12           /* negative offset or other malformed argument                                    */
+};
+
+#define GELIB_HIP_MAX_L 32          /* largest l of an operand part                     */
+#define GELIB_HIP_MAX_PARTS 16      /* parts per operand SO3vec                         */
+#define GELIB_HIP_MAX_OUT_PARTS 40  /* parts of the product / gradient SO3vec           */
+
+/* Message for a status code (static storage). */
+const char *gelib_hip_strerror(int status);
+/* Text of the last HIP runtime error seen by this thread ("" if none). */
+const char *gelib_hip_last_runtime_error(void);
+/* Library version string. */
+const char *gelib_hip_version(void);
+
+/*
+ * Host copy of the coefficient matrix <l1 m1; l2 m2 | l m1+m2>, row-major (2l1+1) x (2l2+1) float,
+ * zero where |m1+m2| > l.  Same values the kernels use.  Replaces SO3CGbank::get<float>(l1,l2,l,0)
+ * (SO3/SO3CGbank.hpp:33-42, 58-95).
+ */
+int gelib_hip_cg_matrix(int l1, int l2, int l, float *out);
+
+/*
+ * Type arithmetic of the product: n_out[l] for l = 0..len-1 (core/Gtype.hpp:115-138).
+ * maxl < 0 keeps every l.  Returns the number of parts, or a negative status.
+ */
+int gelib_hip_so3type_product(int diag, int nx, const int *lx, const int *cx, int ny, const int *ly, const int *cy,
+                              int maxl, int64_t *n_out, int len);
+
+/* ---- part level ---------------------------------------------------------------------------------------------
+ * accumulate != 0 : reference semantics, add into the destination.
+ * accumulate == 0 : overwrite the destination block (channels offs .. offs+n_out-1 of r, or all of xg / yg)
+ *                   without reading it, for callers that would otherwise zero-fill first.
+ */
+
+/* r[m1+m2, offs+i*n2+j] += C[m1,m2] x[m1,i] y[m2,j].
+ * Replaces SO3part_addCGproduct_cu(r,x,y,offs,stream) (cuda/SO3part_addCGproduct.cu:187). */
+int gelib_hip_so3part_cg_fwd(const gelib_part_desc *r, const gelib_part_desc *x, const gelib_part_desc *y, int offs,
+                             int accumulate, void *stream);
+/* xg[m1,i] += sum_{j,m2} C[m1,m2] g[m1+m2, offs+i*n2+j] conj(y[m2,j]).
+ * Replaces SO3part_addCGproduct_back0_cu(xg,g,y,offs,stream) (cuda/SO3part_addCGproduct_back0.cu:224). */
+int gelib_hip_so3part_cg_back0(const gelib_part_desc *xg, const gelib_part_desc *g, const gelib_part_desc *y,
+                               int offs, int accumulate, void *stream);
+/* yg[m2,j] += sum_{i,m1} C[m1,m2] g[m1+m2, offs+i*n2+j] conj(x[m1,i]).
+ * Replaces SO3part_addCGproduct_back1_cu(yg,g,x,offs,stream) (cuda/SO3part_addCGproduct_back1.cu:123). */
+int gelib_hip_so3part_cg_back1(const gelib_part_desc *yg, const gelib_part_desc *g, const gelib_part_desc *x,
+                               int offs, int accumulate, void *stream);
+
+/* r[m1+m2, offs+i] += C[m1,m2] x[m1,i] y[m2,i].  Fills the seam the reference leaves empty
+ * (SO3part::add_DiagCGproduct_dev, SO3/SO3part.hpp:324-326); semantics from SO3/SO3part.hpp:276-290. */
+int gelib_hip_so3part_diagcg_fwd(const gelib_part_desc *r, const gelib_part_desc *x, const gelib_part_desc *y,
+                                 int offs, int accumulate, void *stream);
+/* SO3/SO3part.hpp:292-306 (seam SO3/SO3part.hpp:328-330). */
+int gelib_hip_so3part_diagcg_back0(const gelib_part_desc *xg, const gelib_part_desc *g, const gelib_part_desc *y,
+                                   int offs, int accumulate, void *stream);
+/* SO3/SO3part.hpp:308-322 (seam SO3/SO3part.hpp:332-334). */
+int gelib_hip_so3part_diagcg_back1(const gelib_part_desc *yg, const gelib_part_desc *g, const gelib_part_desc *x,
+                                   int offs, int accumulate, void *stream);
+
+/* ---- SO3vec level: every (l1,l2,l) triple in one call ------------------------------------------------------------
+ * Part lists may come in any order; l is read from dims[3].  Triples are enumerated l1 ascending, l2 ascending,
+ * l ascending, each writing its block at the running per-l channel offset; a product part that is absent is
+ * skipped without moving any other offset (core/Gvec.hpp:311-321).
+ */
+
+/* Replaces the loop of Gpart_add_CGproduct calls in Gvec::add_CGproduct (core/Gvec.hpp:311-321). */
+int gelib_hip_so3vec_cg_fwd(int nr, const gelib_part_desc *r, int nx, const gelib_part_desc *x, int ny,
+                            const gelib_part_desc *y, int accumulate, void *stream);
+/*
+ * Both gradients in one pass over g.  xg (nx parts, shaped like x) and yg (ny parts, shaped like y); either
+ * list may be NULL to compute only the other, which then replaces Gvec::add_CGproduct_back0
+ * (core/Gvec.hpp:323-333) resp. add_CGproduct_back1 (core/Gvec.hpp:335-345).
+ */
+int gelib_hip_so3vec_cg_bwd(const gelib_part_desc *xg, const gelib_part_desc *yg, int ng, const gelib_part_desc *g,
+                            int nx, const gelib_part_desc *x, int ny, const gelib_part_desc *y, int accumulate,
+                            void *stream);
+/* Gvec::add_DiagCGproduct (core/Gvec.hpp:358-367). */
+int gelib_hip_so3vec_diagcg_fwd(int nr, const gelib_part_desc *r, int nx, const gelib_part_desc *x, int ny,
+                                const gelib_part_desc *y, int accumulate, void *stream);
+/* Gvec::add_DiagCGproduct_back0 / _back1 (core/Gvec.hpp:369-389). */
+int gelib_hip_so3vec_diagcg_bwd(const gelib_part_desc *xg, const gelib_part_desc *yg, int ng,
+                                const gelib_part_desc *g, int nx, const gelib_part_desc *x, int ny,
+                                const gelib_part_desc *y, int accumulate, void *stream);
+
+/*
+ * Tuning / introspection (no counterpart in the reference).
+ * gelib_hip_set_option("force_generic", 1) routes every call through the shape-agnostic kernels;
+ * gelib_hip_last_path() tells which kernel family the last call of this thread used
+ * (0 = none, 1 = generic, 2 = unrolled small-l kernels).
+ */
+int gelib_hip_set_option(const char *name, int value);
+int gelib_hip_last_path(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,113 @@
+"""GPU parity of the SO3vec-level entry points (all triples in one call) against the CPU oracle."""
+import numpy as np
+import pytest
+
+from oracle import cg_oracle as ora
+from tests import gpu_util as U
+
+pytestmark = pytest.mark.gpu
+
+torch = pytest.importorskip("torch")
+
+
+@pytest.fixture(scope="module")
+def cabi():
+    assert torch.cuda.is_available(), "GPU tests need a GPU"
+    from gelib_amd import cabi as c
+    c.lib()
+    return c
+
+
+CASES = [
+    # (B, tau_x, tau_y, maxl)
+    (33, {l: 16 for l in range(5)}, {l: 16 for l in range(5)}, 4),      # headline type, small batch
+    (9, {l: 16 for l in range(5)}, {l: 16 for l in range(5)}, -1),
+    (4, {0: 2, 1: 3, 2: 2}, {1: 2, 2: 1}, -1),
+    (4, {0: 1, 2: 4}, {0: 4, 1: 4, 3: 2}, 3),
+    (3, {l: 4 for l in range(3)}, {l: 4 for l in range(3)}, 2),
+    (2, {10: 8}, {10: 8}, -1),                                           # configuration 5 type
+    (5, {l: 8 for l in range(7)}, {l: 8 for l in range(7)}, 6),
+]
+
+
+def run_vec(cabi, B, tx, ty, maxl, diag, seed, force_generic):
+    cabi.set_option("force_generic", int(force_generic))
+    if diag:
+        ty = {l: tx[min(tx)] for l in ty}
+        tx = {l: tx[min(tx)] for l in tx}
+    xs = [U.seeded(seed + l, B, 2 * l + 1, n) for l, n in sorted(tx.items())]
+    ys = [U.seeded(seed + 50 + l, B, 2 * l + 1, n) for l, n in sorted(ty.items())]
+    r32 = ora.vec_fwd(xs, ys, maxl, diag)
+    r64 = ora.vec_fwd([a.astype(np.complex128) for a in xs], [a.astype(np.complex128) for a in ys], maxl, diag)
+    gs = [U.seeded(seed + 100 + i, *p.shape) for i, p in enumerate(r32)]
+    xg32, yg32 = ora.vec_bwd(gs, xs, ys, diag)
+    xg64, yg64 = ora.vec_bwd([a.astype(np.complex128) for a in gs], [a.astype(np.complex128) for a in xs],
+                             [a.astype(np.complex128) for a in ys], diag)
+    dxs, dys, dgs = [U.dev(a) for a in xs], [U.dev(a) for a in ys], [U.dev(a) for a in gs]
+    # overwrite mode into garbage: every channel of every part must be written exactly once
+    drs = [torch.full(p.shape, 7.0 + 1j, dtype=torch.complex64, device="cuda") for p in r32]
+    cabi.so3vec_fwd(drs, dxs, dys, accumulate=False, diag=diag)
+    path_fwd = cabi.last_path()
+    dxg = [torch.full(a.shape, 3.0 - 2j, dtype=torch.complex64, device="cuda") for a in xs]
+    dyg = [torch.full(a.shape, 3.0 - 2j, dtype=torch.complex64, device="cuda") for a in ys]
+    cabi.so3vec_bwd(dxg, dyg, dgs, dxs, dys, accumulate=False, diag=diag)
+    path_bwd = cabi.last_path()
+    torch.cuda.synchronize()
+    tag = "B%d %s x %s maxl %d diag %d" % (B, tx, ty, maxl, diag)
+    for a, b, c in zip(drs, r32, r64):
+        U.assert_parity(U.host(a), b, c, "fwd " + tag)
+    for a, b, c in zip(dxg, xg32, xg64):
+        U.assert_parity(U.host(a), b, c, "xg " + tag, slack=1.5)
+    for a, b, c in zip(dyg, yg32, yg64):
+        U.assert_parity(U.host(a), b, c, "yg " + tag, slack=1.5)
+    # accumulate mode adds on top; back0-only and back1-only calls
+    drs2 = [a.clone() for a in drs]
+    cabi.so3vec_fwd(drs2, dxs, dys, accumulate=True, diag=diag)
+    dxg2 = [torch.zeros_like(a) for a in dxs]
+    dyg2 = [torch.zeros_like(a) for a in dys]
+    cabi.so3vec_bwd(dxg2, None, dgs, dxs, dys, accumulate=True, diag=diag)
+    cabi.so3vec_bwd(None, dyg2, dgs, dxs, dys, accumulate=True, diag=diag)
+    torch.cuda.synchronize()
+    for a, b in zip(drs2, drs):
+        assert U.gate_excess(U.host(a), 2 * U.host(b)) <= 1.0
+    for a, b in zip(dxg2 + dyg2, dxg + dyg):
+        assert U.gate_excess(U.host(a), U.host(b), rtol=2e-5, atol=2e-5) <= 1.0
+    return path_fwd, path_bwd
+
+
+@pytest.mark.parametrize("case", CASES)
+@pytest.mark.parametrize("diag", [False, True])
+def test_vec_generic(cabi, case, diag):
+    assert run_vec(cabi, *case, diag, seed=300, force_generic=True) == (1, 1)
+
+
+@pytest.mark.parametrize("case", CASES)
+@pytest.mark.parametrize("diag", [False, True])
+def test_vec_default_path(cabi, case, diag):
+    run_vec(cabi, *case, diag, seed=400, force_generic=False)
+
+
+def test_absent_output_part_keeps_offsets(cabi):
+    # a product part that is missing is skipped; the blocks of the other parts stay where they are
+    cabi.set_option("force_generic", 0)
+    tx = {0: 2, 1: 2}
+    xs = [U.seeded(1 + l, 3, 2 * l + 1, n) for l, n in tx.items()]
+    ys = [U.seeded(9 + l, 3, 2 * l + 1, n) for l, n in tx.items()]
+    full = ora.vec_fwd(xs, ys)                      # parts l = 0, 1, 2
+    drs = [torch.zeros(p.shape, dtype=torch.complex64, device="cuda") for p in (full[0], full[2])]
+    cabi.so3vec_fwd(drs, [U.dev(a) for a in xs], [U.dev(a) for a in ys], accumulate=True)
+    torch.cuda.synchronize()
+    assert U.gate_excess(U.host(drs[0]), full[0]) <= 1.0
+    assert U.gate_excess(U.host(drs[1]), full[2]) <= 1.0
+
+
+def test_parts_in_any_order(cabi):
+    cabi.set_option("force_generic", 0)
+    xs = [U.seeded(1 + l, 2, 2 * l + 1, 2) for l in range(3)]
+    ys = [U.seeded(7 + l, 2, 2 * l + 1, 2) for l in range(3)]
+    want = ora.vec_fwd(xs, ys, 2)
+    drs = [torch.zeros(p.shape, dtype=torch.complex64, device="cuda") for p in want]
+    cabi.so3vec_fwd(drs[::-1], [U.dev(a) for a in xs[::-1]], [U.dev(a) for a in ys], accumulate=False)
+    torch.cuda.synchronize()
+    for a, b in zip(drs, want):
+        assert U.gate_excess(U.host(a), b) <= 1.0

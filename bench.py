@@ -1,0 +1,184 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused SO3vec CGproduct path on one MI355X.
+
+One "step" = one forward pass (all (l1,l2,l) triples, one launch) plus one backward pass (both gradients, one
+launch) over a batch of synthetic complex64 N(0,1) inputs that already sit in HBM.  The default workload is the
+headline configuration: L=4, 16 channels per part, batch 32768, product capped at l<=4 (65 triples).
+
+Prints ONE JSON line: samples/s (whole job), the roofline of the dominant kernel from HIP-event timings taken
+inside this run, and a CPU baseline (the oracle's loop-order-faithful float32 restatement of the reference's CPU
+path, timed here on one host core over a batch slice; the GPU result for that slice is checked against it).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK = 8.0e12  # B/s, MI355X HBM3E
+
+WORKLOADS = {
+    # name: (kind, B, tau_x, tau_y, maxl, diag)
+    "so3vec_cg_L4_tau16_B32768_maxl4": ("vec", 32768, {l: 16 for l in range(5)}, {l: 16 for l in range(5)}, 4, False),
+    "so3vec_cg_L4_tau16_B32768_uncapped": ("vec", 32768, {l: 16 for l in range(5)}, {l: 16 for l in range(5)}, -1, False),
+    "so3part_cg_2x3to4_n32_B65536": ("vec", 65536, {2: 32}, {3: 32}, 4, False),
+    "so3vec_diagcg_L6_n64_B131072": ("vec", 131072, {l: 64 for l in range(7)}, {l: 64 for l in range(7)}, 6, True),
+    "so3part_cg_10x10_all_l_n8_B16384": ("vec", 16384, {10: 8}, {10: 8}, -1, False),
+}
+ALIASES = {"cfg4": "so3vec_cg_L4_tau16_B32768_maxl4", "cfg4u": "so3vec_cg_L4_tau16_B32768_uncapped",
+           "cfg2": "so3part_cg_2x3to4_n32_B65536", "cfg3": "so3vec_diagcg_L6_n64_B131072",
+           "cfg5": "so3part_cg_10x10_all_l_n8_B16384"}
+
+
+def out_type(tx, ty, maxl, diag):
+    tau = {}
+    for l1, n1 in sorted(tx.items()):
+        for l2, n2 in sorted(ty.items()):
+            for l in range(abs(l1 - l2), l1 + l2 + 1):
+                if maxl < 0 or l <= maxl:
+                    tau[l] = tau.get(l, 0) + (n1 if diag else n1 * n2)
+    return dict(sorted(tau.items()))
+
+
+def algorithmic_bytes(B, tx, ty, tr):
+    """Every operand read once and every result written once, complex64 = 8 B."""
+    X = 8 * B * sum((2 * l + 1) * n for l, n in tx.items())
+    Y = 8 * B * sum((2 * l + 1) * n for l, n in ty.items())
+    R = 8 * B * sum((2 * l + 1) * n for l, n in tr.items())
+    return X + Y + R, R + 2 * X + 2 * Y
+
+
+def seeded_parts(torch, seed, B, tau, device, scale=1.0):
+    parts = []
+    for l, n in sorted(tau.items()):
+        g = torch.Generator(device=device).manual_seed(seed + l)
+        t = torch.randn(B, 2 * l + 1, n, 2, generator=g, device=device, dtype=torch.float32)
+        parts.append(torch.view_as_complex(t) * scale if scale != 1.0 else torch.view_as_complex(t))
+    return parts
+
+
+def cpu_baseline(torch, xs, ys, gs, rs, xgs, ygs, maxl, diag, nsample):
+    """Time the oracle on the first `nsample` samples with one thread and check the GPU slice against it."""
+    import numpy as np
+    from oracle import cg_oracle as ora
+    hx = [t[:nsample].cpu().numpy() for t in xs]
+    hy = [t[:nsample].cpu().numpy() for t in ys]
+    hg = [t[:nsample].cpu().numpy() for t in gs]
+    ora.lib()
+    t0 = time.perf_counter()
+    r = ora.vec_fwd(hx, hy, maxl, diag, nthreads=1)
+    xg, yg = ora.vec_bwd(hg, hx, hy, diag, nthreads=1)
+    dt = time.perf_counter() - t0
+
+    def excess(got, ref):
+        a = got[:nsample].cpu().numpy().view(np.float32).astype(np.float64)
+        b = ref.view(np.float32).astype(np.float64)
+        return float(np.max(np.abs(a - b) / (1e-6 + 1e-5 * np.abs(b))))
+
+    parity = {"fwd_gate_excess": max(excess(a, b) for a, b in zip(rs, r)),
+              "bwd_gate_excess": max(excess(a, b) for a, b in zip(xgs + ygs, xg + yg)),
+              "gate": "|gpu-cpu| <= 1e-6 + 1e-5*|cpu| per real component; excess <= 1 is inside"}
+    return nsample / dt, dt, parity
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="cfg4")
+    ap.add_argument("--batch", type=int, default=0, help="override the batch size (debugging only)")
+    ap.add_argument("--cpu-samples", type=int, default=768)
+    ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--generic", action="store_true", help="force the shape-agnostic kernels")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build runs on ONE GPU; the path shards along the batch with no exchange step, "
+              "so --gpus N>1 has nothing to measure here", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from gelib_amd import cabi
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    cabi.lib()
+    cabi.set_option("force_generic", int(args.generic))
+    dev = torch.device("cuda:0")
+    name = ALIASES.get(args.workload, args.workload)
+    kind, B, tx, ty, maxl, diag = WORKLOADS[name]
+    if args.batch:
+        B = args.batch
+    tr = out_type(tx, ty, maxl, diag)
+    fwd_bytes, bwd_bytes = algorithmic_bytes(B, tx, ty, tr)
+
+    scale_y = 1e-3 if "10x10" in name else 1.0
+    xs = seeded_parts(torch, 1004, B, tx, dev)
+    ys = seeded_parts(torch, 2004, B, ty, dev, scale_y)
+    gs = seeded_parts(torch, 3004, B, tr, dev)
+    rs = [torch.empty(B, 2 * l + 1, n, dtype=torch.complex64, device=dev) for l, n in tr.items()]
+    xgs = [torch.empty_like(t) for t in xs]
+    ygs = [torch.empty_like(t) for t in ys]
+
+    def fwd():
+        cabi.so3vec_fwd(rs, xs, ys, accumulate=False, diag=diag)
+
+    def bwd():
+        cabi.so3vec_bwd(xgs, ygs, gs, xs, ys, accumulate=False, diag=diag)
+
+    for _ in range(args.warmup):
+        fwd()
+        bwd()
+    torch.cuda.synchronize()
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
+    t0 = time.perf_counter()
+    for k in range(args.steps):
+        ev[k][0].record()
+        fwd()
+        ev[k][1].record()
+        bwd()
+        ev[k][2].record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    fwd_ms = sum(e[0].elapsed_time(e[1]) for e in ev) / args.steps
+    bwd_ms = sum(e[1].elapsed_time(e[2]) for e in ev) / args.steps
+    ms_per_step = wall * 1e3 / args.steps
+    path = cabi.last_path()
+
+    if bwd_ms >= fwd_ms:
+        dom, dom_ms, dom_bytes = "so3vec_bwd", bwd_ms, bwd_bytes
+    else:
+        dom, dom_ms, dom_bytes = "so3vec_fwd", fwd_ms, fwd_bytes
+    achieved = dom_bytes / (dom_ms * 1e-3) / 1e9
+    out = {
+        "metric": "SO3vec CGproduct fwd+bwd samples/s at L=4; achieved HBM GB/s vs peak",
+        "value": B / (ms_per_step * 1e-3),
+        "unit": "samples/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": name, "batch": B, "tau_x": {str(k): v for k, v in tx.items()},
+                   "tau_y": {str(k): v for k, v in ty.items()}, "maxl": maxl, "diag": diag,
+                   "triples": sum(1 for l1 in tx for l2 in ty for l in range(abs(l1 - l2), l1 + l2 + 1) if l in tr),
+                   "kernel_path": {1: "generic", 2: "unrolled"}.get(path, str(path)),
+                   "fwd_ms": fwd_ms, "bwd_ms": bwd_ms,
+                   "fwd_GBps": fwd_bytes / (fwd_ms * 1e-3) / 1e9, "bwd_GBps": bwd_bytes / (bwd_ms * 1e-3) / 1e9,
+                   "fwd_bwd_GBps": (fwd_bytes + bwd_bytes) / ((fwd_ms + bwd_ms) * 1e-3) / 1e9,
+                   "fwd_bwd_frac_of_peak": (fwd_bytes + bwd_bytes) / ((fwd_ms + bwd_ms) * 1e-3) / HBM_PEAK},
+        "roofline": {"bound": "hbm", "kernel": dom, "achieved": achieved, "peak": HBM_PEAK / 1e9, "unit": "GB/s",
+                     "frac": achieved * 1e9 / HBM_PEAK, "traffic": None,
+                     "algorithmic_bytes_per_launch": dom_bytes},
+    }
+    if not args.no_cpu:
+        ns = min(args.cpu_samples, B)
+        sps, dt, parity = cpu_baseline(torch, xs, ys, gs, rs, xgs, ygs, maxl, diag, ns)
+        out["cpu_baseline"] = {"value": sps, "unit": "samples/s", "cores": 1, "kind": "port",
+                               "sample": "first %d samples of the same batch, fwd+bwd, %.1f s" % (ns, dt)}
+        out["parity"] = parity
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,391 @@
+// Host side of the unrolled small-l kernels: eligibility, collapsing (batch, grid0, grid1) into one cell index,
+// the per-signature device tables (pairs + coefficient bank) and the per-call block schedule.
+#include <algorithm>
+#include <cstring>
+#include <map>
+#include <mutex>
+#include <vector>
+
+#include "cg_unrolled_dev.h"
+
+namespace gelib_hip {
+
+namespace {
+
+int g_fwd_block_bytes = 384 * 1024;  // product bytes one forward block aims to write
+int g_fwd_ti = 0;                    // 0 = widest tile that divides every n1, else force 1 / 2 / 4
+int g_bwd_enable = 1;
+int g_fwd_enable = 1;
+
+struct DevicePlan {
+  std::vector<PairRec> pairs;
+  PairRec *d_pairs = nullptr;
+  float *d_bank = nullptr;
+  int bank_len = 0;
+  int xsize = 0, ysize = 0;
+};
+
+std::mutex g_plan_mutex;
+std::map<std::vector<int>, DevicePlan> g_plans;  // key starts with the device ordinal
+
+// (b, g0, g1) -> one cell index with one stride, if the strides nest; broadcast-everywhere gives stride 0.
+bool collapse(const PartDev &p, const long long E[3], const long long own[3], long long *cell_stride) {
+  const long long s[3] = {p.sb, p.sg0, p.sg1};
+  int dims[3], nd = 0;
+  for (int d = 0; d < 3; d++)
+    if (E[d] > 1) dims[nd++] = d;
+  if (nd == 0) {
+    *cell_stride = 0;
+    return true;
+  }
+  bool all_bcast = true, none_bcast = true;
+  for (int k = 0; k < nd; k++) {
+    if (own[dims[k]] == E[dims[k]]) all_bcast = false;
+    else none_bcast = false;
+  }
+  if (all_bcast) {
+    *cell_stride = 0;
+    return true;
+  }
+  if (!none_bcast) return false;
+  for (int k = 0; k + 1 < nd; k++)
+    if (s[dims[k]] != E[dims[k + 1]] * s[dims[k + 1]]) return false;
+  *cell_stride = s[dims[nd - 1]];
+  return true;
+}
+
+bool to_fast(const PartDev &p, const long long E[3], const long long own[3], int n, bool is_dest, FastPart *out) {
+  if (n > 1 && p.sc != 1) return false;
+  if (p.sm < 0 || p.sm > 0x3fffffffLL) return false;
+  long long cs;
+  if (!collapse(p, E, own, &cs)) return false;
+  const long long cells = E[0] * E[1] * E[2];
+  if (is_dest && cells > 1 && cs == 0) return false;  // a broadcast destination needs a reduction over cells
+  out->ptr = p.ptr;
+  out->sb = cs;
+  out->sm = (int)p.sm;
+  out->n = n;
+  return true;
+}
+
+PartDev desc_to_dev(const gelib_part_desc *d, const long long E[3], long long own[3]) {
+  PartDev p;
+  p.ptr = (float2 *)d->ptr;
+  long long s[3];
+  for (int k = 0; k < 3; k++) {
+    own[k] = (d->dims[k] == E[k]) ? E[k] : 1;
+    s[k] = (d->dims[k] == E[k] && E[k] > 1) ? d->strides[k] : 0;
+  }
+  p.sb = s[0];
+  p.sg0 = s[1];
+  p.sg1 = s[2];
+  p.sm = d->strides[3];
+  p.sc = d->strides[4];
+  return p;
+}
+
+// Build (or fetch) the device tables for a list of triples.  xs/ys/rs give (l, n) of the l-sorted parts.
+int get_plan(bool diag, const std::vector<VecTriple> &triples, const std::vector<std::pair<int, int>> &xs,
+             const std::vector<std::pair<int, int>> &ys, const std::vector<int> &rls, const DevicePlan **out) {
+  int dev = 0;
+  GELIB_HIP_TRY(hipGetDevice(&dev));
+  std::vector<int> key = {dev, diag ? 1 : 0, (int)xs.size(), (int)ys.size(), (int)rls.size()};
+  for (auto &v : xs) key.push_back(v.first), key.push_back(v.second);
+  for (auto &v : ys) key.push_back(v.first), key.push_back(v.second);
+  for (int l : rls) key.push_back(l);
+  for (auto &t : triples) key.push_back(t.ri), key.push_back(t.offs);
+  std::lock_guard<std::mutex> lock(g_plan_mutex);
+  auto it = g_plans.find(key);
+  if (it != g_plans.end()) {
+    *out = &it->second;
+    return GELIB_HIP_OK;
+  }
+  DevicePlan plan;
+  std::vector<float> bank;
+  std::vector<int> xoff(xs.size()), yoff(ys.size());
+  for (size_t i = 0; i < xs.size(); i++) {
+    xoff[i] = plan.xsize;
+    plan.xsize += (2 * xs[i].first + 1) * xs[i].second;
+  }
+  for (size_t i = 0; i < ys.size(); i++) {
+    yoff[i] = plan.ysize;
+    plan.ysize += (2 * ys[i].first + 1) * ys[i].second;
+  }
+  for (auto &t : triples) {
+    PairRec *p = nullptr;
+    if (!plan.pairs.empty() && plan.pairs.back().xi == t.xi && plan.pairs.back().yi == t.yi) p = &plan.pairs.back();
+    if (!p) {
+      PairRec rec;
+      std::memset(&rec, 0, sizeof(rec));
+      rec.xi = t.xi;
+      rec.yi = t.yi;
+      rec.l1 = t.l1;
+      rec.l2 = t.l2;
+      rec.n1 = xs[t.xi].second;
+      rec.n2 = ys[t.yi].second;
+      for (int d = 0; d < kMaxDl; d++) rec.ri[d] = -1;
+      rec.cg_base = (int)bank.size();
+      rec.xoff = xoff[t.xi];
+      rec.yoff = yoff[t.yi];
+      plan.pairs.push_back(rec);
+      p = &plan.pairs.back();
+    }
+    const int dl = t.l - std::abs(t.l1 - t.l2);
+    p->ri[dl] = t.ri;
+    p->offs[dl] = t.offs;
+    p->cg[dl] = (int)bank.size() - p->cg_base;
+    const size_t n = (size_t)(2 * t.l1 + 1) * (2 * t.l2 + 1);
+    bank.resize(bank.size() + n);
+    cg_matrix_host(t.l1, t.l2, t.l, bank.data() + bank.size() - n);
+    p->cg_len = (int)bank.size() - p->cg_base;
+  }
+  plan.bank_len = (int)bank.size();
+  const size_t pair_bytes = plan.pairs.size() * sizeof(PairRec);
+  const size_t bank_bytes = bank.size() * sizeof(float);
+  char *d = nullptr;
+  GELIB_HIP_TRY(hipMalloc((void **)&d, pair_bytes + bank_bytes));
+  hipError_t e = hipMemcpy(d, plan.pairs.data(), pair_bytes, hipMemcpyHostToDevice);
+  if (e == hipSuccess) e = hipMemcpy(d + pair_bytes, bank.data(), bank_bytes, hipMemcpyHostToDevice);
+  if (e != hipSuccess) {
+    (void)hipFree(d);
+    return record_hip_error(e, "hipMemcpy(plan)");
+  }
+  plan.d_pairs = (PairRec *)d;
+  plan.d_bank = (float *)(d + pair_bytes);
+  auto ins = g_plans.emplace(key, std::move(plan));
+  *out = &ins.first->second;
+  return GELIB_HIP_OK;
+}
+
+bool is_pow2(int v) { return v > 0 && (v & (v - 1)) == 0; }
+int ilog2(int v) {
+  int k = 0;
+  while ((1 << k) < v) k++;
+  return k;
+}
+
+struct FastLists {
+  std::vector<FastPart> x, y, r, xg, yg;
+};
+
+int run_fwd(bool diag, const std::vector<VecTriple> &triples, const std::vector<std::pair<int, int>> &xs,
+            const std::vector<std::pair<int, int>> &ys, const std::vector<int> &rls, const FastLists &f,
+            long long ncells, int offs_add, bool accumulate, hipStream_t s) {
+  const DevicePlan *plan = nullptr;
+  int rc = get_plan(diag, triples, xs, ys, rls, &plan);
+  if (rc) return rc;
+  FwdArgs a;
+  std::memset(&a, 0, sizeof(a));
+  for (size_t i = 0; i < f.x.size(); i++) a.x[i] = f.x[i];
+  for (size_t i = 0; i < f.y.size(); i++) a.y[i] = f.y[i];
+  for (size_t i = 0; i < f.r.size(); i++) a.r[i] = f.r[i];
+  a.pairs = plan->d_pairs;
+  a.bank = plan->d_bank;
+  a.ncells = ncells;
+  a.npairs = (int)plan->pairs.size();
+  a.offs_add = offs_add;
+  a.accumulate = accumulate ? 1 : 0;
+  int ti = 1;
+  if (!diag) {
+    ti = 4;
+    for (auto &p : plan->pairs) {
+      while (ti > 1 && p.n1 % ti) ti >>= 1;
+    }
+    if (g_fwd_ti == 1 || g_fwd_ti == 2 || g_fwd_ti == 4) ti = std::min(ti, g_fwd_ti);
+  }
+  long long nblocks = 0;
+  for (int i = 0; i < a.npairs; i++) {
+    const PairRec &p = plan->pairs[i];
+    long long rows = 0;
+    for (int d = 0; d < kMaxDl; d++)
+      if (p.ri[d] >= 0) rows += 2 * (std::abs(p.l1 - p.l2) + d) + 1;
+    const long long nout = diag ? p.n1 : (long long)p.n1 * p.n2;
+    const long long bytes_per_cell = rows * nout * 8;
+    const long long U = diag ? p.n1 : (long long)(p.n1 / ti) * p.n2;
+    long long cpb = std::max<long long>(1, g_fwd_block_bytes / std::max<long long>(1, bytes_per_cell));
+    cpb = std::max(cpb, (kBlock + U - 1) / U);  // at least one full pass of the block
+    cpb = std::min<long long>(cpb, std::max<long long>(1, (1LL << 28) / std::max<long long>(1, U)));
+    cpb = std::min(cpb, ncells);
+    a.cpb[i] = (int)cpb;
+    a.first_block[i] = (int)nblocks;
+    nblocks += (ncells + cpb - 1) / cpb;
+    if (nblocks > 0x7fffffffLL) return GELIB_HIP_ERR_ARG;
+  }
+  a.first_block[a.npairs] = (int)nblocks;
+  return launch_unrolled_fwd(a, diag, ti, (int)nblocks, s);
+}
+
+int run_bwd(bool diag, const std::vector<VecTriple> &triples, const std::vector<std::pair<int, int>> &xs,
+            const std::vector<std::pair<int, int>> &ys, const std::vector<int> &rls, const FastLists &f,
+            long long ncells, int offs_add, bool accumulate, bool want_x, bool want_y, hipStream_t s, int *used) {
+  *used = 0;
+  // channel counts must be powers of two, the reduced operand must fit a wave, and every pair must cover the
+  // same number of cells per wave
+  int u_common = -1;
+  bool big = true;
+  for (auto &t : triples) {
+    const int n1 = xs[t.xi].second, n2 = ys[t.yi].second;
+    if (!is_pow2(n1) || !is_pow2(n2)) return GELIB_HIP_OK;
+    if (!diag && n2 > kWave) return GELIB_HIP_OK;
+    const int U = diag ? n1 : n1 * n2;
+    if (U < kWave) big = false;
+    if (u_common < 0) u_common = U;
+    else if (u_common != U) u_common = 0;
+  }
+  if (!big && u_common <= 0) return GELIB_HIP_OK;
+  const DevicePlan *plan = nullptr;
+  int rc = get_plan(diag, triples, xs, ys, rls, &plan);
+  if (rc) return rc;
+  BwdArgs a;
+  std::memset(&a, 0, sizeof(a));
+  for (size_t i = 0; i < f.x.size(); i++) a.x[i] = f.x[i];
+  for (size_t i = 0; i < f.y.size(); i++) a.y[i] = f.y[i];
+  for (size_t i = 0; i < f.r.size(); i++) a.g[i] = f.r[i];
+  for (size_t i = 0; i < f.xg.size(); i++) a.xg[i] = f.xg[i];
+  for (size_t i = 0; i < f.yg.size(); i++) a.yg[i] = f.yg[i];
+  a.pairs = plan->d_pairs;
+  a.bank = plan->d_bank;
+  a.ncells = ncells;
+  a.npairs = (int)plan->pairs.size();
+  a.nx = (int)xs.size();
+  a.ny = (int)ys.size();
+  a.offs_add = offs_add;
+  a.accumulate = accumulate ? 1 : 0;
+  a.want_x = want_x ? 1 : 0;
+  a.want_y = want_y ? 1 : 0;
+  a.bank_len = plan->bank_len;
+  a.xsize = plan->xsize;
+  a.ysize = plan->ysize;
+  for (size_t i = 0; i < xs.size(); i++) a.xrows[i] = 2 * xs[i].first + 1;
+  for (size_t i = 0; i < ys.size(); i++) a.yrows[i] = 2 * ys[i].first + 1;
+  a.cells_per_wave = big ? 1 : kWave / u_common;
+  a.log2_u = big ? 6 : ilog2(u_common);
+  const int waves = kBlock / kWave;
+  const size_t lds = sizeof(float) * (size_t)((a.bank_len + 1) & ~1) +
+                     sizeof(float2) * (size_t)waves * a.cells_per_wave * ((size_t)a.xsize + a.ysize);
+  if (lds > 150 * 1024) return GELIB_HIP_OK;
+  const long long cells_per_block = (long long)waves * a.cells_per_wave;
+  const long long nblocks = (ncells + cells_per_block - 1) / cells_per_block;
+  if (nblocks > 0x7fffffffLL) return GELIB_HIP_ERR_ARG;
+  rc = launch_unrolled_bwd(a, diag, (int)nblocks, lds, s);
+  if (rc) return rc;
+  *used = 1;
+  return GELIB_HIP_OK;
+}
+
+}  // namespace
+
+int unrolled_part(int kind, const PartOp &op, bool accumulate, hipStream_t s, int *used) {
+  *used = 0;
+  if (op.l1 > kLT || op.l2 > kLT) return GELIB_HIP_OK;
+  if (kind == 0 && !g_fwd_enable) return GELIB_HIP_OK;
+  if (kind != 0 && !g_bwd_enable) return GELIB_HIP_OK;
+  FastLists f;
+  f.x.resize(1);
+  f.y.resize(1);
+  f.r.resize(1);
+  if (!to_fast(op.r, op.E, op.Dr, op.offs + op.nout, kind == 0, &f.r[0])) return GELIB_HIP_OK;
+  if (!to_fast(op.x, op.E, op.Dx, op.n1, kind == 1, &f.x[0])) return GELIB_HIP_OK;
+  if (!to_fast(op.y, op.E, op.Dy, op.n2, kind == 2, &f.y[0])) return GELIB_HIP_OK;
+  const long long ncells = op.E[0] * op.E[1] * op.E[2];
+  std::vector<VecTriple> triples = {{0, 0, 0, op.l1, op.l2, op.l, 0, op.nout}};
+  std::vector<std::pair<int, int>> xs = {{op.l1, op.n1}}, ys = {{op.l2, op.n2}};
+  std::vector<int> rls = {op.l};
+  if (kind == 0) {
+    int rc = run_fwd(op.diag, triples, xs, ys, rls, f, ncells, op.offs, accumulate, s);
+    if (rc) return rc;
+    *used = 1;
+    return GELIB_HIP_OK;
+  }
+  if (kind == 1) f.xg = f.x;  // destination
+  if (kind == 2) f.yg = f.y;
+  return run_bwd(op.diag, triples, xs, ys, rls, f, ncells, op.offs, accumulate, kind == 1, kind == 2, s, used);
+}
+
+namespace {
+bool lists_to_fast(const std::vector<const gelib_part_desc *> &ds, const long long E[3], bool is_dest,
+                   std::vector<FastPart> *out, std::vector<std::pair<int, int>> *ln) {
+  out->resize(ds.size());
+  for (size_t i = 0; i < ds.size(); i++) {
+    long long own[3];
+    PartDev p = desc_to_dev(ds[i], E, own);
+    const int l = (int)(ds[i]->dims[3] - 1) / 2, n = (int)ds[i]->dims[4];
+    if (!to_fast(p, E, own, n, is_dest, &(*out)[i])) return false;
+    if (ln) ln->push_back({l, n});
+  }
+  return true;
+}
+}  // namespace
+
+int unrolled_vec_fwd(const VecPlan &plan, const std::vector<const gelib_part_desc *> &r,
+                     const std::vector<const gelib_part_desc *> &x, const std::vector<const gelib_part_desc *> &y,
+                     bool accumulate, hipStream_t s, int *used) {
+  *used = 0;
+  if (!g_fwd_enable) return GELIB_HIP_OK;
+  if (x.size() > (size_t)kFastIn || y.size() > (size_t)kFastIn || r.size() > (size_t)kFastOut) return GELIB_HIP_OK;
+  for (auto &t : plan.triples)
+    if (t.l1 > kLT || t.l2 > kLT) return GELIB_HIP_OK;
+  for (auto *d : x)
+    if ((d->dims[3] - 1) / 2 > kLT) return GELIB_HIP_OK;
+  for (auto *d : y)
+    if ((d->dims[3] - 1) / 2 > kLT) return GELIB_HIP_OK;
+  FastLists f;
+  std::vector<std::pair<int, int>> xs, ys, rs;
+  if (!lists_to_fast(x, plan.E, false, &f.x, &xs) || !lists_to_fast(y, plan.E, false, &f.y, &ys) ||
+      !lists_to_fast(r, plan.E, true, &f.r, &rs))
+    return GELIB_HIP_OK;
+  std::vector<int> rls;
+  for (auto &v : rs) rls.push_back(v.first);
+  const long long ncells = plan.E[0] * plan.E[1] * plan.E[2];
+  int rc = run_fwd(plan.diag, plan.triples, xs, ys, rls, f, ncells, 0, accumulate, s);
+  if (rc) return rc;
+  *used = 1;
+  return GELIB_HIP_OK;
+}
+
+int unrolled_vec_bwd(const VecPlan &plan, const std::vector<const gelib_part_desc *> &g,
+                     const std::vector<const gelib_part_desc *> &x, const std::vector<const gelib_part_desc *> &y,
+                     const std::vector<const gelib_part_desc *> &xg, const std::vector<const gelib_part_desc *> &yg,
+                     bool accumulate, hipStream_t s, int *used) {
+  *used = 0;
+  if (!g_bwd_enable) return GELIB_HIP_OK;
+  if (x.size() > (size_t)kFastIn || y.size() > (size_t)kFastIn || g.size() > (size_t)kFastOut) return GELIB_HIP_OK;
+  for (auto *d : x)
+    if ((d->dims[3] - 1) / 2 > kLT) return GELIB_HIP_OK;
+  for (auto *d : y)
+    if ((d->dims[3] - 1) / 2 > kLT) return GELIB_HIP_OK;
+  FastLists f;
+  std::vector<std::pair<int, int>> xs, ys, rs;
+  if (!lists_to_fast(x, plan.E, false, &f.x, &xs) || !lists_to_fast(y, plan.E, false, &f.y, &ys) ||
+      !lists_to_fast(g, plan.E, false, &f.r, &rs))
+    return GELIB_HIP_OK;
+  if (!xg.empty() && !lists_to_fast(xg, plan.E, true, &f.xg, nullptr)) return GELIB_HIP_OK;
+  if (!yg.empty() && !lists_to_fast(yg, plan.E, true, &f.yg, nullptr)) return GELIB_HIP_OK;
+  std::vector<int> rls;
+  for (auto &v : rs) rls.push_back(v.first);
+  const long long ncells = plan.E[0] * plan.E[1] * plan.E[2];
+  return run_bwd(plan.diag, plan.triples, xs, ys, rls, f, ncells, 0, accumulate, !xg.empty(), !yg.empty(), s, used);
+}
+
+int unrolled_set_option(const char *name, int value) {
+  if (!std::strcmp(name, "fwd_block_bytes")) {
+    if (value < 1024) return GELIB_HIP_ERR_ARG;
+    g_fwd_block_bytes = value;
+    return GELIB_HIP_OK;
+  }
+  if (!std::strcmp(name, "fwd_tile")) {
+    g_fwd_ti = value;
+    return GELIB_HIP_OK;
+  }
+  if (!std::strcmp(name, "unrolled_fwd")) {
+    g_fwd_enable = value;
+    return GELIB_HIP_OK;
+  }
+  if (!std::strcmp(name, "unrolled_bwd")) {
+    g_bwd_enable = value;
+    return GELIB_HIP_OK;
+  }
+  return GELIB_HIP_ERR_ARG;
+}
+
+}  // namespace gelib_hip

@@ -47,6 +47,7 @@ struct PairRec {
   int cg_base;       // offset (floats) of this pair's tables in the bank that follows the pair array
   int cg_len;        // floats of coefficient tables belonging to this pair
   int xoff, yoff;    // offsets (complex elements) of the parts inside a per-cell packed x / y image (backward)
+  int log2_u;        // log2 of the channel slots per cell (n1*n2, or n for Diag) when that is a power of two, else -1
 };
 
 // kind: 0 forward, 1 back0 (destination op.x), 2 back1 (destination op.y).  *used = 1 if a launch was made.

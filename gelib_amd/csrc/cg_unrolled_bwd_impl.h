@@ -1,0 +1,409 @@
+// Backward CG / DiagCG product for l1, l2 <= kLT: both gradients from one pass over g, all triples in one launch.
+//
+// Work split.  A block owns a few whole cells (one cell when a cell has >= 256 channel slots).  The operands x, y
+// of those cells are staged once in LDS next to the coefficient bank.  For every (l1,l2) pair the flattened
+// (cell, slot) space is cut into runs of 64 slots; a wave takes every fourth run.  In a run a lane owns one
+// channel pair (i, j) of the gradient block: it reads g[m, i*n2+j] for every m (contiguous across the wave), forms
+// C*g once per (m1,m2) and feeds two complex FMAs,
+//     ax[m1] += (C g) conj(y[m2, j])        ay[m2] += (C g) conj(x[m1, i]),
+// with all m-loops unrolled and x, y, ax, ay, g in registers.  ax is then summed over j inside aligned groups of
+// n2 lanes (DPP butterflies), ay over i with butterflies at lane distance n2 and up, and one lane per group adds
+// the result into the wave's private image of xg / yg in LDS: plain read-add-write in a fixed order, no atomics,
+// no barrier.  After the last pair the four images are summed and written out in contiguous rows.
+//
+// Latency hiding.  The rows of g for the next (pair, run, l) unit are requested before the arithmetic of the
+// current unit starts and land in a second register buffer, so a wave always has one unit of loads in flight.
+#pragma once
+
+#include "cg_unrolled_dev.h"
+
+namespace gelib_hip {
+
+namespace {
+
+constexpr int cabs_(int a) { return a < 0 ? -a : a; }
+constexpr int cmin_(int a, int b) { return a < b ? a : b; }
+constexpr int kWaves = kBlock / kWave;
+
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+
+// Sum every element of v over aligned groups of n lanes (n a power of two <= 64); all lanes of a group end with
+// the totals.  One uniform branch per butterfly step, not per element.
+template <int K>
+__device__ __forceinline__ void group_sum(float2 (&v)[K], int n) {
+#define GELIB_STEP(COND, EXPR_X, EXPR_Y)    \
+  if (COND) {                               \
+    _Pragma("unroll") for (int k = 0; k < K; k++) { \
+      v[k].x += EXPR_X;                     \
+      v[k].y += EXPR_Y;                     \
+    }                                       \
+  }
+  GELIB_STEP(n > 1, dpp_move<0xB1>(v[k].x), dpp_move<0xB1>(v[k].y))    // quad_perm [1,0,3,2]
+  GELIB_STEP(n > 2, dpp_move<0x4E>(v[k].x), dpp_move<0x4E>(v[k].y))    // quad_perm [2,3,0,1]
+  GELIB_STEP(n > 4, dpp_move<0x141>(v[k].x), dpp_move<0x141>(v[k].y))  // row_half_mirror
+  GELIB_STEP(n > 8, dpp_move<0x140>(v[k].x), dpp_move<0x140>(v[k].y))  // row_mirror
+  GELIB_STEP(n > 16, __shfl_xor(v[k].x, 16), __shfl_xor(v[k].y, 16))
+  GELIB_STEP(n > 32, __shfl_xor(v[k].x, 32), __shfl_xor(v[k].y, 32))
+#undef GELIB_STEP
+}
+
+// Sum every element of v over lanes that differ in the bits from `lo` up to (but not including) `hi`.
+template <int K>
+__device__ __forceinline__ void stride_sum(float2 (&v)[K], int lo, int hi) {
+  for (int s = lo; s < hi; s <<= 1) {
+#pragma unroll
+    for (int k = 0; k < K; k++) {
+      v[k].x += __shfl_xor(v[k].x, s);
+      v[k].y += __shfl_xor(v[k].y, s);
+    }
+  }
+}
+
+// All g, x, y pointers that the arithmetic loops dereference are typed as global memory, so the loads are
+// global_load (vmcnt only) rather than flat_load (which also ties up the LDS counter).
+typedef float v2f __attribute__((ext_vector_type(2)));
+typedef const __attribute__((address_space(1))) v2f *GlobalRows;
+
+// Where a lane finds the rows of g of one unit; rows == 0 means "nothing to load".
+struct GRows {
+  GlobalRows ptr;
+  int sm;
+  int rows;
+};
+
+// Coefficients are read through the constant address space: the address is the same for every lane, so the
+// compiler fetches them with scalar loads into SGPRs and they cost neither vector registers nor LDS traffic.
+typedef const __attribute__((address_space(4))) float *CoeffPtr;
+
+template <int ROWS, int KR>
+__device__ __forceinline__ void load_rows_static(float2 (&buf)[KR], GlobalRows ptr, int sm) {
+#pragma unroll
+  for (int m = 0; m < ROWS; m++) {
+    const v2f t = ptr[m * sm];
+    buf[m] = make_float2(t.x, t.y);
+  }
+}
+
+// rows is 2l+1 for some l <= (KR-1)/2, or 0: one jump, then straight-line loads
+template <int KR>
+__device__ __forceinline__ void load_rows(float2 (&buf)[KR], const GRows &d) {
+  static_for<(KR + 1) / 2>([&](auto lc) __attribute__((always_inline)) {
+    constexpr int rows = 2 * decltype(lc)::value + 1;
+    if (d.rows == rows) load_rows_static<rows, KR>(buf, d.ptr, d.sm);
+  });
+}
+
+template <int L1, int L2, int L, int KR, bool WX, bool WY>
+__device__ __forceinline__ void triple_bwd(const float2 (&xv)[2 * L1 + 1], const float2 (&yv)[2 * L2 + 1],
+                                           float2 (&ax)[2 * L1 + 1], float2 (&ay)[2 * L2 + 1],
+                                           CoeffPtr C, const float2 (&g)[KR]) {
+#pragma unroll
+  for (int m1 = -L1; m1 <= L1; m1++) {
+#pragma unroll
+    for (int m2 = -L2; m2 <= L2; m2++) {
+      const int m = m1 + m2;
+      if (m >= -L && m <= L) {
+        const float c = C[(m1 + L1) * (2 * L2 + 1) + (m2 + L2)];
+        const float tr = c * g[m + L].x, ti = c * g[m + L].y;
+        if (WX) {
+          const float2 yc = yv[m2 + L2];
+          ax[m1 + L1].x = fmaf(tr, yc.x, ax[m1 + L1].x);
+          ax[m1 + L1].x = fmaf(ti, yc.y, ax[m1 + L1].x);
+          ax[m1 + L1].y = fmaf(ti, yc.x, ax[m1 + L1].y);
+          ax[m1 + L1].y = fmaf(-tr, yc.y, ax[m1 + L1].y);
+        }
+        if (WY) {
+          const float2 xc = xv[m1 + L1];
+          ay[m2 + L2].x = fmaf(tr, xc.x, ay[m2 + L2].x);
+          ay[m2 + L2].x = fmaf(ti, xc.y, ay[m2 + L2].x);
+          ay[m2 + L2].y = fmaf(ti, xc.x, ay[m2 + L2].y);
+          ay[m2 + L2].y = fmaf(-tr, xc.y, ay[m2 + L2].y);
+        }
+      }
+    }
+  }
+}
+
+// The gradient parts, indexed by their l (the host fills BwdArgs::g that way), copied out of the kernel arguments
+// once so that the unrolled code can name them with compile-time indices.
+template <int LCAP>
+struct GParts {
+  FastPart G[LCAP + 1];
+};
+
+typedef const __attribute__((address_space(4))) PairRec *PairPtr;
+
+// Position of a lane in one run of 64 slots of a pair.
+struct LanePos {
+  int cell_local;  // cell inside the block
+  int u;           // channel slot inside the cell
+  bool live;
+};
+
+__device__ __forceinline__ LanePos lane_pos(int run, int lane, int log2_u, int ncell) {
+  const int flat = (run << 6) + lane;
+  LanePos q;
+  q.cell_local = flat >> log2_u;
+  q.u = flat & ((1 << log2_u) - 1);
+  q.live = q.cell_local < ncell;
+  if (!q.live) q.cell_local = ncell - 1;  // dead lanes read valid memory and never store
+  return q;
+}
+
+// gdesc: the gradient parts by l, in LDS, for the one place where l is only known at run time
+template <int LCAP>
+__device__ __forceinline__ GRows first_unit(const FastPart *gdesc, PairPtr p, long long cell, int u, int offs_add) {
+  GRows d;
+  const int lmin = cabs_(p->l1 - p->l2);
+  const FastPart G = gdesc[lmin];
+  d.rows = (lmin <= LCAP && p->ri[0] >= 0) ? 2 * lmin + 1 : 0;
+  d.sm = G.sm;
+  d.ptr = (GlobalRows)G.ptr + cell * G.sb + (p->offs[0] + offs_add + u);
+  return d;
+}
+
+// One run of one pair.  On entry gcur holds (or is about to receive) the rows of the pair's first l; on exit it
+// holds the rows described by `after`, the first unit of whatever the wave does next.
+template <int L1, int L2, int LCAP, int KR, bool DIAG, bool WX, bool WY>
+__device__ __forceinline__ void pair_bwd(const GParts<LCAP> &gp, PairPtr pr, CoeffPtr Cs, const float2 *xs,
+                                         const float2 *ys, float2 *xacc, float2 *yacc, int xsize, int ysize,
+                                         long long cell0, int offs_add, const LanePos q, float2 (&gcur)[KR],
+                                         const GRows after) {
+  constexpr int LMIN = cabs_(L1 - L2);
+  constexpr int NL = 2 * cmin_(L1, L2) + 1;
+  if constexpr (LMIN > LCAP) {  // no l of this pair can be present; just keep the pipeline fed
+    load_rows<KR>(gcur, after);
+    return;
+  }
+  // scalar loads: the record sits in constant memory and the pointer is uniform
+  const __attribute__((address_space(4))) PairRec &p = *pr;
+  const int N1 = p.n1, N2 = p.n2;
+  const int lg_n2 = DIAG ? 0 : 31 - __clz(N2);
+  const int i = DIAG ? q.u : (q.u >> lg_n2);
+  const int j = DIAG ? q.u : (q.u & (N2 - 1));
+  const int span = p.log2_u < 6 ? (1 << p.log2_u) : kWave;  // lanes of a run that belong to one cell
+  const long long cell = cell0 + q.cell_local;
+
+  float2 xv[2 * L1 + 1], yv[2 * L2 + 1], ax[2 * L1 + 1], ay[2 * L2 + 1];
+  if (WY) {
+    const float2 *xp = xs + q.cell_local * xsize + p.xoff + i;
+#pragma unroll
+    for (int m1 = 0; m1 <= 2 * L1; m1++) xv[m1] = xp[m1 * N1];
+  }
+  if (WX) {
+    const float2 *yp = ys + q.cell_local * ysize + p.yoff + j;
+#pragma unroll
+    for (int m2 = 0; m2 <= 2 * L2; m2++) yv[m2] = yp[m2 * N2];
+  }
+#pragma unroll
+  for (int m1 = 0; m1 <= 2 * L1; m1++) ax[m1] = make_float2(0.f, 0.f);
+#pragma unroll
+  for (int m2 = 0; m2 <= 2 * L2; m2++) ay[m2] = make_float2(0.f, 0.f);
+
+  static_for<NL>([&](auto dl_c) __attribute__((always_inline)) {
+    constexpr int dl = decltype(dl_c)::value;
+    constexpr int L = LMIN + dl;
+    if constexpr (L <= LCAP) {
+      // request the rows of the following unit before touching the current ones
+      float2 gnext[KR];
+      if constexpr (dl + 1 < NL && L + 1 <= LCAP) {
+        if (p.ri[dl + 1] >= 0) {
+          const FastPart G = gp.G[L + 1];
+          load_rows_static<2 * (L + 1) + 1, KR>(gnext, (GlobalRows)G.ptr + cell * G.sb + (p.offs[dl + 1] + offs_add + q.u),
+                                                G.sm);
+        }
+      } else {
+        load_rows<KR>(gnext, after);
+      }
+      if (p.ri[dl] >= 0) triple_bwd<L1, L2, L, KR, WX, WY>(xv, yv, ax, ay, Cs + p.cg[dl], gcur);
+#pragma unroll
+      for (int m = 0; m < KR; m++) gcur[m] = gnext[m];
+    }
+  });
+
+  if (WX) {
+    if (!DIAG) group_sum(ax, N2);
+    if (q.live && (DIAG || j == 0)) {
+      float2 *xa = xacc + q.cell_local * xsize + p.xoff + i;
+#pragma unroll
+      for (int m1 = 0; m1 <= 2 * L1; m1++) {
+        float2 o = xa[m1 * N1];
+        o.x += ax[m1].x;
+        o.y += ax[m1].y;
+        xa[m1 * N1] = o;
+      }
+    }
+  }
+  if (WY) {
+    if (!DIAG) stride_sum(ay, N2, span);
+    if (q.live && (DIAG || (q.u & (span - 1)) < N2)) {
+      float2 *ya = yacc + q.cell_local * ysize + p.yoff + j;
+#pragma unroll
+      for (int m2 = 0; m2 <= 2 * L2; m2++) {
+        float2 o = ya[m2 * N2];
+        o.x += ay[m2].x;
+        o.y += ay[m2].y;
+        ya[m2 * N2] = o;
+      }
+    }
+  }
+}
+
+// Copies between memory and the packed per-cell LDS image of a part list (each part's rows contiguous).
+// TO_LDS: stage operands.  Otherwise: sum the nsum per-wave images (fixed order) and write the gradient out.
+template <bool TO_LDS>
+__device__ __forceinline__ void copy_image(const FastPart (&parts)[kFastIn], const int (&rows)[kFastIn], int nparts,
+                                           float2 *img, int img_size, long long cell0, int ncell, int nsum,
+                                           int sum_stride, bool accumulate) {
+  int off = 0;
+  static_for<kFastIn>([&](auto kc) __attribute__((always_inline)) {
+    constexpr int k = decltype(kc)::value;
+    if (k < nparts) {
+      const FastPart P = parts[k];
+      const int per_cell = rows[k] * P.n;
+      const int total = per_cell * ncell;
+      for (int e = threadIdx.x; e < total; e += kBlock) {
+        const int c = e / per_cell;
+        const int r = e - c * per_cell;
+        const int m = r / P.n;
+        const int ch = r - m * P.n;
+        float2 *gptr = P.ptr + (cell0 + c) * P.sb + m * P.sm + ch;
+        float2 *lptr = img + c * img_size + off + r;
+        if (TO_LDS) {
+          *lptr = *gptr;
+        } else {
+          float2 v = lptr[0];
+          for (int w = 1; w < nsum; w++) {
+            const float2 t = lptr[w * sum_stride];
+            v.x += t.x;
+            v.y += t.y;
+          }
+          if (accumulate) {
+            const float2 o = *gptr;
+            v.x += o.x;
+            v.y += o.y;
+          }
+          *gptr = v;
+        }
+      }
+      off += per_cell;
+    }
+  });
+}
+
+template <int LCAP, bool DIAG, bool WX, bool WY>
+__global__ void __launch_bounds__(kBlock) unrolled_bwd_kernel(const BwdArgs a) {
+  constexpr int KR = 2 * LCAP + 1;
+  extern __shared__ float lds[];
+  const int xsize = a.xsize, ysize = a.ysize, cpb = a.cells_per_block;
+  float2 *xs = reinterpret_cast<float2 *>(lds);  // staged operands of the block's cells
+  float2 *ys = xs + cpb * xsize;
+  float2 *xacc_all = ys + cpb * ysize;                 // [wave][cell][xsize]
+  float2 *yacc_all = xacc_all + kWaves * cpb * xsize;  // [wave][cell][ysize]
+
+  const long long cell0 = (long long)blockIdx.x * cpb;
+  const long long left = a.ncells - cell0;
+  const int ncell = left < cpb ? (int)left : cpb;
+  // readfirstlane tells the compiler the wave index is uniform, so everything derived from it (which pair, which
+  // run) stays in scalar registers and branches on it are scalar branches
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & (kWave - 1);
+
+  if (WY) copy_image<true>(a.x, a.xrows, a.nx, xs, xsize, cell0, ncell, 0, 0, false);
+  if (WX) copy_image<true>(a.y, a.yrows, a.ny, ys, ysize, cell0, ncell, 0, 0, false);
+  __shared__ FastPart gdesc[kFastOut];
+  if (threadIdx.x == 0)
+    static_for<kFastOut>([&](auto l) __attribute__((always_inline)) { gdesc[l.value] = a.g[l.value]; });
+  {
+    const int nacc = kWaves * cpb * (xsize + ysize);
+    for (int i = threadIdx.x; i < nacc; i += kBlock) xacc_all[i] = make_float2(0.f, 0.f);
+  }
+  __syncthreads();
+
+  float2 *xacc = xacc_all + wave * cpb * xsize;
+  float2 *yacc = yacc_all + wave * cpb * ysize;
+
+  // The wave's visits: for each pair in turn, runs wave, wave+4, ... of the pair's cpb*U slots.
+  const PairPtr pairs = (PairPtr)a.pairs;
+  const int npairs = a.npairs, offs_add = a.offs_add;
+  auto runs_of = [&](int k) { return ((cpb << pairs[k].log2_u) + kWave - 1) >> 6; };
+  GParts<LCAP> gp;
+  static_for<LCAP + 1>([&](auto l) __attribute__((always_inline)) { gp.G[l.value] = a.g[l.value]; });
+  float2 gcur[KR];
+  int pidx = 0, run = wave;
+  while (pidx < npairs && run >= runs_of(pidx)) {
+    pidx++;
+    run = wave;
+  }
+  if (pidx < npairs) {
+    const LanePos q = lane_pos(run, lane, pairs[pidx].log2_u, ncell);
+    load_rows<KR>(gcur, first_unit<LCAP>(gdesc, pairs + pidx, cell0 + q.cell_local, q.u, offs_add));
+  }
+  while (pidx < npairs) {
+    const PairPtr p = pairs + pidx;
+    const LanePos q = lane_pos(run, lane, p->log2_u, ncell);
+    // look ahead: the first unit of the wave's next visit is requested during this one
+    int npidx = pidx, nrun = run + kWaves;
+    while (npidx < npairs && nrun >= runs_of(npidx)) {
+      npidx++;
+      nrun = wave;
+    }
+    GRows after;
+    after.rows = 0;
+    after.sm = 0;
+    after.ptr = nullptr;
+    if (npidx < npairs) {
+      const LanePos qn = lane_pos(nrun, lane, pairs[npidx].log2_u, ncell);
+      after = first_unit<LCAP>(gdesc, pairs + npidx, cell0 + qn.cell_local, qn.u, offs_add);
+    }
+    CoeffPtr C = (CoeffPtr)(a.bank + p->cg_base);
+    switch (p->l1 * (kLT + 1) + p->l2) {
+#define GELIB_CASE(A, B)                                                                                         \
+  case A * (kLT + 1) + B:                                                                                        \
+    pair_bwd<A, B, LCAP, KR, DIAG, WX, WY>(gp, p, C, xs, ys, xacc, yacc, xsize, ysize, cell0, offs_add, q, gcur, \
+                                            after);                                                              \
+    break;
+#define GELIB_ROW(A) GELIB_CASE(A, 0) GELIB_CASE(A, 1) GELIB_CASE(A, 2) GELIB_CASE(A, 3) GELIB_CASE(A, 4)
+      GELIB_ROW(0) GELIB_ROW(1) GELIB_ROW(2) GELIB_ROW(3) GELIB_ROW(4)
+#undef GELIB_ROW
+#undef GELIB_CASE
+      default: break;
+    }
+    pidx = npidx;
+    run = nrun;
+  }
+
+  __syncthreads();
+  if (WX) copy_image<false>(a.xg, a.xrows, a.nx, xacc_all, xsize, cell0, ncell, kWaves, cpb * xsize, a.accumulate != 0);
+  if (WY) copy_image<false>(a.yg, a.yrows, a.ny, yacc_all, ysize, cell0, ncell, kWaves, cpb * ysize, a.accumulate != 0);
+}
+
+template <int LCAP, bool DIAG, bool WX, bool WY>
+int launch_variant(const BwdArgs &a, int nblocks, size_t lds, hipStream_t s) {
+  auto kern = unrolled_bwd_kernel<LCAP, DIAG, WX, WY>;
+  static bool attr_set = false;  // benign race: setting the attribute twice is harmless
+  if (!attr_set) {
+    GELIB_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                      152 * 1024));  // dynamic LDS above the 64 KB default; 8 KB left for static use
+    attr_set = true;
+  }
+  hipLaunchKernelGGL(kern, dim3(nblocks), dim3(kBlock), lds, s, a);
+  GELIB_HIP_TRY(hipGetLastError());
+  return GELIB_HIP_OK;
+}
+
+// want_x / want_y select which gradients are computed
+template <int LCAP, bool DIAG>
+int launch_bwd_variants(const BwdArgs &a, int nblocks, size_t lds_bytes, hipStream_t s) {
+  static_assert(kLT == 4, "the case table above lists l1, l2 = 0..4");
+  const bool wx = a.want_x != 0, wy = a.want_y != 0;
+  if (wx && wy) return launch_variant<LCAP, DIAG, true, true>(a, nblocks, lds_bytes, s);
+  if (wx) return launch_variant<LCAP, DIAG, true, false>(a, nblocks, lds_bytes, s);
+  return launch_variant<LCAP, DIAG, false, true>(a, nblocks, lds_bytes, s);
+}
+
+}  // namespace
+
+}  // namespace gelib_hip

@@ -25,7 +25,8 @@ struct FwdArgs {
 };
 
 struct BwdArgs {
-  FastPart x[kFastIn], y[kFastIn], g[kFastOut], xg[kFastIn], yg[kFastIn];
+  FastPart x[kFastIn], y[kFastIn], xg[kFastIn], yg[kFastIn];  // in list order (ascending l)
+  FastPart g[kFastOut];                                       // indexed by l itself; absent parts have ptr == nullptr
   const PairRec *pairs;
   const float *bank;
   long long ncells;
@@ -37,9 +38,10 @@ struct BwdArgs {
   int bank_len;     // floats
   int xsize, ysize; // complex elements of one cell's packed x / y image
   int xrows[kFastIn], yrows[kFastIn];  // 2l+1 of each x / y part
-  int cells_per_wave;
-  int log2_u;       // channels-slots per cell are a power of two in the backward kernels
+  int cells_per_block;
 };
+
+size_t unrolled_bwd_lds_bytes(int bank_len, int xsize, int ysize, int cells_per_block);
 
 // Compile-time loop: f(std::integral_constant<int, 0>{}), ..., f(std::integral_constant<int, N-1>{}).
 template <int... Is, class F>
@@ -73,6 +75,7 @@ __device__ __forceinline__ int pick_int(const int (&arr)[N], int i) {
 
 // ti: channels of the first operand handled per thread (1, 2 or 4); must divide every n1.
 int launch_unrolled_fwd(const FwdArgs &a, bool diag, int ti, int nblocks, hipStream_t s);
-int launch_unrolled_bwd(const BwdArgs &a, bool diag, int nblocks, size_t lds_bytes, hipStream_t s);
+// lcap: largest l present in the gradient
+int launch_unrolled_bwd(const BwdArgs &a, bool diag, int lcap, int nblocks, size_t lds_bytes, hipStream_t s);
 
 }  // namespace gelib_hip

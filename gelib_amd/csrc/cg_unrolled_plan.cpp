@@ -84,6 +84,13 @@ PartDev desc_to_dev(const gelib_part_desc *d, const long long E[3], long long ow
   return p;
 }
 
+bool is_pow2(int v) { return v > 0 && (v & (v - 1)) == 0; }
+int ilog2(int v) {
+  int k = 0;
+  while ((1 << k) < v) k++;
+  return k;
+}
+
 // Build (or fetch) the device tables for a list of triples.  xs/ys/rs give (l, n) of the l-sorted parts.
 int get_plan(bool diag, const std::vector<VecTriple> &triples, const std::vector<std::pair<int, int>> &xs,
              const std::vector<std::pair<int, int>> &ys, const std::vector<int> &rls, const DevicePlan **out) {
@@ -125,6 +132,10 @@ int get_plan(bool diag, const std::vector<VecTriple> &triples, const std::vector
       rec.n2 = ys[t.yi].second;
       for (int d = 0; d < kMaxDl; d++) rec.ri[d] = -1;
       rec.cg_base = (int)bank.size();
+      {
+        const long long U = diag ? rec.n1 : (long long)rec.n1 * rec.n2;
+        rec.log2_u = (U > 0 && (U & (U - 1)) == 0 && U <= (1 << 20)) ? ilog2((int)U) : -1;
+      }
       rec.xoff = xoff[t.xi];
       rec.yoff = yoff[t.yi];
       plan.pairs.push_back(rec);
@@ -155,13 +166,6 @@ int get_plan(bool diag, const std::vector<VecTriple> &triples, const std::vector
   auto ins = g_plans.emplace(key, std::move(plan));
   *out = &ins.first->second;
   return GELIB_HIP_OK;
-}
-
-bool is_pow2(int v) { return v > 0 && (v & (v - 1)) == 0; }
-int ilog2(int v) {
-  int k = 0;
-  while ((1 << k) < v) k++;
-  return k;
 }
 
 struct FastLists {
@@ -219,20 +223,16 @@ int run_bwd(bool diag, const std::vector<VecTriple> &triples, const std::vector<
             const std::vector<std::pair<int, int>> &ys, const std::vector<int> &rls, const FastLists &f,
             long long ncells, int offs_add, bool accumulate, bool want_x, bool want_y, hipStream_t s, int *used) {
   *used = 0;
-  // channel counts must be powers of two, the reduced operand must fit a wave, and every pair must cover the
-  // same number of cells per wave
-  int u_common = -1;
-  bool big = true;
+  // channel counts must be powers of two and the reduced operand must fit a wave
+  int u_min = 1 << 30;
   for (auto &t : triples) {
     const int n1 = xs[t.xi].second, n2 = ys[t.yi].second;
     if (!is_pow2(n1) || !is_pow2(n2)) return GELIB_HIP_OK;
     if (!diag && n2 > kWave) return GELIB_HIP_OK;
-    const int U = diag ? n1 : n1 * n2;
-    if (U < kWave) big = false;
-    if (u_common < 0) u_common = U;
-    else if (u_common != U) u_common = 0;
+    const long long U = diag ? n1 : (long long)n1 * n2;
+    if (U > (1 << 20)) return GELIB_HIP_OK;
+    u_min = std::min<int>(u_min, (int)U);
   }
-  if (!big && u_common <= 0) return GELIB_HIP_OK;
   const DevicePlan *plan = nullptr;
   int rc = get_plan(diag, triples, xs, ys, rls, &plan);
   if (rc) return rc;
@@ -240,7 +240,7 @@ int run_bwd(bool diag, const std::vector<VecTriple> &triples, const std::vector<
   std::memset(&a, 0, sizeof(a));
   for (size_t i = 0; i < f.x.size(); i++) a.x[i] = f.x[i];
   for (size_t i = 0; i < f.y.size(); i++) a.y[i] = f.y[i];
-  for (size_t i = 0; i < f.r.size(); i++) a.g[i] = f.r[i];
+  for (size_t i = 0; i < f.r.size(); i++) a.g[rls[i]] = f.r[i];  // indexed by l
   for (size_t i = 0; i < f.xg.size(); i++) a.xg[i] = f.xg[i];
   for (size_t i = 0; i < f.yg.size(); i++) a.yg[i] = f.yg[i];
   a.pairs = plan->d_pairs;
@@ -258,16 +258,17 @@ int run_bwd(bool diag, const std::vector<VecTriple> &triples, const std::vector<
   a.ysize = plan->ysize;
   for (size_t i = 0; i < xs.size(); i++) a.xrows[i] = 2 * xs[i].first + 1;
   for (size_t i = 0; i < ys.size(); i++) a.yrows[i] = 2 * ys[i].first + 1;
-  a.cells_per_wave = big ? 1 : kWave / u_common;
-  a.log2_u = big ? 6 : ilog2(u_common);
-  const int waves = kBlock / kWave;
-  const size_t lds = sizeof(float) * (size_t)((a.bank_len + 1) & ~1) +
-                     sizeof(float2) * (size_t)waves * a.cells_per_wave * ((size_t)a.xsize + a.ysize);
+  // enough cells per block to give every wave a full run of 64 slots, as far as LDS allows
+  int cpb = std::max(1, kBlock / std::min(kBlock, u_min));
+  while (cpb > 1 && unrolled_bwd_lds_bytes(a.bank_len, a.xsize, a.ysize, cpb) > 64 * 1024) cpb >>= 1;
+  const size_t lds = unrolled_bwd_lds_bytes(a.bank_len, a.xsize, a.ysize, cpb);
   if (lds > 150 * 1024) return GELIB_HIP_OK;
-  const long long cells_per_block = (long long)waves * a.cells_per_wave;
-  const long long nblocks = (ncells + cells_per_block - 1) / cells_per_block;
+  a.cells_per_block = cpb;
+  const long long nblocks = (ncells + cpb - 1) / cpb;
   if (nblocks > 0x7fffffffLL) return GELIB_HIP_ERR_ARG;
-  rc = launch_unrolled_bwd(a, diag, (int)nblocks, lds, s);
+  int lcap = 0;
+  for (auto &t : triples) lcap = std::max(lcap, t.l);
+  rc = launch_unrolled_bwd(a, diag, lcap, (int)nblocks, lds, s);
   if (rc) return rc;
   *used = 1;
   return GELIB_HIP_OK;

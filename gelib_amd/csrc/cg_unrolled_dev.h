@@ -13,7 +13,8 @@ constexpr int kFastOut = 2 * kLT + 1;  // product parts l = 0..2*kLT
 constexpr int kBlock = 256;
 
 struct FwdArgs {
-  FastPart x[kFastIn], y[kFastIn], r[kFastOut];
+  FastPart x[kFastIn], y[kFastIn];  // in list order (ascending l)
+  FastPart r[kFastOut];             // indexed by l itself; absent parts have ptr == nullptr
   const PairRec *pairs;  // device
   const float *bank;     // device, concatenated coefficient tables
   long long ncells;
@@ -53,28 +54,38 @@ __device__ __forceinline__ void static_for(F &&f) {
   static_for_impl(std::make_integer_sequence<int, N>{}, static_cast<F &&>(f));
 }
 
-// Kernel-argument arrays must only be indexed with compile-time constants (a run-time index, or a loop the
-// optimiser unrolls late, makes the compiler keep a copy of the whole argument block in scratch memory); these
-// pick an entry with scalar selects instead.
+// Kernel-argument arrays must only be indexed with compile-time constants: a run-time index (or a chain of
+// selects between entries, which the optimiser folds back into one) makes the compiler keep a copy of the
+// argument block in scratch memory.  These pick an entry by OR-ing together masked copies of every entry, which
+// stays scalar arithmetic on values already loaded from the argument block.
 template <int N>
 __device__ __forceinline__ FastPart pick_part(const FastPart (&arr)[N], int i) {
-  FastPart r = arr[0];
+  unsigned long long ptr = 0, sb = 0;
+  unsigned sm = 0, n = 0;
   static_for<N>([&](auto k) __attribute__((always_inline)) {
-    if (k.value > 0 && i == k.value) r = arr[k.value];
+    const unsigned long long m64 = (i == k.value) ? ~0ull : 0ull;
+    const unsigned m32 = (i == k.value) ? ~0u : 0u;
+    ptr |= m64 & (unsigned long long)arr[k.value].ptr;
+    sb |= m64 & (unsigned long long)arr[k.value].sb;
+    sm |= m32 & (unsigned)arr[k.value].sm;
+    n |= m32 & (unsigned)arr[k.value].n;
   });
+  FastPart r;
+  r.ptr = (float2 *)ptr;
+  r.sb = (long long)sb;
+  r.sm = (int)sm;
+  r.n = (int)n;
   return r;
 }
 template <int N>
 __device__ __forceinline__ int pick_int(const int (&arr)[N], int i) {
-  int r = arr[0];
-  static_for<N>([&](auto k) __attribute__((always_inline)) {
-    if (k.value > 0 && i == k.value) r = arr[k.value];
-  });
-  return r;
+  unsigned r = 0;
+  static_for<N>([&](auto k) __attribute__((always_inline)) { r |= ((i == k.value) ? ~0u : 0u) & (unsigned)arr[k.value]; });
+  return (int)r;
 }
 
 // ti: channels of the first operand handled per thread (1, 2 or 4); must divide every n1.
-int launch_unrolled_fwd(const FwdArgs &a, bool diag, int ti, int nblocks, hipStream_t s);
+int launch_unrolled_fwd(const FwdArgs &a, bool diag, int ti, int lcap, int nblocks, size_t lds_bytes, hipStream_t s);
 // lcap: largest l present in the gradient
 int launch_unrolled_bwd(const BwdArgs &a, bool diag, int lcap, int nblocks, size_t lds_bytes, hipStream_t s);
 

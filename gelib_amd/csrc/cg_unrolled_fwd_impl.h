@@ -1,11 +1,13 @@
 // Forward CG / DiagCG product for l1, l2 <= kLT, all (l1,l2,l) triples of an SO3vec product in one launch.
 //
-// Work split: a block owns one (x part, y part) pair and a run of cells; its 256 threads cover the flattened
-// (cell, slot) space, a slot being one channel pair (i0, j).  Each thread keeps its operands in registers --
-// y[m2, j] and TI values x[m1, i0 + k*n1/TI] -- so one scaled value C*y[m2,j] feeds TI complex FMAs, and the
-// TI results of a row are n1/TI * n2 channels apart: every store instruction of a wave writes one contiguous
-// 512-byte run of the product row.  All loops over l, m and m1 are unrolled at compile time; the coefficient
-// tables of the block's pair sit in LDS and are read at immediate offsets.
+// Work split: a block owns one (x part, y part) pair and a run of cells.  It first copies the two operand parts
+// of its cells into LDS (the only loads from memory it ever waits for); after that its 256 threads sweep the
+// flattened (cell, slot) space, a slot being one channel pair (i0, j).  A thread holds y[m2, j] and TI values
+// x[m1, i0 + k*n1/TI] in registers, so one scaled value C*y[m2,j] feeds TI complex FMAs, and its TI results of a
+// row lie n1/TI * n2 channels apart: every store instruction of a wave writes one contiguous 512-byte run of the
+// product row.  The store stream is never interrupted by a wait on a load: stores and loads share one in-order
+// counter on this hardware, so a load issued behind a burst of stores would not return before they have drained.
+// All loops over l, m and m1 are unrolled at compile time; the coefficients are fetched with scalar loads.
 #pragma once
 
 #include "cg_unrolled_dev.h"
@@ -17,11 +19,18 @@ namespace {
 constexpr int cabs_(int a) { return a < 0 ? -a : a; }
 constexpr int cmin_(int a, int b) { return a < b ? a : b; }
 
+// Coefficients are read through the constant address space: the address is the same for every lane, so the
+// compiler fetches them with scalar loads into SGPRs and they cost neither vector registers nor LDS traffic.
+typedef const __attribute__((address_space(4))) float *CoeffPtr;
+typedef const __attribute__((address_space(4))) PairRec *PairPtr;
+typedef float v2f __attribute__((ext_vector_type(2)));
+typedef __attribute__((address_space(1))) v2f *GlobalOut;  // product rows: global_store, not flat_store
+
 // One (l1,l2,l) triple for one thread: rows m = -L..L of the block, TI channels each.
 template <int L1, int L2, int L, int TI>
 __device__ __forceinline__ void triple_fwd(const float2 (&xv)[TI][2 * L1 + 1], const float2 (&yv)[2 * L2 + 1],
-                                           const float *__restrict__ C, float2 *__restrict__ rp, int sm, int kstride,
-                                           bool accumulate, bool live) {
+                                           CoeffPtr C, GlobalOut rp, int sm, int kstride, bool accumulate,
+                                           bool live) {
 #pragma unroll
   for (int m = -L; m <= L; m++) {
     float2 acc[TI];
@@ -44,69 +53,84 @@ __device__ __forceinline__ void triple_fwd(const float2 (&xv)[TI][2 * L1 + 1], c
       }
     }
     if (live) {
-      float2 *row = rp + (m + L) * sm;
+      GlobalOut row = rp + (m + L) * sm;
 #pragma unroll
       for (int k = 0; k < TI; k++) {
-        float2 v = acc[k];
-        if (accumulate) {
-          const float2 o = row[k * kstride];
-          v.x += o.x;
-          v.y += o.y;
-        }
+        v2f v;
+        v.x = acc[k].x;
+        v.y = acc[k].y;
+        if (accumulate) v += row[k * kstride];
         row[k * kstride] = v;
       }
     }
   }
 }
 
-// The block's view of its pair: operand parts and the product part of each l, picked out of the kernel
-// arguments once per block.
-struct PairParts {
-  FastPart X, Y;
-  FastPart R[kMaxDl];
+// The product parts, indexed by their l (the host fills FwdArgs::r that way), copied out of the kernel arguments
+// once so that the unrolled code can name them with compile-time indices.
+template <int LCAP>
+struct RParts {
+  FastPart R[LCAP + 1];
 };
 
-template <int L1, int L2, int TI, bool DIAG>
-__device__ __forceinline__ void pair_fwd(const PairParts &pp, const PairRec &p, const float *Cs, int offs_add,
-                                         bool accumulate, long long cell, int u, bool live) {
-  const FastPart X = pp.X;
-  const FastPart Y = pp.Y;
+template <int L1, int L2, int LCAP, int TI, bool DIAG>
+__device__ __forceinline__ void pair_fwd(const RParts<LCAP> &rp_all, PairPtr pr, CoeffPtr Cs, const float2 *xs,
+                                         const float2 *ys, int offs_add, bool accumulate, long long cell, int dc,
+                                         int u, bool live) {
+  const __attribute__((address_space(4))) PairRec &p = *pr;
+  const int N1 = p.n1, N2 = p.n2;
   int i0, j;
   if (DIAG) {
     i0 = u;
     j = u;
   } else {
-    i0 = u / p.n2;
-    j = u - i0 * p.n2;
+    i0 = u / N2;
+    j = u - i0 * N2;
   }
-  const int istep = p.n1 / TI;  // the thread's k-th channel of x is i0 + k*istep
-  const float2 *xp = X.ptr + cell * X.sb + i0;
-  const float2 *yp = Y.ptr + cell * Y.sb + j;
+  const int istep = N1 / TI;  // the thread's k-th channel of x is i0 + k*istep
+  const float2 *xp = xs + dc * (2 * L1 + 1) * N1 + i0;
+  const float2 *yp = ys + dc * (2 * L2 + 1) * N2 + j;
   float2 xv[TI][2 * L1 + 1], yv[2 * L2 + 1];
 #pragma unroll
   for (int m1 = 0; m1 <= 2 * L1; m1++)
 #pragma unroll
-    for (int k = 0; k < TI; k++) xv[k][m1] = xp[m1 * X.sm + k * istep];
+    for (int k = 0; k < TI; k++) xv[k][m1] = xp[m1 * N1 + k * istep];
 #pragma unroll
-  for (int m2 = 0; m2 <= 2 * L2; m2++) yv[m2] = yp[m2 * Y.sm];
+  for (int m2 = 0; m2 <= 2 * L2; m2++) yv[m2] = yp[m2 * N2];
 
   constexpr int LMIN = cabs_(L1 - L2);
   constexpr int NL = 2 * cmin_(L1, L2) + 1;
-  const int kstride = DIAG ? 0 : istep * p.n2;
+  const int kstride = DIAG ? 0 : istep * N2;
   static_for<NL>([&](auto dl_c) __attribute__((always_inline)) {
     constexpr int dl = decltype(dl_c)::value;
     constexpr int L = LMIN + dl;
-    if (p.ri[dl] >= 0) {
-      const FastPart R = pp.R[dl];
-      float2 *rp = R.ptr + cell * R.sb + (p.offs[dl] + offs_add + u);
-      triple_fwd<L1, L2, L, TI>(xv, yv, Cs + p.cg[dl], rp, R.sm, kstride, accumulate, live);
+    if constexpr (L <= LCAP) {
+      if (p.ri[dl] >= 0) {
+        const FastPart R = rp_all.R[L];
+        GlobalOut rp = (GlobalOut)R.ptr + cell * R.sb + (p.offs[dl] + offs_add + u);
+        triple_fwd<L1, L2, L, TI>(xv, yv, Cs + p.cg[dl], rp, R.sm, kstride, accumulate, live);
+      }
     }
   });
 }
 
-template <bool DIAG, int TI>
+// memory -> LDS copy of one operand part for the block's cells; rows become contiguous (row stride n)
+__device__ __forceinline__ void stage_part(float2 *dst, const FastPart P, int rows, long long cell0, int ncell) {
+  const int per_cell = rows * P.n;
+  const int total = per_cell * ncell;
+  for (int e = threadIdx.x; e < total; e += kBlock) {
+    const int c = e / per_cell;
+    const int r = e - c * per_cell;
+    const int m = r / P.n;
+    const int ch = r - m * P.n;
+    const v2f t = ((const __attribute__((address_space(1))) v2f *)P.ptr)[(cell0 + c) * P.sb + m * P.sm + ch];
+    dst[e] = make_float2(t.x, t.y);
+  }
+}
+
+template <int LCAP, bool DIAG, int TI>
 __global__ void __launch_bounds__(kBlock) unrolled_fwd_kernel(const FwdArgs a) {
-  __shared__ float Cs[kMaxDl * (2 * kLT + 1) * (2 * kLT + 1)];
+  extern __shared__ float2 lds_ops[];
   int pidx = 0, first = 0;
   static_for<kMaxPairs>([&](auto k) __attribute__((always_inline)) {
     if (k.value > 0 && k.value < a.npairs && (int)blockIdx.x >= a.first_block[k.value]) {
@@ -114,23 +138,27 @@ __global__ void __launch_bounds__(kBlock) unrolled_fwd_kernel(const FwdArgs a) {
       first = a.first_block[k.value];
     }
   });
-  const PairRec &p = a.pairs[pidx];
-  for (int i = threadIdx.x; i < p.cg_len; i += kBlock) Cs[i] = a.bank[p.cg_base + i];
-  __syncthreads();
-
-  PairParts pp;
-  pp.X = pick_part(a.x, p.xi);
-  pp.Y = pick_part(a.y, p.yi);
-  static_for<kMaxDl>([&](auto d) __attribute__((always_inline)) { pp.R[d.value] = pick_part(a.r, p.ri[d.value]); });
-  const int offs_add = a.offs_add;
-  const bool accumulate = a.accumulate != 0;
+  const PairPtr p = (PairPtr)a.pairs + pidx;
   const int cpb = pick_int(a.cpb, pidx);
   const long long cell0 = (long long)((int)blockIdx.x - first) * cpb;
   const long long left = a.ncells - cell0;
   const int ncell = left < cpb ? (int)left : cpb;
-  const int U = DIAG ? p.n1 : (p.n1 / TI) * p.n2;
+  const int l1 = p->l1, l2 = p->l2, n1 = p->n1, n2 = p->n2;
+
+  float2 *xs = lds_ops;
+  float2 *ys = xs + cpb * (2 * l1 + 1) * n1;
+  stage_part(xs, pick_part(a.x, p->xi), 2 * l1 + 1, cell0, ncell);
+  stage_part(ys, pick_part(a.y, p->yi), 2 * l2 + 1, cell0, ncell);
+  RParts<LCAP> rp_all;
+  static_for<LCAP + 1>([&](auto l) __attribute__((always_inline)) { rp_all.R[l.value] = a.r[l.value]; });
+  const int offs_add = a.offs_add;
+  const bool accumulate = a.accumulate != 0;
+  __syncthreads();
+
+  const int U = DIAG ? n1 : (n1 / TI) * n2;
   const int slots = ncell * U;
-  const int code = p.l1 * (kLT + 1) + p.l2;
+  const CoeffPtr C = (CoeffPtr)(a.bank + p->cg_base);
+  const int code = l1 * (kLT + 1) + l2;
   for (int w0 = 0; w0 < slots; w0 += kBlock) {
     const int w = w0 + threadIdx.x;
     const bool live = w < slots;
@@ -140,7 +168,7 @@ __global__ void __launch_bounds__(kBlock) unrolled_fwd_kernel(const FwdArgs a) {
     const long long cell = cell0 + dc;
     switch (code) {
 #define GELIB_CASE(A, B) \
-  case A * (kLT + 1) + B: pair_fwd<A, B, TI, DIAG>(pp, p, Cs, offs_add, accumulate, cell, u, live); break;
+  case A * (kLT + 1) + B: pair_fwd<A, B, LCAP, TI, DIAG>(rp_all, p, C, xs, ys, offs_add, accumulate, cell, dc, u, live); break;
 #define GELIB_ROW(A) GELIB_CASE(A, 0) GELIB_CASE(A, 1) GELIB_CASE(A, 2) GELIB_CASE(A, 3) GELIB_CASE(A, 4)
       GELIB_ROW(0) GELIB_ROW(1) GELIB_ROW(2) GELIB_ROW(3) GELIB_ROW(4)
 #undef GELIB_ROW
@@ -150,10 +178,10 @@ __global__ void __launch_bounds__(kBlock) unrolled_fwd_kernel(const FwdArgs a) {
   }
 }
 
-template <bool DIAG, int TI>
-int launch_fwd_variant(const FwdArgs &a, int nblocks, hipStream_t s) {
+template <int LCAP, bool DIAG, int TI>
+int launch_fwd_variant(const FwdArgs &a, int nblocks, size_t lds_bytes, hipStream_t s) {
   static_assert(kLT == 4, "the case table above lists l1, l2 = 0..4");
-  hipLaunchKernelGGL((unrolled_fwd_kernel<DIAG, TI>), dim3(nblocks), dim3(kBlock), 0, s, a);
+  hipLaunchKernelGGL((unrolled_fwd_kernel<LCAP, DIAG, TI>), dim3(nblocks), dim3(kBlock), lds_bytes, s, a);
   GELIB_HIP_TRY(hipGetLastError());
   return GELIB_HIP_OK;
 }

@@ -13,6 +13,7 @@ namespace gelib_hip {
 namespace {
 
 int g_fwd_block_bytes = 384 * 1024;  // product bytes one forward block aims to write
+int g_fwd_lds_bytes = 16 * 1024;     // LDS one forward block may use for its staged operands
 int g_fwd_ti = 0;                    // 0 = widest tile that divides every n1, else force 1 / 2 / 4
 int g_bwd_enable = 1;
 int g_fwd_enable = 1;
@@ -174,7 +175,13 @@ struct FastLists {
 
 int run_fwd(bool diag, const std::vector<VecTriple> &triples, const std::vector<std::pair<int, int>> &xs,
             const std::vector<std::pair<int, int>> &ys, const std::vector<int> &rls, const FastLists &f,
-            long long ncells, int offs_add, bool accumulate, hipStream_t s) {
+            long long ncells, int offs_add, bool accumulate, hipStream_t s, int *used) {
+  *used = 0;
+  // one cell's two operand parts must fit the LDS staging area
+  for (auto &t : triples) {
+    const long long op_bytes = 8LL * ((2 * t.l1 + 1) * (long long)xs[t.xi].second + (2 * t.l2 + 1) * (long long)ys[t.yi].second);
+    if (op_bytes > g_fwd_lds_bytes) return GELIB_HIP_OK;
+  }
   const DevicePlan *plan = nullptr;
   int rc = get_plan(diag, triples, xs, ys, rls, &plan);
   if (rc) return rc;
@@ -182,7 +189,7 @@ int run_fwd(bool diag, const std::vector<VecTriple> &triples, const std::vector<
   std::memset(&a, 0, sizeof(a));
   for (size_t i = 0; i < f.x.size(); i++) a.x[i] = f.x[i];
   for (size_t i = 0; i < f.y.size(); i++) a.y[i] = f.y[i];
-  for (size_t i = 0; i < f.r.size(); i++) a.r[i] = f.r[i];
+  for (size_t i = 0; i < f.r.size(); i++) a.r[rls[i]] = f.r[i];  // indexed by l
   a.pairs = plan->d_pairs;
   a.bank = plan->d_bank;
   a.ncells = ncells;
@@ -198,6 +205,9 @@ int run_fwd(bool diag, const std::vector<VecTriple> &triples, const std::vector<
     if (g_fwd_ti == 1 || g_fwd_ti == 2 || g_fwd_ti == 4) ti = std::min(ti, g_fwd_ti);
   }
   long long nblocks = 0;
+  size_t lds_bytes = 0;
+  int lcap = 0;
+  for (auto &t : triples) lcap = std::max(lcap, t.l);
   for (int i = 0; i < a.npairs; i++) {
     const PairRec &p = plan->pairs[i];
     long long rows = 0;
@@ -207,16 +217,21 @@ int run_fwd(bool diag, const std::vector<VecTriple> &triples, const std::vector<
     const long long bytes_per_cell = rows * nout * 8;
     const long long U = diag ? p.n1 : (long long)(p.n1 / ti) * p.n2;
     long long cpb = std::max<long long>(1, g_fwd_block_bytes / std::max<long long>(1, bytes_per_cell));
-    cpb = std::max(cpb, (kBlock + U - 1) / U);  // at least one full pass of the block
+    const long long op_bytes = 8LL * ((2 * p.l1 + 1) * (long long)p.n1 + (2 * p.l2 + 1) * (long long)p.n2);
+    cpb = std::min(cpb, std::max<long long>(1, g_fwd_lds_bytes / op_bytes));
     cpb = std::min<long long>(cpb, std::max<long long>(1, (1LL << 28) / std::max<long long>(1, U)));
     cpb = std::min(cpb, ncells);
     a.cpb[i] = (int)cpb;
+    lds_bytes = std::max(lds_bytes, (size_t)(cpb * op_bytes));
     a.first_block[i] = (int)nblocks;
     nblocks += (ncells + cpb - 1) / cpb;
     if (nblocks > 0x7fffffffLL) return GELIB_HIP_ERR_ARG;
   }
   a.first_block[a.npairs] = (int)nblocks;
-  return launch_unrolled_fwd(a, diag, ti, (int)nblocks, s);
+  rc = launch_unrolled_fwd(a, diag, ti, lcap, (int)nblocks, lds_bytes, s);
+  if (rc) return rc;
+  *used = 1;
+  return GELIB_HIP_OK;
 }
 
 int run_bwd(bool diag, const std::vector<VecTriple> &triples, const std::vector<std::pair<int, int>> &xs,
@@ -293,10 +308,7 @@ int unrolled_part(int kind, const PartOp &op, bool accumulate, hipStream_t s, in
   std::vector<std::pair<int, int>> xs = {{op.l1, op.n1}}, ys = {{op.l2, op.n2}};
   std::vector<int> rls = {op.l};
   if (kind == 0) {
-    int rc = run_fwd(op.diag, triples, xs, ys, rls, f, ncells, op.offs, accumulate, s);
-    if (rc) return rc;
-    *used = 1;
-    return GELIB_HIP_OK;
+    return run_fwd(op.diag, triples, xs, ys, rls, f, ncells, op.offs, accumulate, s, used);
   }
   if (kind == 1) f.xg = f.x;  // destination
   if (kind == 2) f.yg = f.y;
@@ -338,10 +350,7 @@ int unrolled_vec_fwd(const VecPlan &plan, const std::vector<const gelib_part_des
   std::vector<int> rls;
   for (auto &v : rs) rls.push_back(v.first);
   const long long ncells = plan.E[0] * plan.E[1] * plan.E[2];
-  int rc = run_fwd(plan.diag, plan.triples, xs, ys, rls, f, ncells, 0, accumulate, s);
-  if (rc) return rc;
-  *used = 1;
-  return GELIB_HIP_OK;
+  return run_fwd(plan.diag, plan.triples, xs, ys, rls, f, ncells, 0, accumulate, s, used);
 }
 
 int unrolled_vec_bwd(const VecPlan &plan, const std::vector<const gelib_part_desc *> &g,
@@ -372,6 +381,11 @@ int unrolled_set_option(const char *name, int value) {
   if (!std::strcmp(name, "fwd_block_bytes")) {
     if (value < 1024) return GELIB_HIP_ERR_ARG;
     g_fwd_block_bytes = value;
+    return GELIB_HIP_OK;
+  }
+  if (!std::strcmp(name, "fwd_lds_bytes")) {
+    if (value < 1024 || value > 60 * 1024) return GELIB_HIP_ERR_ARG;
+    g_fwd_lds_bytes = value;
     return GELIB_HIP_OK;
   }
   if (!std::strcmp(name, "fwd_tile")) {

@@ -17,6 +17,7 @@ SYMBOLS = [
     "gelib_hip_so3part_diagcg_fwd", "gelib_hip_so3part_diagcg_back0", "gelib_hip_so3part_diagcg_back1",
     "gelib_hip_so3vec_cg_fwd", "gelib_hip_so3vec_cg_bwd", "gelib_hip_so3vec_diagcg_fwd",
     "gelib_hip_so3vec_diagcg_bwd", "gelib_hip_set_option", "gelib_hip_last_path",
+    "gelib_hip_malloc", "gelib_hip_free", "gelib_hip_memcpy", "gelib_hip_memset", "gelib_hip_synchronize",
 ]
 
 

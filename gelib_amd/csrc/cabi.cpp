@@ -448,6 +448,36 @@ int gelib_hip_so3vec_diagcg_bwd(const gelib_part_desc *xg, const gelib_part_desc
   return vec_bwd_entry(true, xg, yg, ng, g, nx, x, ny, y, accumulate, stream);
 }
 
+int gelib_hip_malloc(void **ptr, uint64_t bytes) {
+  if (!ptr) return GELIB_HIP_ERR_NULL;
+  *ptr = nullptr;
+  if (bytes == 0) return GELIB_HIP_OK;
+  GELIB_HIP_TRY(hipMalloc(ptr, bytes));
+  return GELIB_HIP_OK;
+}
+int gelib_hip_free(void *ptr) {
+  if (ptr) GELIB_HIP_TRY(hipFree(ptr));
+  return GELIB_HIP_OK;
+}
+int gelib_hip_memcpy(void *dst, const void *src, uint64_t bytes, int kind) {
+  if (bytes == 0) return GELIB_HIP_OK;
+  if (!dst || !src) return GELIB_HIP_ERR_NULL;
+  const hipMemcpyKind k = kind == 0 ? hipMemcpyHostToDevice : (kind == 1 ? hipMemcpyDeviceToHost : hipMemcpyDeviceToDevice);
+  if (kind < 0 || kind > 2) return GELIB_HIP_ERR_ARG;
+  GELIB_HIP_TRY(hipMemcpy(dst, src, bytes, k));
+  return GELIB_HIP_OK;
+}
+int gelib_hip_memset(void *ptr, int value, uint64_t bytes) {
+  if (bytes == 0) return GELIB_HIP_OK;
+  if (!ptr) return GELIB_HIP_ERR_NULL;
+  GELIB_HIP_TRY(hipMemset(ptr, value, bytes));
+  return GELIB_HIP_OK;
+}
+int gelib_hip_synchronize(void) {
+  GELIB_HIP_TRY(hipDeviceSynchronize());
+  return GELIB_HIP_OK;
+}
+
 int gelib_hip_set_option(const char *name, int value) {
   if (!name) return GELIB_HIP_ERR_NULL;
   if (!std::strcmp(name, "force_generic")) {

@@ -124,6 +124,18 @@ int gelib_hip_so3vec_diagcg_bwd(const gelib_part_desc *xg, const gelib_part_desc
                                 const gelib_part_desc *y, int accumulate, void *stream);
 
 /*
+ * Device memory helpers for host code that does not include the HIP headers itself (the C++ mirror of the
+ * reference's classes uses them where the reference relies on cnine's device transport, e.g. the
+ * TensorView(x, dev) constructor used at SO3/SO3part.hpp:182-183).  kind: 0 host->device, 1 device->host,
+ * 2 device->device.  All synchronous.
+ */
+int gelib_hip_malloc(void **ptr, uint64_t bytes);
+int gelib_hip_free(void *ptr);
+int gelib_hip_memcpy(void *dst, const void *src, uint64_t bytes, int kind);
+int gelib_hip_memset(void *ptr, int value, uint64_t bytes);
+int gelib_hip_synchronize(void);
+
+/*
  * Tuning / introspection (no counterpart in the reference).
  * gelib_hip_set_option("force_generic", 1) routes every call through the shape-agnostic kernels;
  * gelib_hip_last_path() tells which kernel family the last call of this thread used

@@ -1,0 +1,140 @@
+"""SO3vec: an SO(3)-covariant vector, a dict {l: (b, 2l+1, n_l) complex64 tensor} -- the class and autograd functions
+of python/src/gelib/SO3vec.py:22-309 for the CG product path.  The products are ONE fused launch per call: the
+forward writes into uninitialised parts and the backward computes both gradients from a single pass over g."""
+import torch
+
+from gelib_amd.gelib_common import backend, common_batch
+from gelib_amd.SO3part import SO3part
+
+
+class SO3vec:
+
+    def __init__(self, *args):
+        self.parts = {}
+        for x in args:
+            assert isinstance(x, torch.Tensor)
+            p = SO3part(x)
+            self.parts[p.getl()] = x
+
+    @classmethod
+    def zeros(cls, b, tau, device='cpu'):
+        R = SO3vec()
+        for l, n in tau.items():
+            R.parts[l] = SO3part.zeros(b, l, n, device=device)
+        return R
+
+    @classmethod
+    def randn(cls, b, tau, device='cpu'):
+        R = SO3vec()
+        for l, n in tau.items():
+            R.parts[l] = SO3part.randn(b, l, n, device=device)
+        return R
+
+    @classmethod
+    def zeros_like(cls, x):
+        R = SO3vec()
+        for l, p in x.parts.items():
+            R.parts[l] = SO3part(torch.zeros_like(p))
+        return R
+
+    @classmethod
+    def randn_like(cls, x):
+        R = SO3vec()
+        for l, p in x.parts.items():
+            R.parts[l] = SO3part.randn_like(p)
+        return R
+
+    def backend(self):
+        return backend().SO3vec.view(self.parts)
+
+    def getb(self):
+        return self.parts[min(self.parts)].size(0)
+
+    def tau(self):
+        return {l: p.size(-1) for l, p in self.parts.items()}
+
+    get_type = tau
+
+    def requires_grad_(self):
+        for p in self.parts.values():
+            p.requires_grad_()
+
+    def get_grad(self):
+        return SO3vec(*[p.grad for p in self.parts.values()])
+
+    def apply(self, R):
+        r = SO3vec()
+        for l, p in self.parts.items():
+            r.parts[l] = SO3part(p).apply(R)
+        return r
+
+    def odot(self, y):
+        assert list(self.parts.keys()) == list(y.parts.keys())
+        return sum(SO3part(self.parts[l]).odot(y.parts[l]) for l in self.parts.keys())
+
+    def __add__(self, y):
+        assert list(self.parts.keys()) == list(y.parts.keys())
+        return SO3vec(*[self.parts[l] + y.parts[l] for l in self.parts.keys()])
+
+    def CGproduct(self, y, maxl=-1):
+        xparts = list(self.parts.values())
+        yparts = list(y.parts.values())
+        return SO3vec(*SO3vec_CGproductFn.apply(len(xparts), len(yparts), maxl, *(xparts + yparts)))
+
+    def DiagCGproduct(self, y, maxl=-1):
+        xparts = list(self.parts.values())
+        yparts = list(y.parts.values())
+        return SO3vec(*SO3vec_DiagCGproductFn.apply(len(xparts), len(yparts), maxl, *(xparts + yparts)))
+
+    def __repr__(self):
+        return "<SO3vec of type %s [b=%d]>" % (self.tau(), self.getb())
+
+
+def _product_fn(diag):
+    gb_type = "DiagCGproduct" if diag else "CGproduct"
+
+    class Fn(torch.autograd.Function):
+
+        @staticmethod
+        def forward(ctx, k1, k2, maxl, *args):
+            gb = backend()
+            ctx.k1, ctx.k2 = k1, k2
+            ctx.save_for_backward(*args)
+            x = gb.SO3vec.view(list(args[0:k1]))
+            y = gb.SO3vec.view(list(args[k1:k1 + k2]))
+            b = common_batch(args[0], args[k1])
+            tau = getattr(x.get_tau(), gb_type)(y.get_tau(), maxl)
+            # uninitialised outputs: every channel of every part is written exactly once by the fused launch
+            rparts = [torch.empty([b, 2 * l + 1, n], dtype=torch.complex64, device=args[0].device)
+                      for l, n in tau.get_parts().items()]
+            r = gb.SO3vec.view(rparts)
+            (r.setDiagCGproduct if diag else r.setCGproduct)(x, y)
+            return tuple(SO3part(t) for t in rparts)
+
+        @staticmethod
+        def backward(ctx, *gargs):
+            gb = backend()
+            k1, k2 = ctx.k1, ctx.k2
+            saved = ctx.saved_tensors
+            grads = [torch.empty_like(t) for t in saved]
+            x = gb.SO3vec.view(list(saved[0:k1]))
+            y = gb.SO3vec.view(list(saved[k1:k1 + k2]))
+            g = gb.SO3vec.view([t.contiguous() for t in gargs])
+            xg = gb.SO3vec.view(grads[0:k1])
+            yg = gb.SO3vec.view(grads[k1:k1 + k2])
+            if any(t.size(0) != gargs[0].size(0) for t in saved):
+                # a batch-broadcast operand: its gradient is a sum over the batch, done by the accumulate path
+                for t in grads:
+                    t.zero_()
+                getattr(xg, "add%s_back0" % gb_type)(g, y)
+                getattr(yg, "add%s_back1" % gb_type)(g, x)
+            else:
+                getattr(gb.SO3vec, "set%s_back" % gb_type)(xg, yg, g, x, y)
+            return tuple([None, None, None] + grads)
+
+    Fn.__name__ = "SO3vec_%sFn" % gb_type
+    return Fn
+
+
+SO3vec_CGproductFn = _product_fn(False)
+SO3vec_DiagCGproductFn = _product_fn(True)

@@ -38,6 +38,21 @@ class GtypeBase {};
 class GpartBase {};
 class GvecBase {};
 
+// HIP stream the products are queued on (per thread; nullptr = the default stream).  The PyTorch binding sets it
+// to torch's current stream before every call, where the reference creates a private stream per call
+// (CUDA_STREAM, SO3/SO3part.hpp:260).
+inline void *&gelib_stream() {
+  thread_local void *s = nullptr;
+  return s;
+}
+
+// 1 = the reference's "+=" into the destination (default); 0 = overwrite, for callers that hand in uninitialised
+// outputs instead of zero-filled ones (SO3vec level only).
+inline int &accumulate_mode() {
+  thread_local int a = 1;
+  return a;
+}
+
 inline void gelib_check(const int rc) {
   if (rc == 0) return;
   std::string msg = gelib_hip_strerror(rc);
@@ -262,27 +277,27 @@ class SO3part : public cnine::BatchedTensor<std::complex<TYPE>>, public GpartBas
   // ---- device seams (SO3/SO3part.hpp:259-269, 324-334): destination first, as in the reference ----
   static void add_CGproduct_dev(const SO3part &r, SO3part x, SO3part y, const int offs = 0) {
     auto R = r.descriptor(), X = x.descriptor(), Y = y.descriptor();
-    gelib_check(gelib_hip_so3part_cg_fwd(&R, &X, &Y, offs, 1, nullptr));
+    gelib_check(gelib_hip_so3part_cg_fwd(&R, &X, &Y, offs, 1, gelib_stream()));
   }
   static void add_CGproduct_back0_dev(const SO3part &xg, SO3part g, SO3part y, const int offs = 0) {
     auto XG = xg.descriptor(), G = g.descriptor(), Y = y.descriptor();
-    gelib_check(gelib_hip_so3part_cg_back0(&XG, &G, &Y, offs, 1, nullptr));
+    gelib_check(gelib_hip_so3part_cg_back0(&XG, &G, &Y, offs, 1, gelib_stream()));
   }
   static void add_CGproduct_back1_dev(const SO3part &yg, SO3part g, SO3part x, const int offs = 0) {
     auto YG = yg.descriptor(), G = g.descriptor(), X = x.descriptor();
-    gelib_check(gelib_hip_so3part_cg_back1(&YG, &G, &X, offs, 1, nullptr));
+    gelib_check(gelib_hip_so3part_cg_back1(&YG, &G, &X, offs, 1, gelib_stream()));
   }
   static void add_DiagCGproduct_dev(const SO3part &r, SO3part x, SO3part y, const int offs = 0) {
     auto R = r.descriptor(), X = x.descriptor(), Y = y.descriptor();
-    gelib_check(gelib_hip_so3part_diagcg_fwd(&R, &X, &Y, offs, 1, nullptr));
+    gelib_check(gelib_hip_so3part_diagcg_fwd(&R, &X, &Y, offs, 1, gelib_stream()));
   }
   static void add_DiagCGproduct_back0_dev(const SO3part &xg, SO3part g, SO3part y, const int offs = 0) {
     auto XG = xg.descriptor(), G = g.descriptor(), Y = y.descriptor();
-    gelib_check(gelib_hip_so3part_diagcg_back0(&XG, &G, &Y, offs, 1, nullptr));
+    gelib_check(gelib_hip_so3part_diagcg_back0(&XG, &G, &Y, offs, 1, gelib_stream()));
   }
   static void add_DiagCGproduct_back1_dev(const SO3part &yg, SO3part g, SO3part x, const int offs = 0) {
     auto YG = yg.descriptor(), G = g.descriptor(), X = x.descriptor();
-    gelib_check(gelib_hip_so3part_diagcg_back1(&YG, &G, &X, offs, 1, nullptr));
+    gelib_check(gelib_hip_so3part_diagcg_back1(&YG, &G, &X, offs, 1, gelib_stream()));
   }
 
   std::string classname() const { return "GElib::SO3part"; }
@@ -315,7 +330,7 @@ inline void skip_on(const int rc) {
   void NAME(GPART dest, GPART a, GPART b, const int offs = 0) {                                   \
     detail::check_devices(dest, a, b);                                                            \
     auto D = dest.descriptor(), A = a.descriptor(), B = b.descriptor();                           \
-    detail::skip_on(ENTRY(&D, &A, &B, offs, 1, nullptr));                                         \
+    detail::skip_on(ENTRY(&D, &A, &B, offs, 1, gelib_stream()));                                         \
   }
 GELIB_PART_DISPATCH(Gpart_add_CGproduct, gelib_hip_so3part_cg_fwd)              // (r, x, y, offs)
 GELIB_PART_DISPATCH(Gpart_add_CGproduct_back0, gelib_hip_so3part_cg_back0)      // (xg, g, y, offs)
@@ -432,7 +447,7 @@ class SO3vec : public GvecBase {
     on_gpu(*this), on_gpu(x), on_gpu(y);
     auto R = descs(*this), X = descs(x), Y = descs(y);
     auto fn = diag ? gelib_hip_so3vec_diagcg_fwd : gelib_hip_so3vec_cg_fwd;
-    detail::skip_on(fn((int)R.size(), R.data(), (int)X.size(), X.data(), (int)Y.size(), Y.data(), 1, nullptr));
+    detail::skip_on(fn((int)R.size(), R.data(), (int)X.size(), X.data(), (int)Y.size(), Y.data(), accumulate_mode(), gelib_stream()));
   }
   static void bwd(const bool diag, const SO3vec *xg, const SO3vec *yg, const SO3vec &g, const SO3vec &x, const SO3vec &y) {
     on_gpu(g), on_gpu(x), on_gpu(y);
@@ -442,7 +457,7 @@ class SO3vec : public GvecBase {
     auto G = descs(g), X = descs(x), Y = descs(y);
     auto fn = diag ? gelib_hip_so3vec_diagcg_bwd : gelib_hip_so3vec_cg_bwd;
     detail::skip_on(fn(xg ? XG.data() : nullptr, yg ? YG.data() : nullptr, (int)G.size(), G.data(), (int)X.size(), X.data(),
-                       (int)Y.size(), Y.data(), 1, nullptr));
+                       (int)Y.size(), Y.data(), accumulate_mode(), gelib_stream()));
   }
 };
 

@@ -1,0 +1,156 @@
+"""The Python surface (gelib_amd.SO3part / SO3vec / CGproduct / DiagCGproduct with autograd) on the GPU: the
+identities of the reference's own CI suite (python/tests/ci_tests/test_SO3part.py, test_SO3vec.py) --
+equivariance under a random rotation and exact bilinearity of the gradients -- plus agreement with the CPU oracle."""
+import numpy as np
+import pytest
+
+from oracle import cg_oracle as ora
+from tests import gpu_util as U
+
+pytestmark = pytest.mark.gpu
+
+torch = pytest.importorskip("torch")
+
+
+@pytest.fixture(scope="module")
+def G():
+    assert torch.cuda.is_available()
+    import gelib_amd
+    from gelib_amd import gelib_base  # noqa: F401  (fails loudly if the extension was not built)
+    return gelib_amd
+
+
+def part_part_backprop(G, b, l, n, fn, arg0, bx=None):
+    x = G.SO3part.randn(bx or b, l, n, device="cuda")
+    y = G.SO3part.randn(b, l, n, device="cuda")
+    x.requires_grad_()
+    y.requires_grad_()
+    z = fn(x, y, arg0)
+    test_vec = G.SO3part.randn_like(z)
+    loss = z.odot(test_vec)
+    loss.backward(torch.tensor(1.0, device="cuda"))
+    xeps = G.SO3part.randn_like(x)
+    xloss = fn(x + xeps, y, arg0).odot(test_vec)
+    assert torch.allclose(xloss - loss, xeps.odot(x.grad), rtol=1e-3, atol=1e-3)
+    yeps = G.SO3part.randn_like(y)
+    yloss = fn(x, y + yeps, arg0).odot(test_vec)
+    assert torch.allclose(yloss - loss, yeps.odot(y.grad), rtol=1e-3, atol=1e-3)
+
+
+@pytest.mark.parametrize("b", [1, 2])
+@pytest.mark.parametrize("l", [1, 2, 4])
+@pytest.mark.parametrize("n", [1, 2, 4, 8])
+@pytest.mark.parametrize("diag", [False, True])
+def test_part_equivariance(G, b, l, n, diag):
+    fn = G.DiagCGproduct if diag else G.CGproduct
+    x = G.SO3part.randn(b, l, n, device="cuda")
+    y = G.SO3part.randn(b, l, n, device="cuda")
+    z = fn(x, y, l)
+    R = G.SO3element.random()
+    zr = fn(x.apply(R), y.apply(R), l)
+    assert torch.allclose(z.apply(R), zr, rtol=1e-3, atol=1e-4)
+
+
+@pytest.mark.parametrize("b", [1, 2])
+@pytest.mark.parametrize("l", [1, 2, 4])
+@pytest.mark.parametrize("n", [1, 4, 8])
+@pytest.mark.parametrize("diag", [False, True])
+def test_part_backprop(G, b, l, n, diag):
+    part_part_backprop(G, b, l, n, G.DiagCGproduct if diag else G.CGproduct, l)
+
+
+@pytest.mark.parametrize("b", [2, 5])
+@pytest.mark.parametrize("l", [2, 4])
+def test_part_backprop_bcast(G, b, l):
+    part_part_backprop(G, b, l, 4, G.CGproduct, l, bx=1)
+
+
+def test_part_matches_oracle(G):
+    x = G.SO3part.randn(4, 2, 8, device="cuda")
+    y = G.SO3part.randn(4, 3, 8, device="cuda")
+    z = G.CGproduct(x, y, 4)
+    assert isinstance(z, G.SO3part) and z.shape == (4, 9, 64) and z.dtype == torch.complex64
+    assert U.gate_excess(U.host(z), ora.cg_fwd(U.host(x), U.host(y), 4)) <= 1.0
+    zd = G.DiagCGproduct(x, x, 3)
+    assert U.gate_excess(U.host(zd), ora.cg_fwd(U.host(x), U.host(x), 3, diag=True)) <= 1.0
+
+
+@pytest.mark.parametrize("maxl", [2, 4])
+@pytest.mark.parametrize("b", [1, 3])
+@pytest.mark.parametrize("nc", [1, 4])
+@pytest.mark.parametrize("diag", [False, True])
+def test_vec_equivariance(G, b, nc, maxl, diag):
+    fn = G.DiagCGproduct if diag else G.CGproduct
+    tau = {l: nc for l in range(maxl + 1)}
+    x = G.SO3vec.randn(b, tau, device="cuda")
+    y = G.SO3vec.randn(b, tau, device="cuda")
+    R = G.SO3element.random()
+    z = fn(x, y, maxl=maxl)
+    zr = fn(x.apply(R), y.apply(R), maxl=maxl)
+    rz = z.apply(R)
+    for i in range(maxl + 1):
+        assert torch.allclose(rz.parts[i], zr.parts[i], rtol=1e-3, atol=1e-4)
+
+
+@pytest.mark.parametrize("nc", [1, 4])
+@pytest.mark.parametrize("maxl", [2, 4])
+@pytest.mark.parametrize("b", [1, 3])
+@pytest.mark.parametrize("diag", [False, True])
+@pytest.mark.parametrize("bcast", [False, True])
+def test_vec_backprop(G, b, nc, maxl, diag, bcast):
+    fn = G.DiagCGproduct if diag else G.CGproduct
+    tau = {l: nc for l in range(maxl + 1)}
+    x = G.SO3vec.randn(1 if bcast else b, tau, device="cuda")
+    y = G.SO3vec.randn(b, tau, device="cuda")
+    x.requires_grad_()
+    y.requires_grad_()
+    z = fn(x, y)
+    test_vec = G.SO3vec.randn_like(z)
+    loss = z.odot(test_vec)
+    loss.backward(torch.tensor(1.0, device="cuda"))
+    xgrad, ygrad = x.get_grad(), y.get_grad()
+    xeps = G.SO3vec.randn_like(x)
+    xloss = fn(x + xeps, y).odot(test_vec)
+    assert torch.allclose(xloss - loss, xeps.odot(xgrad), rtol=1e-3, atol=1e-3)
+    yeps = G.SO3vec.randn_like(y)
+    yloss = fn(x, y + yeps).odot(test_vec)
+    assert torch.allclose(yloss - loss, yeps.odot(ygrad), rtol=1e-3, atol=1e-3)
+
+
+def test_vec_matches_oracle_and_uses_fused_kernels(G):
+    from gelib_amd import cabi
+    tau = {l: 16 for l in range(5)}
+    x = G.SO3vec.randn(7, tau, device="cuda")
+    y = G.SO3vec.randn(7, tau, device="cuda")
+    x.requires_grad_()
+    y.requires_grad_()
+    z = G.CGproduct(x, y, maxl=4)
+    assert cabi.last_path() == 2
+    assert {l: p.size(-1) for l, p in z.parts.items()} == {0: 1280, 1: 3072, 2: 4096, 3: 4352, 4: 3840}
+    hx = [U.host(p) for p in x.parts.values()]
+    hy = [U.host(p) for p in y.parts.values()]
+    want = ora.vec_fwd(hx, hy, 4)
+    for a, b in zip(z.parts.values(), want):
+        assert U.gate_excess(U.host(a), b) <= 1.0
+    g = [torch.randn_like(p) for p in z.parts.values()]
+    torch.autograd.backward(list(z.parts.values()), g)
+    assert cabi.last_path() == 2
+    hg = [U.host(t) for t in g]
+    wxg, wyg = ora.vec_bwd(hg, hx, hy)
+    x64, y64, g64 = ([a.astype(np.complex128) for a in L] for L in (hx, hy, hg))
+    exg, eyg = ora.vec_bwd(g64, x64, y64)
+    for p, b, c in zip(list(x.parts.values()) + list(y.parts.values()), wxg + wyg, exg + eyg):
+        U.assert_parity(U.host(p.grad), b, c, "vec grad", slack=4.0)
+
+
+def test_errors_are_exceptions(G):
+    x = G.SO3part.randn(2, 1, 4)          # host tensor
+    with pytest.raises(RuntimeError):
+        G.CGproduct(x, x, 1)
+    xc = G.SO3part.randn(2, 1, 4, device="cuda")
+    with pytest.raises(RuntimeError):
+        G.CGproduct(xc, xc, 3)            # l outside the triangle
+    with pytest.raises((RuntimeError, AssertionError)):
+        G.DiagCGproduct(xc, G.SO3part.randn(2, 1, 5, device="cuda"), 1)
+    with pytest.raises((RuntimeError, AssertionError)):
+        G.CGproduct(G.SO3part.randn(3, 1, 4, device="cuda"), xc, 1)

@@ -57,9 +57,9 @@ def run_vec(cabi, B, tx, ty, maxl, diag, seed, force_generic):
     for a, b, c in zip(drs, r32, r64):
         U.assert_parity(U.host(a), b, c, "fwd " + tag)
     for a, b, c in zip(dxg, xg32, xg64):
-        U.assert_parity(U.host(a), b, c, "xg " + tag, slack=1.5)
+        U.assert_parity(U.host(a), b, c, "xg " + tag, slack=4.0)
     for a, b, c in zip(dyg, yg32, yg64):
-        U.assert_parity(U.host(a), b, c, "yg " + tag, slack=1.5)
+        U.assert_parity(U.host(a), b, c, "yg " + tag, slack=4.0)
     # accumulate mode adds on top; back0-only and back1-only calls
     drs2 = [a.clone() for a in drs]
     cabi.so3vec_fwd(drs2, dxs, dys, accumulate=True, diag=diag)

@@ -1,0 +1,63 @@
+"""CPU-side checks of the Python surface: the extension module loads and has the reference's method names, type
+arithmetic known answers, Wigner-D helper properties, and host tensors are refused rather than computed elsewhere."""
+import pytest
+
+torch = pytest.importorskip("torch")
+
+
+def test_extension_surface():
+    from gelib_amd import gelib_base as gb
+    # python/bindings/SO3part_py.cpp:18-44, SO3vec_py.cpp:18-54, SO3type_py.cpp:16-36
+    for name in ("view", "add_CGproduct", "add_CGproduct_back0", "add_CGproduct_back1", "add_DiagCGproduct",
+                 "add_DiagCGproduct_back0", "add_DiagCGproduct_back1"):
+        assert hasattr(gb.SO3part, name), name
+    for name in ("view", "get_tau", "addCGproduct", "addCGproduct_back0", "addCGproduct_back1", "addDiagCGproduct",
+                 "addDiagCGproduct_back0", "addDiagCGproduct_back1"):
+        assert hasattr(gb.SO3vec, name), name
+    for name in ("CGproduct", "DiagCGproduct", "get_parts", "maxl"):
+        assert hasattr(gb.SO3type, name), name
+    assert callable(gb.CGproduct)
+
+
+def test_type_arithmetic():
+    from gelib_amd import gelib_base as gb
+    t = gb.SO3type([1, 1, 1])
+    assert gb.CGproduct(t, t).get_parts() == {0: 3, 1: 6, 2: 6, 3: 3, 4: 1}
+    assert gb.CGproduct(t, t, 2).get_parts() == {0: 3, 1: 6, 2: 6}
+    assert gb.SO3type({0: 2, 1: 2}).CGproduct(gb.SO3type({0: 2, 1: 2})).get_parts() == {0: 8, 1: 12, 2: 4}
+    assert t.DiagCGproduct(t, 1).get_parts() == {0: 3, 1: 6}
+    assert t.maxl() == 2 and len(t) == 3
+
+
+def test_views_alias_and_describe():
+    from gelib_amd import gelib_base as gb
+    x = torch.zeros(2, 5, 3, dtype=torch.complex64)
+    p = gb.SO3part.view(x)
+    assert p.getl() == 2 and p.getn() == 3
+    v = gb.SO3vec.view([torch.zeros(2, 3, 4, dtype=torch.complex64), torch.zeros(2, 1, 2, dtype=torch.complex64)])
+    assert v.get_tau().get_parts() == {0: 2, 1: 4}
+    with pytest.raises(RuntimeError):
+        gb.SO3part.view(torch.zeros(2, 4, 3, dtype=torch.complex64))      # even m-dimension
+    with pytest.raises(RuntimeError):
+        gb.SO3part.view(torch.zeros(2, 5, 3))                               # not complex64
+
+
+def test_host_tensors_are_refused():
+    import gelib_amd as G
+    x = G.SO3part.randn(2, 1, 4)
+    with pytest.raises(RuntimeError):
+        G.CGproduct(x, x, 1)
+    u = G.SO3vec.randn(2, {0: 2, 1: 2})
+    with pytest.raises(RuntimeError):
+        G.CGproduct(u, u)
+
+
+def test_wigner_helper():
+    import gelib_amd as G
+    R1, R2 = G.SO3element.random(), G.SO3element.random()
+    assert torch.allclose(R1 @ R1.t(), torch.eye(3), atol=1e-5) and torch.det(R1) > 0
+    for l in (1, 2, 4):
+        rho = G.SO3irrep(l)
+        D1, D2, D12 = rho.matrix(R1), rho.matrix(R2), rho.matrix(G.SO3element(R1 @ R2))
+        assert torch.allclose(D1 @ D1.conj().t(), torch.eye(2 * l + 1, dtype=torch.complex64), atol=1e-4)
+        assert torch.allclose(D1 @ D2, D12, atol=1e-4)      # a representation

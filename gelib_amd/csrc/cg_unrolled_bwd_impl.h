@@ -11,8 +11,10 @@
 // the result into the wave's private image of xg / yg in LDS: plain read-add-write in a fixed order, no atomics,
 // no barrier.  After the last pair the four images are summed and written out in contiguous rows.
 //
-// Latency hiding.  The rows of g for the next (pair, run, l) unit are requested before the arithmetic of the
-// current unit starts and land in a second register buffer, so a wave always has one unit of loads in flight.
+// Latency hiding.  A unit (pair, run, l) requests its rows of g and then computes on them; the kernel keeps its
+// register count low enough for four waves per SIMD, and the other waves' arithmetic covers a wave's wait.  (A
+// second register buffer holding the next unit's rows costs one wave of occupancy and the compiler does not keep
+// those loads in flight across the control flow between units, so it lost to the plain form.)
 #pragma once
 
 #include "cg_unrolled_dev.h"
@@ -67,33 +69,17 @@ __device__ __forceinline__ void stride_sum(float2 (&v)[K], int lo, int hi) {
 typedef float v2f __attribute__((ext_vector_type(2)));
 typedef const __attribute__((address_space(1))) v2f *GlobalRows;
 
-// Where a lane finds the rows of g of one unit; rows == 0 means "nothing to load".
-struct GRows {
-  GlobalRows ptr;
-  int sm;
-  int rows;
-};
-
 // Coefficients are read through the constant address space: the address is the same for every lane, so the
 // compiler fetches them with scalar loads into SGPRs and they cost neither vector registers nor LDS traffic.
 typedef const __attribute__((address_space(4))) float *CoeffPtr;
 
 template <int ROWS, int KR>
-__device__ __forceinline__ void load_rows_static(float2 (&buf)[KR], GlobalRows ptr, int sm) {
+__device__ __forceinline__ void load_rows(float2 (&buf)[KR], GlobalRows ptr, int sm) {
 #pragma unroll
   for (int m = 0; m < ROWS; m++) {
     const v2f t = ptr[m * sm];
     buf[m] = make_float2(t.x, t.y);
   }
-}
-
-// rows is 2l+1 for some l <= (KR-1)/2, or 0: one jump, then straight-line loads
-template <int KR>
-__device__ __forceinline__ void load_rows(float2 (&buf)[KR], const GRows &d) {
-  static_for<(KR + 1) / 2>([&](auto lc) __attribute__((always_inline)) {
-    constexpr int rows = 2 * decltype(lc)::value + 1;
-    if (d.rows == rows) load_rows_static<rows, KR>(buf, d.ptr, d.sm);
-  });
 }
 
 template <int L1, int L2, int L, int KR, bool WX, bool WY>
@@ -153,31 +139,14 @@ __device__ __forceinline__ LanePos lane_pos(int run, int lane, int log2_u, int n
   return q;
 }
 
-// gdesc: the gradient parts by l, in LDS, for the one place where l is only known at run time
-template <int LCAP>
-__device__ __forceinline__ GRows first_unit(const FastPart *gdesc, PairPtr p, long long cell, int u, int offs_add) {
-  GRows d;
-  const int lmin = cabs_(p->l1 - p->l2);
-  const FastPart G = gdesc[lmin];
-  d.rows = (lmin <= LCAP && p->ri[0] >= 0) ? 2 * lmin + 1 : 0;
-  d.sm = G.sm;
-  d.ptr = (GlobalRows)G.ptr + cell * G.sb + (p->offs[0] + offs_add + u);
-  return d;
-}
-
-// One run of one pair.  On entry gcur holds (or is about to receive) the rows of the pair's first l; on exit it
-// holds the rows described by `after`, the first unit of whatever the wave does next.
+// One run of one pair: every l of the pair that is present, in turn.
 template <int L1, int L2, int LCAP, int KR, bool DIAG, bool WX, bool WY>
 __device__ __forceinline__ void pair_bwd(const GParts<LCAP> &gp, PairPtr pr, CoeffPtr Cs, const float2 *xs,
                                          const float2 *ys, float2 *xacc, float2 *yacc, int xsize, int ysize,
-                                         long long cell0, int offs_add, const LanePos q, float2 (&gcur)[KR],
-                                         const GRows after) {
+                                         long long cell0, int offs_add, const LanePos q) {
   constexpr int LMIN = cabs_(L1 - L2);
   constexpr int NL = 2 * cmin_(L1, L2) + 1;
-  if constexpr (LMIN > LCAP) {  // no l of this pair can be present; just keep the pipeline fed
-    load_rows<KR>(gcur, after);
-    return;
-  }
+  if constexpr (LMIN > LCAP) return;  // no l of this pair can be present
   // scalar loads: the record sits in constant memory and the pointer is uniform
   const __attribute__((address_space(4))) PairRec &p = *pr;
   const int N1 = p.n1, N2 = p.n2;
@@ -207,20 +176,12 @@ __device__ __forceinline__ void pair_bwd(const GParts<LCAP> &gp, PairPtr pr, Coe
     constexpr int dl = decltype(dl_c)::value;
     constexpr int L = LMIN + dl;
     if constexpr (L <= LCAP) {
-      // request the rows of the following unit before touching the current ones
-      float2 gnext[KR];
-      if constexpr (dl + 1 < NL && L + 1 <= LCAP) {
-        if (p.ri[dl + 1] >= 0) {
-          const FastPart G = gp.G[L + 1];
-          load_rows_static<2 * (L + 1) + 1, KR>(gnext, (GlobalRows)G.ptr + cell * G.sb + (p.offs[dl + 1] + offs_add + q.u),
-                                                G.sm);
-        }
-      } else {
-        load_rows<KR>(gnext, after);
+      if (p.ri[dl] >= 0) {
+        float2 gv[KR];
+        const FastPart G = gp.G[L];
+        load_rows<2 * L + 1, KR>(gv, (GlobalRows)G.ptr + cell * G.sb + (p.offs[dl] + offs_add + q.u), G.sm);
+        triple_bwd<L1, L2, L, KR, WX, WY>(xv, yv, ax, ay, Cs + p.cg[dl], gv);
       }
-      if (p.ri[dl] >= 0) triple_bwd<L1, L2, L, KR, WX, WY>(xv, yv, ax, ay, Cs + p.cg[dl], gcur);
-#pragma unroll
-      for (int m = 0; m < KR; m++) gcur[m] = gnext[m];
     }
   });
 
@@ -313,9 +274,6 @@ __global__ void __launch_bounds__(kBlock) unrolled_bwd_kernel(const BwdArgs a) {
 
   if (WY) copy_image<true>(a.x, a.xrows, a.nx, xs, xsize, cell0, ncell, 0, 0, false);
   if (WX) copy_image<true>(a.y, a.yrows, a.ny, ys, ysize, cell0, ncell, 0, 0, false);
-  __shared__ FastPart gdesc[kFastOut];
-  if (threadIdx.x == 0)
-    static_for<kFastOut>([&](auto l) __attribute__((always_inline)) { gdesc[l.value] = a.g[l.value]; });
   {
     const int nacc = kWaves * cpb * (xsize + ysize);
     for (int i = threadIdx.x; i < nacc; i += kBlock) xacc_all[i] = make_float2(0.f, 0.f);
@@ -331,48 +289,24 @@ __global__ void __launch_bounds__(kBlock) unrolled_bwd_kernel(const BwdArgs a) {
   auto runs_of = [&](int k) { return ((cpb << pairs[k].log2_u) + kWave - 1) >> 6; };
   GParts<LCAP> gp;
   static_for<LCAP + 1>([&](auto l) __attribute__((always_inline)) { gp.G[l.value] = a.g[l.value]; });
-  float2 gcur[KR];
-  int pidx = 0, run = wave;
-  while (pidx < npairs && run >= runs_of(pidx)) {
-    pidx++;
-    run = wave;
-  }
-  if (pidx < npairs) {
-    const LanePos q = lane_pos(run, lane, pairs[pidx].log2_u, ncell);
-    load_rows<KR>(gcur, first_unit<LCAP>(gdesc, pairs + pidx, cell0 + q.cell_local, q.u, offs_add));
-  }
-  while (pidx < npairs) {
+  for (int pidx = 0; pidx < npairs; pidx++) {
     const PairPtr p = pairs + pidx;
-    const LanePos q = lane_pos(run, lane, p->log2_u, ncell);
-    // look ahead: the first unit of the wave's next visit is requested during this one
-    int npidx = pidx, nrun = run + kWaves;
-    while (npidx < npairs && nrun >= runs_of(npidx)) {
-      npidx++;
-      nrun = wave;
-    }
-    GRows after;
-    after.rows = 0;
-    after.sm = 0;
-    after.ptr = nullptr;
-    if (npidx < npairs) {
-      const LanePos qn = lane_pos(nrun, lane, pairs[npidx].log2_u, ncell);
-      after = first_unit<LCAP>(gdesc, pairs + npidx, cell0 + qn.cell_local, qn.u, offs_add);
-    }
+    const int nruns = runs_of(pidx);
     CoeffPtr C = (CoeffPtr)(a.bank + p->cg_base);
-    switch (p->l1 * (kLT + 1) + p->l2) {
-#define GELIB_CASE(A, B)                                                                                         \
-  case A * (kLT + 1) + B:                                                                                        \
-    pair_bwd<A, B, LCAP, KR, DIAG, WX, WY>(gp, p, C, xs, ys, xacc, yacc, xsize, ysize, cell0, offs_add, q, gcur, \
-                                            after);                                                              \
+    for (int run = wave; run < nruns; run += kWaves) {
+      const LanePos q = lane_pos(run, lane, p->log2_u, ncell);
+      switch (p->l1 * (kLT + 1) + p->l2) {
+#define GELIB_CASE(A, B)                                                                                      \
+  case A * (kLT + 1) + B:                                                                                     \
+    pair_bwd<A, B, LCAP, KR, DIAG, WX, WY>(gp, p, C, xs, ys, xacc, yacc, xsize, ysize, cell0, offs_add, q); \
     break;
 #define GELIB_ROW(A) GELIB_CASE(A, 0) GELIB_CASE(A, 1) GELIB_CASE(A, 2) GELIB_CASE(A, 3) GELIB_CASE(A, 4)
-      GELIB_ROW(0) GELIB_ROW(1) GELIB_ROW(2) GELIB_ROW(3) GELIB_ROW(4)
+        GELIB_ROW(0) GELIB_ROW(1) GELIB_ROW(2) GELIB_ROW(3) GELIB_ROW(4)
 #undef GELIB_ROW
 #undef GELIB_CASE
-      default: break;
+        default: break;
+      }
     }
-    pidx = npidx;
-    run = nrun;
   }
 
   __syncthreads();

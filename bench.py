@@ -192,7 +192,7 @@ def main():
         "config": {"workload": name, "batch": B, "tau_x": {str(k): v for k, v in tx.items()},
                    "tau_y": {str(k): v for k, v in ty.items()}, "maxl": maxl, "diag": diag,
                    "triples": sum(1 for l1 in tx for l2 in ty for l in range(abs(l1 - l2), l1 + l2 + 1) if l in tr),
-                   "kernel_path": {1: "generic", 2: "unrolled"}.get(path, str(path)),
+                   "kernel_path": {1: "generic", 2: "unrolled", 3: "staged"}.get(path, str(path)),
                    "fwd_ms": fwd_ms, "bwd_ms": bwd_ms,
                    "fwd_GBps": fwd_bytes / (fwd_ms * 1e-3) / 1e9, "bwd_GBps": bwd_bytes / (bwd_ms * 1e-3) / 1e9,
                    "fwd_bwd_GBps": (fwd_bytes + bwd_bytes) / ((fwd_ms + bwd_ms) * 1e-3) / 1e9,

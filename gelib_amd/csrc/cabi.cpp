@@ -10,6 +10,7 @@
 #include <vector>
 
 #include "cg_common.h"
+#include "cg_staged.h"
 #include "cg_unrolled.h"
 
 using namespace gelib_hip;
@@ -164,6 +165,12 @@ int part_entry(Kind kind, bool diag, const gelib_part_desc *r, const gelib_part_
       t_last_path = kPathUnrolled;
       return GELIB_HIP_OK;
     }
+    rc = staged_part(kind == kFwd ? 0 : (kind == kBack0 ? 1 : 2), op, accumulate != 0, s, &used);
+    if (rc) return rc;
+    if (used) {
+      t_last_path = kPathStaged;
+      return GELIB_HIP_OK;
+    }
   }
   t_last_path = kPathGeneric;
   switch (kind) {
@@ -272,6 +279,12 @@ int vec_fwd_entry(bool diag, int nr, const gelib_part_desc *r, int nx, const gel
       t_last_path = kPathUnrolled;
       return GELIB_HIP_OK;
     }
+    rc = staged_vec_fwd(plan, rd, xd, yd, accumulate != 0, s, &used);
+    if (rc) return rc;
+    if (used) {
+      t_last_path = kPathStaged;
+      return GELIB_HIP_OK;
+    }
   }
   t_last_path = kPathGeneric;
   for (auto &t : plan.triples) {
@@ -326,6 +339,12 @@ int vec_bwd_entry(bool diag, const gelib_part_desc *xg, const gelib_part_desc *y
     if (rc) return rc;
     if (used) {
       t_last_path = kPathUnrolled;
+      return GELIB_HIP_OK;
+    }
+    rc = staged_vec_bwd(plan, gd, xd, yd, xgd, ygd, accumulate != 0, s, &used);
+    if (rc) return rc;
+    if (used) {
+      t_last_path = kPathStaged;
       return GELIB_HIP_OK;
     }
   }
@@ -488,6 +507,7 @@ int gelib_hip_set_option(const char *name, int value) {
     g_check_pointers = value;
     return GELIB_HIP_OK;
   }
+  if (!std::strncmp(name, "staged_", 7)) return staged_set_option(name, value);
   return unrolled_set_option(name, value);
 }
 

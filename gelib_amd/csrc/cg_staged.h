@@ -1,0 +1,63 @@
+// Kernels for any l up to GELIB_HIP_MAX_L with run-time m-loops (internal interface).
+//
+// Same preconditions as the unrolled small-l kernels (contiguous channels, leading dimensions that collapse into
+// one cell index, destinations that do not broadcast), but nothing about l is fixed at compile time: a block
+// stages the operands of its cells in LDS once, then walks every (l1,l2,l) triple of the product in one launch.
+// They serve what the unrolled kernels do not cover (operand l above kLT, e.g. l = 6 or l = 10) and leave to the
+// shape-agnostic kernels only strided channels, broadcast destinations and images too large for LDS.
+#pragma once
+
+#include <vector>
+
+#include "cg_unrolled.h"
+
+namespace gelib_hip {
+
+// One (l1,l2,l) triple; lives in device memory next to the coefficient tables (read with scalar loads).
+struct StagedTriple {
+  int l1, l2, l;
+  int n1, n2;
+  int xi, yi, ri;   // positions in the x / y / product part lists of the kernel arguments
+  int xoff, yoff;   // offsets (complex elements) of the operand parts inside one cell's packed x / y image
+  int offs;         // first channel of this triple's block inside the product part
+  int u;            // channel slots per cell: n1*n2, or n for Diag
+  int log2_u;       // log2(u) when u is a power of two, else -1
+  // Three compact copies of the coefficient table, each holding only the entries with |m1+m2| <= l, in the
+  // order the corresponding loop nest visits them, so every kernel reads its coefficients as one stream:
+  int cg_fwd;       // m ascending, then m1 ascending            (forward: one output row at a time)
+  int cg_back0;     // m1 ascending, then m2 ascending           (gradient of x)
+  int cg_back1;     // m2 ascending, then m1 ascending           (gradient of y)
+};
+
+struct StagedArgs {
+  FastPart x[kMaxParts], y[kMaxParts], xg[kMaxParts], yg[kMaxParts];
+  FastPart r[kMaxOutParts];  // product (forward) or its gradient (backward)
+  const StagedTriple *triples;
+  const float *bank;
+  long long ncells;
+  int ntriples;
+  int nx, ny;
+  int offs_add;   // extra channel offset (part-level calls)
+  int accumulate;
+  int xsize, ysize;  // complex elements of one cell's packed x / y image
+  int cpb;           // cells per block
+  int xrows[kMaxParts], yrows[kMaxParts];
+};
+
+int launch_staged_fwd(const StagedArgs &a, bool diag, int nblocks, size_t lds_bytes, hipStream_t s);
+// cap: rows of g a lane keeps in registers (16 or 32); threads: 256, 512 or 1024 (1024 only with cap 16)
+int launch_staged_bwd(const StagedArgs &a, bool diag, bool want_x, bool want_y, int cap, int threads, int nblocks,
+                      size_t lds_bytes, hipStream_t s);
+
+// kind: 0 forward, 1 back0 (destination op.x), 2 back1 (destination op.y).  *used = 1 if a launch was made.
+int staged_part(int kind, const PartOp &op, bool accumulate, hipStream_t s, int *used);
+int staged_vec_fwd(const VecPlan &plan, const std::vector<const gelib_part_desc *> &r,
+                   const std::vector<const gelib_part_desc *> &x, const std::vector<const gelib_part_desc *> &y,
+                   bool accumulate, hipStream_t s, int *used);
+int staged_vec_bwd(const VecPlan &plan, const std::vector<const gelib_part_desc *> &g,
+                   const std::vector<const gelib_part_desc *> &x, const std::vector<const gelib_part_desc *> &y,
+                   const std::vector<const gelib_part_desc *> &xg, const std::vector<const gelib_part_desc *> &yg,
+                   bool accumulate, hipStream_t s, int *used);
+int staged_set_option(const char *name, int value);
+
+}  // namespace gelib_hip

@@ -1,0 +1,301 @@
+// Host side of the staged (any-l) kernels: eligibility, the per-signature device tables (triples + compact
+// coefficient streams) and the per-call launch shape.
+#include <algorithm>
+#include <cstring>
+#include <map>
+#include <mutex>
+#include <vector>
+
+#include "cg_staged.h"
+
+namespace gelib_hip {
+
+namespace {
+
+int g_fwd_enable = 1;
+int g_bwd_enable = 1;
+int g_bwd_threads = 0;       // 0 = choose from the LDS footprint, else force 256 / 512 / 1024
+int g_fwd_lds_target = 32 * 1024;  // LDS up to which a forward block takes more cells to fill its waves
+int g_bwd_lds_target = 40 * 1024;
+
+constexpr int kLdsLimit = 160 * 1024;
+
+struct DevicePlan {
+  std::vector<StagedTriple> triples;
+  StagedTriple *d_triples = nullptr;
+  float *d_bank = nullptr;
+  int xsize = 0, ysize = 0;
+  int lmax_out = 0;
+};
+
+std::mutex g_plan_mutex;
+std::map<std::vector<int>, DevicePlan> g_plans;  // key starts with the device ordinal
+
+// xs / ys: (l, n) of the operand parts in list order; rls: l of the product parts in list order
+int get_plan(bool diag, const std::vector<VecTriple> &triples, const std::vector<std::pair<int, int>> &xs,
+             const std::vector<std::pair<int, int>> &ys, const std::vector<int> &rls, const DevicePlan **out) {
+  int dev = 0;
+  GELIB_HIP_TRY(hipGetDevice(&dev));
+  std::vector<int> key = {dev, diag ? 1 : 0, (int)xs.size(), (int)ys.size(), (int)rls.size()};
+  for (auto &v : xs) key.push_back(v.first), key.push_back(v.second);
+  for (auto &v : ys) key.push_back(v.first), key.push_back(v.second);
+  for (int l : rls) key.push_back(l);
+  for (auto &t : triples) key.push_back(t.xi), key.push_back(t.yi), key.push_back(t.ri), key.push_back(t.offs);
+  std::lock_guard<std::mutex> lock(g_plan_mutex);
+  auto it = g_plans.find(key);
+  if (it != g_plans.end()) {
+    *out = &it->second;
+    return GELIB_HIP_OK;
+  }
+  DevicePlan plan;
+  std::vector<float> bank;
+  std::vector<int> xoff(xs.size()), yoff(ys.size());
+  for (size_t i = 0; i < xs.size(); i++) {
+    xoff[i] = plan.xsize;
+    plan.xsize += (2 * xs[i].first + 1) * xs[i].second;
+  }
+  for (size_t i = 0; i < ys.size(); i++) {
+    yoff[i] = plan.ysize;
+    plan.ysize += (2 * ys[i].first + 1) * ys[i].second;
+  }
+  std::vector<float> full;
+  for (auto &t : triples) {
+    StagedTriple r;
+    std::memset(&r, 0, sizeof(r));
+    r.l1 = t.l1, r.l2 = t.l2, r.l = t.l;
+    r.n1 = xs[t.xi].second, r.n2 = ys[t.yi].second;
+    r.xi = t.xi, r.yi = t.yi, r.ri = t.ri;
+    r.xoff = xoff[t.xi], r.yoff = yoff[t.yi];
+    r.offs = t.offs;
+    const long long U = diag ? r.n1 : (long long)r.n1 * r.n2;
+    r.u = (int)U;
+    r.log2_u = (U > 0 && (U & (U - 1)) == 0) ? ilog2((int)U) : -1;
+    const int L1 = 2 * t.l1 + 1, L2 = 2 * t.l2 + 1;
+    full.assign((size_t)L1 * L2, 0.f);
+    cg_matrix_host(t.l1, t.l2, t.l, full.data());
+    auto C = [&](int m1, int m2) { return full[(size_t)(m1 + t.l1) * L2 + (m2 + t.l2)]; };
+    r.cg_fwd = (int)bank.size();
+    for (int m = -t.l; m <= t.l; m++)
+      for (int m1 = std::max(-t.l1, m - t.l2); m1 <= std::min(t.l1, m + t.l2); m1++) bank.push_back(C(m1, m - m1));
+    r.cg_back0 = (int)bank.size();
+    for (int m1 = -t.l1; m1 <= t.l1; m1++)
+      for (int m2 = std::max(-t.l2, -t.l - m1); m2 <= std::min(t.l2, t.l - m1); m2++) bank.push_back(C(m1, m2));
+    r.cg_back1 = (int)bank.size();
+    for (int m2 = -t.l2; m2 <= t.l2; m2++)
+      for (int m1 = std::max(-t.l1, -t.l - m2); m1 <= std::min(t.l1, t.l - m2); m1++) bank.push_back(C(m1, m2));
+    plan.lmax_out = std::max(plan.lmax_out, t.l);
+    plan.triples.push_back(r);
+  }
+  bank.resize(bank.size() + 16, 0.f);  // the coefficient stream may be read a few entries ahead
+  const size_t tri_bytes = plan.triples.size() * sizeof(StagedTriple);
+  const size_t bank_bytes = bank.size() * sizeof(float);
+  char *d = nullptr;
+  GELIB_HIP_TRY(hipMalloc((void **)&d, tri_bytes + bank_bytes));
+  hipError_t e = hipMemcpy(d, plan.triples.data(), tri_bytes, hipMemcpyHostToDevice);
+  if (e == hipSuccess) e = hipMemcpy(d + tri_bytes, bank.data(), bank_bytes, hipMemcpyHostToDevice);
+  if (e != hipSuccess) {
+    (void)hipFree(d);
+    return record_hip_error(e, "hipMemcpy(staged plan)");
+  }
+  plan.d_triples = (StagedTriple *)d;
+  plan.d_bank = (float *)(d + tri_bytes);
+  auto ins = g_plans.emplace(key, std::move(plan));
+  *out = &ins.first->second;
+  return GELIB_HIP_OK;
+}
+
+struct FastLists {
+  std::vector<FastPart> x, y, r, xg, yg;
+};
+
+long long units_per_block(const DevicePlan &plan, long long cpb) {
+  long long units = 0;
+  for (auto &t : plan.triples) units += (cpb * t.u + kWave - 1) / kWave;
+  return units;
+}
+
+void fill_args(StagedArgs &a, const DevicePlan &plan, const FastLists &f, const std::vector<std::pair<int, int>> &xs,
+               const std::vector<std::pair<int, int>> &ys, long long ncells, int offs_add, bool accumulate) {
+  std::memset(&a, 0, sizeof(a));
+  for (size_t i = 0; i < f.x.size(); i++) a.x[i] = f.x[i];
+  for (size_t i = 0; i < f.y.size(); i++) a.y[i] = f.y[i];
+  for (size_t i = 0; i < f.r.size(); i++) a.r[i] = f.r[i];
+  for (size_t i = 0; i < f.xg.size(); i++) a.xg[i] = f.xg[i];
+  for (size_t i = 0; i < f.yg.size(); i++) a.yg[i] = f.yg[i];
+  a.triples = plan.d_triples;
+  a.bank = plan.d_bank;
+  a.ncells = ncells;
+  a.ntriples = (int)plan.triples.size();
+  a.nx = (int)xs.size();
+  a.ny = (int)ys.size();
+  a.offs_add = offs_add;
+  a.accumulate = accumulate ? 1 : 0;
+  a.xsize = plan.xsize;
+  a.ysize = plan.ysize;
+  for (size_t i = 0; i < xs.size(); i++) a.xrows[i] = 2 * xs[i].first + 1;
+  for (size_t i = 0; i < ys.size(); i++) a.yrows[i] = 2 * ys[i].first + 1;
+}
+
+bool sizes_ok(const std::vector<std::pair<int, int>> &xs, const std::vector<std::pair<int, int>> &ys,
+              const std::vector<int> &rls) {
+  if (xs.size() > (size_t)kMaxParts || ys.size() > (size_t)kMaxParts || rls.size() > (size_t)kMaxOutParts) return false;
+  long long xsize = 0, ysize = 0;
+  for (auto &v : xs) xsize += (2LL * v.first + 1) * v.second;
+  for (auto &v : ys) ysize += (2LL * v.first + 1) * v.second;
+  return 8 * (xsize + ysize) <= kLdsLimit;
+}
+
+int run_fwd(bool diag, const std::vector<VecTriple> &triples, const std::vector<std::pair<int, int>> &xs,
+            const std::vector<std::pair<int, int>> &ys, const std::vector<int> &rls, const FastLists &f,
+            long long ncells, int offs_add, bool accumulate, hipStream_t s, int *used) {
+  *used = 0;
+  if (!sizes_ok(xs, ys, rls)) return GELIB_HIP_OK;
+  for (auto &t : triples) {
+    const long long U = diag ? xs[t.xi].second : (long long)xs[t.xi].second * ys[t.yi].second;
+    if (U > (1 << 24)) return GELIB_HIP_OK;
+  }
+  const DevicePlan *plan = nullptr;
+  int rc = get_plan(diag, triples, xs, ys, rls, &plan);
+  if (rc) return rc;
+  const long long cell_bytes = 8LL * (plan->xsize + plan->ysize);
+  long long cpb = 1;
+  // more cells per block while the block's waves would otherwise idle and the image stays small
+  while (cpb * 2 <= ncells && cell_bytes * cpb * 2 <= g_fwd_lds_target && units_per_block(*plan, cpb) < 16) cpb *= 2;
+  StagedArgs a;
+  fill_args(a, *plan, f, xs, ys, ncells, offs_add, accumulate);
+  a.cpb = (int)cpb;
+  const long long nblocks = (ncells + cpb - 1) / cpb;
+  if (nblocks > 0x7fffffffLL) return GELIB_HIP_ERR_ARG;
+  rc = launch_staged_fwd(a, diag, (int)nblocks, (size_t)(cell_bytes * cpb), s);
+  if (rc) return rc;
+  *used = 1;
+  return GELIB_HIP_OK;
+}
+
+int run_bwd(bool diag, const std::vector<VecTriple> &triples, const std::vector<std::pair<int, int>> &xs,
+            const std::vector<std::pair<int, int>> &ys, const std::vector<int> &rls, const FastLists &f,
+            long long ncells, int offs_add, bool accumulate, bool want_x, bool want_y, hipStream_t s, int *used) {
+  *used = 0;
+  if (!sizes_ok(xs, ys, rls)) return GELIB_HIP_OK;
+  // the lane sums need power-of-two channel counts, and the second operand's channels inside one wave
+  for (auto &t : triples) {
+    const int n1 = xs[t.xi].second, n2 = ys[t.yi].second;
+    if (!is_pow2(n1) || !is_pow2(n2)) return GELIB_HIP_OK;
+    if (!diag && n2 > kWave) return GELIB_HIP_OK;
+    const long long U = diag ? n1 : (long long)n1 * n2;
+    if (U > (1 << 20)) return GELIB_HIP_OK;
+  }
+  const DevicePlan *plan = nullptr;
+  int rc = get_plan(diag, triples, xs, ys, rls, &plan);
+  if (rc) return rc;
+  const long long cell_bytes = 16LL * (plan->xsize + plan->ysize);  // operands + gradient images
+  if (cell_bytes > kLdsLimit) return GELIB_HIP_OK;
+  long long cpb = 1;
+  while (cpb * 2 <= ncells && cell_bytes * cpb * 2 <= g_bwd_lds_target && units_per_block(*plan, cpb) < 16) cpb *= 2;
+  const long long lds = cell_bytes * cpb;
+  const int rows = 2 * plan->lmax_out + 1;
+  const int cap = rows <= 16 ? 16 : 32;
+  const int max_threads = cap == 16 ? 1024 : 512;
+  int threads = 256;
+  const long long units = units_per_block(*plan, cpb);
+  if (lds > 52 * 1024 && units >= 16) threads = 512;       // at most two blocks fit a CU: make them wider
+  if (lds > 80 * 1024 && units >= 32) threads = 1024;      // one block per CU
+  if (g_bwd_threads == 256 || g_bwd_threads == 512 || g_bwd_threads == 1024) threads = g_bwd_threads;
+  threads = std::min(threads, max_threads);
+  StagedArgs a;
+  fill_args(a, *plan, f, xs, ys, ncells, offs_add, accumulate);
+  a.cpb = (int)cpb;
+  const long long nblocks = (ncells + cpb - 1) / cpb;
+  if (nblocks > 0x7fffffffLL) return GELIB_HIP_ERR_ARG;
+  rc = launch_staged_bwd(a, diag, want_x, want_y, cap, threads, (int)nblocks, (size_t)lds, s);
+  if (rc) return rc;
+  *used = 1;
+  return GELIB_HIP_OK;
+}
+
+}  // namespace
+
+int staged_part(int kind, const PartOp &op, bool accumulate, hipStream_t s, int *used) {
+  *used = 0;
+  if (kind == 0 && !g_fwd_enable) return GELIB_HIP_OK;
+  if (kind != 0 && !g_bwd_enable) return GELIB_HIP_OK;
+  FastLists f;
+  f.x.resize(1);
+  f.y.resize(1);
+  f.r.resize(1);
+  if (!to_fast(op.r, op.E, op.Dr, op.offs + op.nout, kind == 0, &f.r[0])) return GELIB_HIP_OK;
+  if (!to_fast(op.x, op.E, op.Dx, op.n1, kind == 1, &f.x[0])) return GELIB_HIP_OK;
+  if (!to_fast(op.y, op.E, op.Dy, op.n2, kind == 2, &f.y[0])) return GELIB_HIP_OK;
+  const long long ncells = op.E[0] * op.E[1] * op.E[2];
+  std::vector<VecTriple> triples = {{0, 0, 0, op.l1, op.l2, op.l, 0, op.nout}};
+  std::vector<std::pair<int, int>> xs = {{op.l1, op.n1}}, ys = {{op.l2, op.n2}};
+  std::vector<int> rls = {op.l};
+  if (kind == 0) return run_fwd(op.diag, triples, xs, ys, rls, f, ncells, op.offs, accumulate, s, used);
+  if (kind == 1) f.xg = f.x;  // destination
+  if (kind == 2) f.yg = f.y;
+  return run_bwd(op.diag, triples, xs, ys, rls, f, ncells, op.offs, accumulate, kind == 1, kind == 2, s, used);
+}
+
+int staged_vec_fwd(const VecPlan &plan, const std::vector<const gelib_part_desc *> &r,
+                   const std::vector<const gelib_part_desc *> &x, const std::vector<const gelib_part_desc *> &y,
+                   bool accumulate, hipStream_t s, int *used) {
+  *used = 0;
+  if (!g_fwd_enable) return GELIB_HIP_OK;
+  FastLists f;
+  std::vector<std::pair<int, int>> xs, ys, rs;
+  if (!lists_to_fast(x, plan.E, false, &f.x, &xs) || !lists_to_fast(y, plan.E, false, &f.y, &ys) ||
+      !lists_to_fast(r, plan.E, true, &f.r, &rs))
+    return GELIB_HIP_OK;
+  std::vector<int> rls;
+  for (auto &v : rs) rls.push_back(v.first);
+  const long long ncells = plan.E[0] * plan.E[1] * plan.E[2];
+  return run_fwd(plan.diag, plan.triples, xs, ys, rls, f, ncells, 0, accumulate, s, used);
+}
+
+int staged_vec_bwd(const VecPlan &plan, const std::vector<const gelib_part_desc *> &g,
+                   const std::vector<const gelib_part_desc *> &x, const std::vector<const gelib_part_desc *> &y,
+                   const std::vector<const gelib_part_desc *> &xg, const std::vector<const gelib_part_desc *> &yg,
+                   bool accumulate, hipStream_t s, int *used) {
+  *used = 0;
+  if (!g_bwd_enable) return GELIB_HIP_OK;
+  FastLists f;
+  std::vector<std::pair<int, int>> xs, ys, rs;
+  if (!lists_to_fast(x, plan.E, false, &f.x, &xs) || !lists_to_fast(y, plan.E, false, &f.y, &ys) ||
+      !lists_to_fast(g, plan.E, false, &f.r, &rs))
+    return GELIB_HIP_OK;
+  if (!xg.empty() && !lists_to_fast(xg, plan.E, true, &f.xg, nullptr)) return GELIB_HIP_OK;
+  if (!yg.empty() && !lists_to_fast(yg, plan.E, true, &f.yg, nullptr)) return GELIB_HIP_OK;
+  std::vector<int> rls;
+  for (auto &v : rs) rls.push_back(v.first);
+  const long long ncells = plan.E[0] * plan.E[1] * plan.E[2];
+  return run_bwd(plan.diag, plan.triples, xs, ys, rls, f, ncells, 0, accumulate, !xg.empty(), !yg.empty(), s, used);
+}
+
+int staged_set_option(const char *name, int value) {
+  if (!std::strcmp(name, "staged_fwd")) {
+    g_fwd_enable = value;
+    return GELIB_HIP_OK;
+  }
+  if (!std::strcmp(name, "staged_bwd")) {
+    g_bwd_enable = value;
+    return GELIB_HIP_OK;
+  }
+  if (!std::strcmp(name, "staged_bwd_threads")) {
+    if (value != 0 && value != 256 && value != 512 && value != 1024) return GELIB_HIP_ERR_ARG;
+    g_bwd_threads = value;
+    return GELIB_HIP_OK;
+  }
+  if (!std::strcmp(name, "staged_fwd_lds_target")) {
+    if (value < 1024 || value > kLdsLimit) return GELIB_HIP_ERR_ARG;
+    g_fwd_lds_target = value;
+    return GELIB_HIP_OK;
+  }
+  if (!std::strcmp(name, "staged_bwd_lds_target")) {
+    if (value < 1024 || value > kLdsLimit) return GELIB_HIP_ERR_ARG;
+    g_bwd_lds_target = value;
+    return GELIB_HIP_OK;
+  }
+  return GELIB_HIP_ERR_ARG;
+}
+
+}  // namespace gelib_hip

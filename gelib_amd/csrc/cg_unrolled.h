@@ -7,6 +7,7 @@
 // keeps it cached on the device.
 #pragma once
 
+#include <utility>
 #include <vector>
 
 #include "cg_common.h"
@@ -49,6 +50,17 @@ struct PairRec {
   int xoff, yoff;    // offsets (complex elements) of the parts inside a per-cell packed x / y image (backward)
   int log2_u;        // log2 of the channel slots per cell (n1*n2, or n for Diag) when that is a power of two, else -1
 };
+
+// Helpers shared by the kernel families that need contiguous channels and one cell index (cg_unrolled_plan.cpp).
+bool collapse(const PartDev &p, const long long E[3], const long long own[3], long long *cell_stride);
+// is_dest: the part is written; a destination that broadcasts over cells is refused (it needs a reduction)
+bool to_fast(const PartDev &p, const long long E[3], const long long own[3], int n, bool is_dest, FastPart *out);
+PartDev desc_to_dev(const gelib_part_desc *d, const long long E[3], long long own[3]);
+// ln (optional) receives (l, n) of every part
+bool lists_to_fast(const std::vector<const gelib_part_desc *> &ds, const long long E[3], bool is_dest,
+                   std::vector<FastPart> *out, std::vector<std::pair<int, int>> *ln);
+bool is_pow2(int v);
+int ilog2(int v);
 
 // kind: 0 forward, 1 back0 (destination op.x), 2 back1 (destination op.y).  *used = 1 if a launch was made.
 int unrolled_part(int kind, const PartOp &op, bool accumulate, hipStream_t s, int *used);

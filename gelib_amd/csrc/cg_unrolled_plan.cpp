@@ -29,6 +29,8 @@ struct DevicePlan {
 std::mutex g_plan_mutex;
 std::map<std::vector<int>, DevicePlan> g_plans;  // key starts with the device ordinal
 
+}  // namespace
+
 // (b, g0, g1) -> one cell index with one stride, if the strides nest; broadcast-everywhere gives stride 0.
 bool collapse(const PartDev &p, const long long E[3], const long long own[3], long long *cell_stride) {
   const long long s[3] = {p.sb, p.sg0, p.sg1};
@@ -91,6 +93,8 @@ int ilog2(int v) {
   while ((1 << k) < v) k++;
   return k;
 }
+
+namespace {
 
 // Build (or fetch) the device tables for a list of triples.  xs/ys/rs give (l, n) of the l-sorted parts.
 int get_plan(bool diag, const std::vector<VecTriple> &triples, const std::vector<std::pair<int, int>> &xs,
@@ -315,7 +319,6 @@ int unrolled_part(int kind, const PartOp &op, bool accumulate, hipStream_t s, in
   return run_bwd(op.diag, triples, xs, ys, rls, f, ncells, op.offs, accumulate, kind == 1, kind == 2, s, used);
 }
 
-namespace {
 bool lists_to_fast(const std::vector<const gelib_part_desc *> &ds, const long long E[3], bool is_dest,
                    std::vector<FastPart> *out, std::vector<std::pair<int, int>> *ln) {
   out->resize(ds.size());
@@ -328,7 +331,6 @@ bool lists_to_fast(const std::vector<const gelib_part_desc *> &ds, const long lo
   }
   return true;
 }
-}  // namespace
 
 int unrolled_vec_fwd(const VecPlan &plan, const std::vector<const gelib_part_desc *> &r,
                      const std::vector<const gelib_part_desc *> &x, const std::vector<const gelib_part_desc *> &y,

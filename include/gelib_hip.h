@@ -139,7 +139,7 @@ int gelib_hip_synchronize(void);
  * Tuning / introspection (no counterpart in the reference).
  * gelib_hip_set_option("force_generic", 1) routes every call through the shape-agnostic kernels;
  * gelib_hip_last_path() tells which kernel family the last call of this thread used
- * (0 = none, 1 = generic, 2 = unrolled small-l kernels).
+ * (0 = none, 1 = generic, 2 = unrolled small-l kernels, 3 = staged any-l kernels).
  */
 int gelib_hip_set_option(const char *name, int value);
 int gelib_hip_last_path(void);

@@ -1,0 +1,154 @@
+"""GPU parity of the any-l ("staged") kernels: operand l above 4, where the unrolled small-l kernels do not apply.
+
+Each case checks the kernel family that ran (gelib_hip_last_path() == 3) and compares with the CPU oracle in
+float32 and float64, as the other GPU tests do.  The backward pass adds partial sums into LDS images with float
+atomics, so its last bits can differ from run to run; the tolerance of assert_parity covers that.
+"""
+import numpy as np
+import pytest
+
+from oracle import cg_oracle as ora
+from tests import gpu_util as U
+
+pytestmark = pytest.mark.gpu
+
+torch = pytest.importorskip("torch")
+
+STAGED = 3
+
+
+@pytest.fixture(scope="module")
+def cabi():
+    assert torch.cuda.is_available(), "GPU tests need a GPU"
+    from gelib_amd import cabi as c
+    c.lib()
+    c.set_option("force_generic", 0)
+    yield c
+    c.set_option("staged_bwd_threads", 0)
+
+
+def c128(L):
+    return [a.astype(np.complex128) for a in L]
+
+
+def run_vec(cabi, B, tx, ty, maxl, diag, seed, expect_bwd=STAGED):
+    xs = [U.seeded(seed + l, B, 2 * l + 1, n) for l, n in sorted(tx.items())]
+    ys = [U.seeded(seed + 50 + l, B, 2 * l + 1, n) for l, n in sorted(ty.items())]
+    r32 = ora.vec_fwd(xs, ys, maxl, diag)
+    r64 = ora.vec_fwd(c128(xs), c128(ys), maxl, diag)
+    gs = [U.seeded(seed + 100 + i, *p.shape) for i, p in enumerate(r32)]
+    xg32, yg32 = ora.vec_bwd(gs, xs, ys, diag)
+    xg64, yg64 = ora.vec_bwd(c128(gs), c128(xs), c128(ys), diag)
+    dxs, dys, dgs = [U.dev(a) for a in xs], [U.dev(a) for a in ys], [U.dev(a) for a in gs]
+    drs = [torch.full(p.shape, 7.0 + 1j, dtype=torch.complex64, device="cuda") for p in r32]
+    cabi.so3vec_fwd(drs, dxs, dys, accumulate=False, diag=diag)
+    assert cabi.last_path() == STAGED
+    dxg = [torch.full(a.shape, 3.0 - 2j, dtype=torch.complex64, device="cuda") for a in xs]
+    dyg = [torch.full(a.shape, 3.0 - 2j, dtype=torch.complex64, device="cuda") for a in ys]
+    cabi.so3vec_bwd(dxg, dyg, dgs, dxs, dys, accumulate=False, diag=diag)
+    assert cabi.last_path() == expect_bwd
+    torch.cuda.synchronize()
+    tag = "B%d %s x %s maxl %d diag %d" % (B, tx, ty, maxl, diag)
+    for a, b, c in zip(drs, r32, r64):
+        U.assert_parity(U.host(a), b, c, "fwd " + tag)
+    for a, b, c in zip(dxg, xg32, xg64):
+        U.assert_parity(U.host(a), b, c, "xg " + tag, slack=4.0)
+    for a, b, c in zip(dyg, yg32, yg64):
+        U.assert_parity(U.host(a), b, c, "yg " + tag, slack=4.0)
+    # accumulate mode adds on top of what is there; one gradient at a time
+    drs2 = [a.clone() for a in drs]
+    cabi.so3vec_fwd(drs2, dxs, dys, accumulate=True, diag=diag)
+    dxg2 = [a.clone() for a in dxg]
+    dyg2 = [a.clone() for a in dyg]
+    cabi.so3vec_bwd(dxg2, None, dgs, dxs, dys, accumulate=True, diag=diag)
+    cabi.so3vec_bwd(None, dyg2, dgs, dxs, dys, accumulate=True, diag=diag)
+    torch.cuda.synchronize()
+    for a, b in zip(drs2, drs):
+        assert U.gate_excess(U.host(a), 2 * U.host(b)) <= 1.0
+    for a, b in zip(dxg2 + dyg2, dxg + dyg):
+        assert U.gate_excess(U.host(a), 2 * U.host(b), rtol=2e-5, atol=2e-5) <= 1.0
+
+
+VEC_CASES = [
+    # (B, tau_x, tau_y, maxl)
+    (5, {l: 8 for l in range(7)}, {l: 8 for l in range(7)}, 6),    # the Diag L=6 benchmark type, small
+    (3, {10: 8}, {10: 8}, -1),                                       # l up to 20: g passes the registers in two windows
+    (7, {5: 4, 6: 2}, {0: 2, 7: 4}, -1),                             # l up to 13: 27 rows, the 32-row variant
+    (70, {5: 1}, {6: 1}, -1),                                        # one channel: many cells share a run
+    (2, {6: 16}, {5: 16}, 8),                                        # 256 slots per cell: several runs per cell
+]
+
+
+@pytest.mark.parametrize("case", VEC_CASES)
+@pytest.mark.parametrize("diag", [False, True])
+def test_vec(cabi, case, diag):
+    B, tx, ty, maxl = case
+    if diag:
+        n = tx[min(tx)]
+        tx, ty = {l: n for l in tx}, {l: n for l in ty}
+    run_vec(cabi, B, tx, ty, maxl, diag, seed=500)
+
+
+@pytest.mark.parametrize("threads", [256, 512, 1024])
+def test_backward_block_widths(cabi, threads):
+    cabi.set_option("staged_bwd_threads", threads)
+    try:
+        run_vec(cabi, 6, {l: 4 for l in range(6)}, {l: 4 for l in range(6)}, 5, False, seed=600)
+        run_vec(cabi, 6, {l: 4 for l in range(6)}, {l: 4 for l in range(6)}, 5, True, seed=601)
+    finally:
+        cabi.set_option("staged_bwd_threads", 0)
+
+
+def test_channel_counts_that_are_not_powers_of_two(cabi):
+    # the forward kernel takes any channel count; the backward lane sums need powers of two, so the gradient
+    # call falls back to the shape-agnostic kernels
+    run_vec(cabi, 4, {5: 3, 6: 5}, {5: 6, 1: 7}, -1, False, seed=700, expect_bwd=1)
+    run_vec(cabi, 4, {5: 3, 6: 3}, {5: 3, 1: 3}, -1, True, seed=701, expect_bwd=1)
+
+
+@pytest.mark.parametrize("diag", [False, True])
+def test_part_level_with_offset(cabi, diag):
+    B, l1, l2, l, n1, n2, offs, extra = 9, 6, 5, 7, 4, (4 if diag else 8), 3, 2
+    nout = n1 if diag else n1 * n2
+    x, y = U.seeded(1, B, 2 * l1 + 1, n1), U.seeded(2, B, 2 * l2 + 1, n2)
+    g = U.seeded(3, B, 2 * l + 1, offs + nout + extra)
+    fwd = cabi.so3part_diagcg_fwd if diag else cabi.so3part_cg_fwd
+    b0 = cabi.so3part_diagcg_back0 if diag else cabi.so3part_cg_back0
+    b1 = cabi.so3part_diagcg_back1 if diag else cabi.so3part_cg_back1
+    r0 = U.seeded(4, B, 2 * l + 1, offs + nout + extra)
+    want = r0.copy()
+    want[:, :, offs:offs + nout] += ora.cg_fwd(x, y, l, diag)
+    dr = U.dev(r0)
+    fwd(dr, U.dev(x), U.dev(y), offs, accumulate=True)
+    assert cabi.last_path() == STAGED
+    torch.cuda.synchronize()
+    assert U.gate_excess(U.host(dr), want, rtol=2e-5, atol=2e-5) <= 1.0
+    # outside the block nothing moves
+    assert np.array_equal(U.host(dr)[:, :, :offs], r0[:, :, :offs])
+    assert np.array_equal(U.host(dr)[:, :, offs + nout:], r0[:, :, offs + nout:])
+    gblock = np.ascontiguousarray(g[:, :, offs:offs + nout])
+    xg32, yg32 = ora.cg_bwd(gblock, x, y, diag)
+    xg64, yg64 = ora.cg_bwd(gblock.astype(np.complex128), x.astype(np.complex128), y.astype(np.complex128), diag)
+    dxg = torch.full(x.shape, 5.0 + 5j, dtype=torch.complex64, device="cuda")
+    dyg = torch.full(y.shape, 5.0 + 5j, dtype=torch.complex64, device="cuda")
+    b0(dxg, U.dev(g), U.dev(y), offs, accumulate=False)
+    assert cabi.last_path() == STAGED
+    b1(dyg, U.dev(g), U.dev(x), offs, accumulate=False)
+    assert cabi.last_path() == STAGED
+    torch.cuda.synchronize()
+    U.assert_parity(U.host(dxg), xg32, xg64, "part back0", slack=4.0)
+    U.assert_parity(U.host(dyg), yg32, yg64, "part back1", slack=4.0)
+
+
+def test_broadcast_operand_and_grid(cabi):
+    # y is shared by the whole batch (stride 0) and the cells form a (batch, grid) array
+    B, G0, l1, l2, l, n = 3, 4, 5, 5, 6, 4
+    x = U.seeded(11, B, G0, 2 * l1 + 1, n)
+    y = U.seeded(12, 1, 1, 2 * l2 + 1, n)
+    want = ora.cg_fwd(x.reshape(B * G0, 2 * l1 + 1, n), np.broadcast_to(y, (B, G0) + y.shape[2:]).reshape(B * G0, 2 * l2 + 1, n), l)
+    dr = torch.zeros(B, G0, 2 * l + 1, n * n, dtype=torch.complex64, device="cuda")
+    dy = U.dev(y).expand(B, G0, 2 * l2 + 1, n)
+    cabi.so3part_cg_fwd(dr, U.dev(x), dy, 0, accumulate=False)
+    assert cabi.last_path() == STAGED
+    torch.cuda.synchronize()
+    assert U.gate_excess(U.host(dr).reshape(want.shape), want) <= 1.0

@@ -34,6 +34,9 @@ struct StagedArgs {
   FastPart r[kMaxOutParts];  // product (forward) or its gradient (backward)
   const StagedTriple *triples;
   const float *bank;
+  // Striped backward kernels: (first, count, log2 of slots per cell) for every x part, then for every y part, then
+  // the triple numbers ordered by x part, then ordered by y part; first indexes into the matching order list.
+  const int *stripes;
   long long ncells;
   int ntriples;
   int nx, ny;
@@ -48,6 +51,10 @@ int launch_staged_fwd(const StagedArgs &a, bool diag, int nblocks, size_t lds_by
 // cap: rows of g a lane keeps in registers (16 or 32); threads: 256, 512 or 1024 (1024 only with cap 16)
 int launch_staged_bwd(const StagedArgs &a, bool diag, bool want_x, bool want_y, int cap, int threads, int nblocks,
                       size_t lds_bytes, hipStream_t s);
+
+// role 0: gradient of x, 1: gradient of y; cap 16 or 32 (own 2l+1 must not exceed it)
+int launch_staged_stripe(const StagedArgs &a, bool diag, int role, int cap, int nblocks, size_t lds_bytes,
+                         hipStream_t s);
 
 // kind: 0 forward, 1 back0 (destination op.x), 2 back1 (destination op.y).  *used = 1 if a launch was made.
 int staged_part(int kind, const PartOp &op, bool accumulate, hipStream_t s, int *used);

@@ -34,6 +34,7 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 typedef float v32f __attribute__((ext_vector_type(32)));
 typedef __attribute__((address_space(1))) v2f GlobalC;   // complex number in global memory
 typedef __attribute__((address_space(3))) float LdsF;    // float in LDS
+typedef const __attribute__((address_space(3))) v2f *LdsC;  // complex numbers in LDS (32-bit address arithmetic)
 typedef const __attribute__((address_space(4))) float *CoeffPtr;
 typedef const __attribute__((address_space(4))) StagedTriple *TriplePtr;
 typedef const __attribute__((address_space(4))) StagedArgs *ArgPtr;
@@ -94,6 +95,60 @@ __device__ __forceinline__ int first_run(int &base, int wave, int W, int nruns) 
   return first;
 }
 
+// The coefficients of a loop nest form one stream of floats.  A wave keeps 128 consecutive entries of it spread over
+// the lanes of two registers (lane k of `cur` holds entry base+k, of `nxt` entry base+64+k) and hands one entry at
+// a time to the whole wave with a lane read, so the inner loops wait on no memory for their coefficients; the
+// following 64 entries are requested a full register ahead of their use.
+struct CoeffStream {
+  const __attribute__((address_space(1))) float *src;
+  int base;
+  float cur, nxt;
+  __device__ __forceinline__ void start(const float *bank, int pos, int lane) {
+    src = (const __attribute__((address_space(1))) float *)bank;
+    base = pos;
+    cur = src[pos + lane];
+    nxt = src[pos + kWave + lane];
+  }
+  // afterwards base <= pos < base + 64
+  __device__ __forceinline__ void seek(int pos, int lane) {
+    if (pos >= base + 2 * kWave) {  // a long skip: start over at pos
+      base = pos;
+      cur = src[pos + lane];
+      nxt = src[pos + kWave + lane];
+    } else if (pos >= base + kWave) {
+      cur = nxt;
+      base += kWave;
+      nxt = src[base + kWave + lane];
+    }
+  }
+};
+
+__device__ __forceinline__ float lane_value(float v, int k) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), k));
+}
+
+// term(c) for the len <= 64 stream entries from pos on
+template <class F>
+__device__ __forceinline__ void for_coeffs(CoeffStream &cs, int pos, int len, int lane, F &&term) {
+  cs.seek(pos, lane);
+  // the position in the stream is the same for the whole wave; saying so keeps the loop counters scalar
+  const int k = __builtin_amdgcn_readfirstlane(pos - cs.base);
+  len = __builtin_amdgcn_readfirstlane(len);
+  const int first = min(len, kWave - k);
+  // four terms per trip: their LDS reads are independent, so the wave waits once for four of them
+  int t = 0;
+  for (; t + 4 <= first; t += 4) {
+    const float c0 = lane_value(cs.cur, k + t), c1 = lane_value(cs.cur, k + t + 1);
+    const float c2 = lane_value(cs.cur, k + t + 2), c3 = lane_value(cs.cur, k + t + 3);
+    term(c0);
+    term(c1);
+    term(c2);
+    term(c3);
+  }
+  for (; t < first; t++) term(lane_value(cs.cur, k + t));
+  for (; t < len; t++) term(lane_value(cs.nxt, t - first));
+}
+
 // ---- forward ------------------------------------------------------------------------------------------------------
 template <bool DIAG>
 __global__ void __launch_bounds__(256) staged_fwd_kernel(const StagedArgs) {
@@ -112,7 +167,7 @@ __global__ void __launch_bounds__(256) staged_fwd_kernel(const StagedArgs) {
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & (kWave - 1);
   const int W = blockDim.x >> 6;
   const TriplePtr triples = (TriplePtr)a->triples;
-  const CoeffPtr bank = (CoeffPtr)a->bank;
+  const float *bank = a->bank;
   const int ntriples = a->ntriples, offs_add = a->offs_add;
   const bool accumulate = a->accumulate != 0;
   int base = 0;
@@ -132,18 +187,19 @@ __global__ void __launch_bounds__(256) staged_fwd_kernel(const StagedArgs) {
       const int u = fc - cl * U;
       const int i = DIAG ? u : u / n2;
       const int j = DIAG ? u : u - i * n2;
-      const float2 *xb = xs + cl * xsize + tr->xoff + i;
-      const float2 *yb = ys + cl * ysize + tr->yoff + j;
+      const LdsC xb = (LdsC)xs + (cl * xsize + tr->xoff + i);
+      const LdsC yb = (LdsC)ys + (cl * ysize + tr->yoff + j);
       GlobalC *rp = (GlobalC *)R.ptr + (cell0 + cl) * R.sb + (tr->offs + offs_add + u);
-      CoeffPtr cp = bank + tr->cg_fwd;
+      int pos = tr->cg_fwd;
+      CoeffStream cs;
+      cs.start(bank, pos, lane);
       for (int m = -l; m <= l; m++) {
         const int m1lo = max(-l1, m - l2), m1hi = min(l1, m + l2);
-        const float2 *xp = xb + (m1lo + l1) * n1;
-        const float2 *yp = yb + (m - m1lo + l2) * n2;
+        LdsC xp = xb + (m1lo + l1) * n1;
+        LdsC yp = yb + (m - m1lo + l2) * n2;
         float ar = 0.f, ai = 0.f;
-        for (int m1 = m1lo; m1 <= m1hi; m1++) {
-          const float c = *cp++;
-          const float2 xv = *xp, yv = *yp;
+        for_coeffs(cs, pos, m1hi - m1lo + 1, lane, [&](float c) __attribute__((always_inline)) {
+          const v2f xv = *xp, yv = *yp;
           xp += n1;
           yp -= n2;
           const float pr = c * xv.x, pi = c * xv.y;  // (C x) y, the reference's order
@@ -151,7 +207,8 @@ __global__ void __launch_bounds__(256) staged_fwd_kernel(const StagedArgs) {
           ar = fmaf(-pi, yv.y, ar);
           ai = fmaf(pr, yv.y, ai);
           ai = fmaf(pi, yv.x, ai);
-        }
+        });
+        pos += m1hi - m1lo + 1;
         if (live) {
           GlobalC *dst = rp + (long long)(m + l) * R.sm;
           v2f o = {ar, ai};
@@ -177,6 +234,11 @@ struct RowRegs<16> {
     re[M] = r, im[M] = i;
   }
   __device__ __forceinline__ void get(int m, float &r, float &i) const { r = re[m], i = im[m]; }
+  __device__ __forceinline__ void add(int m, float r, float i) { re[m] += r, im[m] += i; }
+  template <int M>
+  __device__ __forceinline__ float2 row() const {
+    return make_float2(re[M], im[M]);
+  }
 };
 
 template <>
@@ -188,6 +250,11 @@ struct RowRegs<32> {
     re[M] = r, im[M] = i;
   }
   __device__ __forceinline__ void get(int m, float &r, float &i) const { r = re[m], i = im[m]; }
+  __device__ __forceinline__ void add(int m, float r, float i) { re[m] += r, im[m] += i; }
+  template <int M>
+  __device__ __forceinline__ float2 row() const {
+    return make_float2(re[M], im[M]);
+  }
 };
 
 template <int CAP>
@@ -195,6 +262,57 @@ constexpr int bwd_max_threads() {
   return CAP == 16 ? 1024 : 512;
 }
 
+// Rows w0 .. w0+CAP-1 of a lane's column of g into the registers.  Rows past the end repeat the last one (never
+// used): the loads stay unconditional, which keeps the register rows one straight chain of writes instead of a
+// merge of alternatives at every row.
+template <int CAP>
+__device__ __forceinline__ void load_window(RowRegs<CAP> &G, GlobalC *gp, int sm, int w0, int rows) {
+  static_for<CAP>([&](auto mc) __attribute__((always_inline)) {
+    constexpr int M = decltype(mc)::value;
+    const int row = min(w0 + M, rows - 1);
+    const v2f v = gp[(long long)row * sm];
+    G.template set<M>(v.x, v.y);
+  });
+}
+
+// One gradient's loop nest over the rows of g in the window [wlo, whi] (as values of m = m1 + m2):
+//     for every own row o:   emit(o + lo_own,  sum_q  C[o,q] g[o+q] conj(other[q]))
+// with (o, q) = (m1, m2) for the gradient of x and (m2, m1) for the gradient of y; `other` is the other operand's
+// part in LDS (rows nq apart) and pos the start of the matching coefficient stream.
+template <int CAP, class E>
+__device__ __forceinline__ void gradient_pass(const RowRegs<CAP> &G, int wlo, int whi, int l_own, int l_other, int l,
+                                              LdsC other, int nq, const float *bank, int pos, int lane, E &&emit) {
+  CoeffStream cs;
+  cs.start(bank, pos, lane);
+  for (int o = -l_own; o <= l_own; o++) {
+    const int qlo = max(-l_other, -l - o), qhi = min(l_other, l - o);
+    if (qlo > qhi) continue;
+    const int lo = max(qlo, wlo - o), hi = min(qhi, whi - o);
+    const int row_pos = pos + (lo - qlo);
+    pos += qhi - qlo + 1;
+    if (lo > hi) continue;
+    LdsC qp = other + (lo + l_other) * nq;
+    int k = o + lo - wlo;  // row inside the window
+    float ar = 0.f, ai = 0.f;
+    for_coeffs(cs, row_pos, hi - lo + 1, lane, [&](float c) __attribute__((always_inline)) {
+      float gr, gi;
+      G.get(k, gr, gi);
+      const v2f v = *qp;
+      k++;
+      qp += nq;
+      const float pr = c * gr, pi = c * gi;  // (C g) conj(other)
+      ar = fmaf(pr, v.x, ar);
+      ar = fmaf(pi, v.y, ar);
+      ai = fmaf(pi, v.x, ai);
+      ai = fmaf(-pr, v.y, ai);
+    });
+    emit(o + l_own, ar, ai);
+  }
+}
+
+// Both gradients from one pass over g; partial sums go to gradient images in LDS with float atomics.  This is the
+// form that accepts everything (any mix of channel counts, operand l up to the maximum); LDS float atomics are
+// slow on this hardware, so the striped kernel below is used whenever its conditions hold.
 template <int CAP, bool DIAG, bool WX, bool WY>
 __global__ void __launch_bounds__(bwd_max_threads<CAP>()) staged_bwd_kernel(const StagedArgs) {
   const ArgPtr a = kernel_args();
@@ -218,7 +336,7 @@ __global__ void __launch_bounds__(bwd_max_threads<CAP>()) staged_bwd_kernel(cons
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & (kWave - 1);
   const int W = blockDim.x >> 6;
   const TriplePtr triples = (TriplePtr)a->triples;
-  const CoeffPtr bank = (CoeffPtr)a->bank;
+  const float *bank = a->bank;
   const int ntriples = a->ntriples, offs_add = a->offs_add;
   RowRegs<CAP> G;
   G.clear();
@@ -246,81 +364,33 @@ __global__ void __launch_bounds__(bwd_max_threads<CAP>()) staged_bwd_kernel(cons
       // g is taken through the registers in windows of CAP rows (one window unless 2l+1 > CAP); each window adds
       // the terms whose row m1+m2 falls inside it
       for (int w0 = 0; w0 < rows; w0 += CAP) {
-        static_for<CAP>([&](auto mc) __attribute__((always_inline)) {
-          constexpr int M = decltype(mc)::value;
-          // rows past the end repeat the last one (never used): the loads stay unconditional, which keeps the
-          // register rows one straight chain of writes instead of a merge of alternatives at every row
-          const int row = min(w0 + M, rows - 1);
-          const v2f v = gp[(long long)row * P.sm];
-          G.template set<M>(v.x, v.y);
-        });
-        const int wlo = w0 - l, whi = w0 + CAP - 1 - l;  // the window as a range of m = m1 + m2
-
+        load_window<CAP>(G, gp, P.sm, w0, rows);
+        const int wlo = w0 - l, whi = w0 + CAP - 1 - l;
         if (WX) {
-          const float2 *yb = ys + cl * ysize + tr->yoff + j;
           LdsF *xa = (LdsF *)(xacc + cl * xsize + tr->xoff + i);
-          CoeffPtr cp = bank + tr->cg_back0;
-          for (int m1 = -l1; m1 <= l1; m1++) {
-            const int m2lo = max(-l2, -l - m1), m2hi = min(l2, l - m1);
-            if (m2lo > m2hi) continue;
-            const int lo = max(m2lo, wlo - m1), hi = min(m2hi, whi - m1);
-            CoeffPtr cq = cp + (lo - m2lo);
-            cp += m2hi - m2lo + 1;
-            if (lo > hi) continue;
-            const float2 *yp = yb + (lo + l2) * n2;
-            int k = m1 + lo - wlo;  // row inside the window
-            float2 acc[1] = {make_float2(0.f, 0.f)};
-            for (int m2 = lo; m2 <= hi; m2++, k++, yp += n2) {
-              const float c = *cq++;
-              float gr, gi;
-              G.get(k, gr, gi);
-              const float2 yv = *yp;
-              const float pr = c * gr, pi = c * gi;  // (C g) conj(y)
-              acc[0].x = fmaf(pr, yv.x, acc[0].x);
-              acc[0].x = fmaf(pi, yv.y, acc[0].x);
-              acc[0].y = fmaf(pi, yv.x, acc[0].y);
-              acc[0].y = fmaf(-pr, yv.y, acc[0].y);
-            }
-            if (!DIAG) group_sum(acc, n2);
-            if (live && (DIAG || j == 0)) {
-              LdsF *dst = xa + 2 * (m1 + l1) * n1;
-              __hip_atomic_fetch_add(dst, acc[0].x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-              __hip_atomic_fetch_add(dst + 1, acc[0].y, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-            }
-          }
+          gradient_pass<CAP>(G, wlo, whi, l1, l2, l, (LdsC)ys + (cl * ysize + tr->yoff + j), n2, bank, tr->cg_back0,
+                             lane, [&](int row, float ar, float ai) __attribute__((always_inline)) {
+                               float2 acc[1] = {make_float2(ar, ai)};
+                               if (!DIAG) group_sum(acc, n2);
+                               if (live && (DIAG || j == 0)) {
+                                 LdsF *dst = xa + 2 * row * n1;
+                                 __hip_atomic_fetch_add(dst, acc[0].x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                                 __hip_atomic_fetch_add(dst + 1, acc[0].y, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                               }
+                             });
         }
         if (WY) {
-          const float2 *xb = xs + cl * xsize + tr->xoff + i;
           LdsF *ya = (LdsF *)(yacc + cl * ysize + tr->yoff + j);
-          CoeffPtr cp = bank + tr->cg_back1;
-          for (int m2 = -l2; m2 <= l2; m2++) {
-            const int m1lo = max(-l1, -l - m2), m1hi = min(l1, l - m2);
-            if (m1lo > m1hi) continue;
-            const int lo = max(m1lo, wlo - m2), hi = min(m1hi, whi - m2);
-            CoeffPtr cq = cp + (lo - m1lo);
-            cp += m1hi - m1lo + 1;
-            if (lo > hi) continue;
-            const float2 *xp = xb + (lo + l1) * n1;
-            int k = lo + m2 - wlo;
-            float2 acc[1] = {make_float2(0.f, 0.f)};
-            for (int m1 = lo; m1 <= hi; m1++, k++, xp += n1) {
-              const float c = *cq++;
-              float gr, gi;
-              G.get(k, gr, gi);
-              const float2 xv = *xp;
-              const float pr = c * gr, pi = c * gi;  // (C g) conj(x)
-              acc[0].x = fmaf(pr, xv.x, acc[0].x);
-              acc[0].x = fmaf(pi, xv.y, acc[0].x);
-              acc[0].y = fmaf(pi, xv.x, acc[0].y);
-              acc[0].y = fmaf(-pr, xv.y, acc[0].y);
-            }
-            if (!DIAG) stride_sum(acc, n2, span);
-            if (live && (DIAG || (u & (span - 1)) < n2)) {
-              LdsF *dst = ya + 2 * (m2 + l2) * n2;
-              __hip_atomic_fetch_add(dst, acc[0].x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-              __hip_atomic_fetch_add(dst + 1, acc[0].y, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-            }
-          }
+          gradient_pass<CAP>(G, wlo, whi, l2, l1, l, (LdsC)xs + (cl * xsize + tr->xoff + i), n1, bank, tr->cg_back1,
+                             lane, [&](int row, float ar, float ai) __attribute__((always_inline)) {
+                               float2 acc[1] = {make_float2(ar, ai)};
+                               if (!DIAG) stride_sum(acc, n2, span);
+                               if (live && (DIAG || (u & (span - 1)) < n2)) {
+                                 LdsF *dst = ya + 2 * row * n2;
+                                 __hip_atomic_fetch_add(dst, acc[0].x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                                 __hip_atomic_fetch_add(dst + 1, acc[0].y, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                               }
+                             });
         }
       }
     }
@@ -333,6 +403,133 @@ __global__ void __launch_bounds__(bwd_max_threads<CAP>()) staged_bwd_kernel(cons
   } else {
     if (WX) copy_image<1>(a->xg, a->xrows, a->nx, xacc, xsize, cell0, ncell);
     if (WY) copy_image<1>(a->yg, a->yrows, a->ny, yacc, ysize, cell0, ncell);
+  }
+}
+
+// ---- backward, one gradient per launch, sums kept in registers ---------------------------------------------------------
+// ROLE 0 computes the gradient of x, ROLE 1 that of y.  All triples that feed one part of that gradient form a
+// stripe; a wave takes a (stripe, 64 channel slots) unit, walks the stripe's triples and keeps the part's rows in a
+// second set of register rows (again indexed with a wave-uniform run-time row), so nothing is shared between waves:
+// no atomics, no gradient image in LDS, a fixed summation order.  The sums over the lanes that share i (resp. j)
+// are taken once per unit, on the finished rows, and the rows are stored straight to memory.  LDS holds only the
+// other operand.  The price is that each launch reads g, i.e. g is read twice for the two gradients.
+// Conditions (checked by the host): inside a stripe the other operand's channel count does not change, so a
+// lane's (i, j) stays the same across the stripe's triples; own l at most (CAP-1)/2.
+// Units are handed out through a counter in LDS, heaviest stripes (largest l) first.
+constexpr int kStripeHeader = 2;  // complex elements in front of the operand image (holds the unit counter)
+
+template <int CAP, bool DIAG, int ROLE>
+__global__ void __launch_bounds__(256) staged_stripe_kernel(const StagedArgs) {
+  const ArgPtr a = kernel_args();
+  extern __shared__ float2 staged_lds[];
+  // the unit counter sits in front of the image, in the dynamic allocation: with any static LDS the kernel could
+  // no longer ask for the full 160 KB
+  int &next_unit = *reinterpret_cast<int *>(staged_lds);
+  const int cpb = a->cpb;
+  const int osize = ROLE == 0 ? a->ysize : a->xsize;  // the other operand's image
+  float2 *os = staged_lds + kStripeHeader;
+  const long long cell0 = (long long)blockIdx.x * cpb;
+  const long long left = a->ncells - cell0;
+  const int ncell = left < cpb ? (int)left : cpb;
+  if (ROLE == 0) copy_image<0>(a->y, a->yrows, a->ny, os, osize, cell0, ncell);
+  else copy_image<0>(a->x, a->xrows, a->nx, os, osize, cell0, ncell);
+  if (threadIdx.x == 0) next_unit = 0;
+  __syncthreads();
+
+  const int lane = threadIdx.x & (kWave - 1);
+  const TriplePtr triples = (TriplePtr)a->triples;
+  const float *bank = a->bank;
+  const int offs_add = a->offs_add;
+  const bool accumulate = a->accumulate != 0;
+  const int nstripes = ROLE == 0 ? a->nx : a->ny;
+  const IntPtr table = (IntPtr)a->stripes + (ROLE == 0 ? 0 : 3 * a->nx);  // (first, count, log2 slots) per stripe
+  const IntPtr order = (IntPtr)a->stripes + 3 * (a->nx + a->ny) + (ROLE == 0 ? 0 : a->ntriples);
+  RowRegs<CAP> G, A;
+  G.clear();
+  for (;;) {
+    int idx = 0;
+    if (lane == 0) idx = __hip_atomic_fetch_add(&next_unit, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    idx = __builtin_amdgcn_readfirstlane(idx);
+    // which stripe: the last (largest l) first
+    int k = nstripes - 1, log2_u = 0;
+    for (; k >= 0; k--) {
+      log2_u = table[3 * k + 2];
+      const int units = log2_u >= 6 ? cpb : (((cpb << log2_u) + kWave - 1) >> 6);
+      if (idx < units) break;
+      idx -= units;
+    }
+    if (k < 0) break;  // every unit has been taken: the counter only grows, so every wave gets here
+    const int first = table[3 * k], count = table[3 * k + 1];
+    const FastPart OWN = load_part((ROLE == 0 ? a->xg : a->yg) + k);
+    const int own_rows = ROLE == 0 ? a->xrows[k] : a->yrows[k];
+    const int nsub = log2_u >= 6 ? (1 << (log2_u - 6)) : 1;  // runs of 64 slots inside one cell
+    const int span = log2_u < 6 ? (1 << log2_u) : kWave;
+    // channel count of the other operand, the same for the whole stripe (1 for a stripe without triples)
+    int n_other = 1;
+    if (count > 0) {
+      const TriplePtr t0 = triples + order[first];
+      n_other = ROLE == 0 ? t0->n2 : t0->n1;
+    }
+    const int n_own = OWN.n;
+    const int n1 = ROLE == 0 ? n_own : n_other, n2 = ROLE == 0 ? n_other : n_own;
+    const int lg_n2 = DIAG ? 0 : 31 - __clz(n2);
+    A.clear();
+    for (int sub = 0; sub < nsub; sub++) {
+      const int flat = log2_u >= 6 ? ((idx << log2_u) + (sub << 6) + lane) : ((idx << 6) + lane);
+      int cl = flat >> log2_u;
+      const int u = flat & ((1 << log2_u) - 1);
+      const bool live = cl < ncell;
+      if (!live) cl = ncell - 1;  // dead lanes read valid memory and never store
+      const int i = DIAG ? u : (u >> lg_n2);
+      const int j = DIAG ? u : (u & (n2 - 1));
+      for (int t = 0; t < count; t++) {
+        const TriplePtr tr = triples + order[first + t];
+        const int l1 = tr->l1, l2 = tr->l2, l = tr->l;
+        const FastPart P = load_part(a->r + tr->ri);
+        GlobalC *gp = (GlobalC *)P.ptr + (cell0 + cl) * P.sb + (tr->offs + offs_add + u);
+        const int rows = 2 * l + 1;
+        for (int w0 = 0; w0 < rows; w0 += CAP) {
+          load_window<CAP>(G, gp, P.sm, w0, rows);
+          const int wlo = w0 - l, whi = w0 + CAP - 1 - l;
+          auto add_row = [&](int row, float ar, float ai) __attribute__((always_inline)) { A.add(row, ar, ai); };
+          if (ROLE == 0)
+            gradient_pass<CAP>(G, wlo, whi, l1, l2, l, (LdsC)os + (cl * osize + tr->yoff + j), n2, bank, tr->cg_back0,
+                               lane, add_row);
+          else
+            gradient_pass<CAP>(G, wlo, whi, l2, l1, l, (LdsC)os + (cl * osize + tr->xoff + i), n1, bank, tr->cg_back1,
+                               lane, add_row);
+        }
+      }
+      // the gradient of x is complete for this run's i; the gradient of y still sums over the other runs' i
+      if (ROLE == 1 && sub + 1 < nsub) continue;
+      float2 out[CAP];
+      static_for<CAP>([&](auto mc) __attribute__((always_inline)) {
+        constexpr int M = decltype(mc)::value;
+        out[M] = A.template row<M>();
+      });
+      bool writer = live;
+      if (!DIAG) {
+        if (ROLE == 0) {
+          group_sum(out, n2);
+          writer = live && j == 0;
+        } else {
+          stride_sum(out, n2, span);
+          writer = live && (u & (span - 1)) < n2;
+        }
+      }
+      GlobalC *dst = (GlobalC *)OWN.ptr + (cell0 + cl) * OWN.sb + (ROLE == 0 ? i : j);
+      if (writer) {
+        static_for<CAP>([&](auto mc) __attribute__((always_inline)) {
+          constexpr int M = decltype(mc)::value;
+          if (M < own_rows) {
+            v2f o = {out[M].x, out[M].y};
+            if (accumulate) o += dst[(long long)M * OWN.sm];
+            dst[(long long)M * OWN.sm] = o;
+          }
+        });
+      }
+      A.clear();
+    }
   }
 }
 
@@ -374,6 +571,20 @@ int launch_bwd_caps(const StagedArgs &a, bool wx, bool wy, int cap, int threads,
   return GELIB_HIP_ERR_ARG;
 }
 
+template <int CAP, bool DIAG, int ROLE>
+int launch_stripe_variant(const StagedArgs &a, int nblocks, size_t lds, hipStream_t s) {
+  static bool attr_set = false;
+  return launch(staged_stripe_kernel<CAP, DIAG, ROLE>, a, 256, nblocks, lds, s, &attr_set);
+}
+
+template <int CAP>
+int launch_stripe_cap(const StagedArgs &a, bool diag, int role, int nblocks, size_t lds, hipStream_t s) {
+  if (diag) return role == 0 ? launch_stripe_variant<CAP, true, 0>(a, nblocks, lds, s)
+                             : launch_stripe_variant<CAP, true, 1>(a, nblocks, lds, s);
+  return role == 0 ? launch_stripe_variant<CAP, false, 0>(a, nblocks, lds, s)
+                   : launch_stripe_variant<CAP, false, 1>(a, nblocks, lds, s);
+}
+
 }  // namespace
 
 int launch_staged_fwd(const StagedArgs &a, bool diag, int nblocks, size_t lds_bytes, hipStream_t s) {
@@ -388,6 +599,15 @@ int launch_staged_bwd(const StagedArgs &a, bool diag, bool want_x, bool want_y, 
   if (lds_bytes > (size_t)kMaxDynamicLds || (!want_x && !want_y)) return GELIB_HIP_ERR_ARG;
   if (diag) return launch_bwd_caps<true>(a, want_x, want_y, cap, threads, nblocks, lds_bytes, s);
   return launch_bwd_caps<false>(a, want_x, want_y, cap, threads, nblocks, lds_bytes, s);
+}
+
+int launch_staged_stripe(const StagedArgs &a, bool diag, int role, int cap, int nblocks, size_t lds_bytes,
+                         hipStream_t s) {
+  lds_bytes += kStripeHeader * sizeof(float2);
+  if (lds_bytes > (size_t)kMaxDynamicLds || (role != 0 && role != 1)) return GELIB_HIP_ERR_ARG;
+  if (cap == 16) return launch_stripe_cap<16>(a, diag, role, nblocks, lds_bytes, s);
+  if (cap == 32) return launch_stripe_cap<32>(a, diag, role, nblocks, lds_bytes, s);
+  return GELIB_HIP_ERR_ARG;
 }
 
 }  // namespace gelib_hip

@@ -14,6 +14,7 @@ namespace {
 
 int g_fwd_enable = 1;
 int g_bwd_enable = 1;
+int g_bwd_stripes = 1;       // striped (register-accumulating) backward kernels: 0 never, 1 where they pay, 2 wherever they apply
 int g_bwd_threads = 0;       // 0 = choose from the LDS footprint, else force 256 / 512 / 1024
 int g_fwd_lds_target = 32 * 1024;  // LDS up to which a forward block takes more cells to fill its waves
 int g_bwd_lds_target = 40 * 1024;
@@ -24,8 +25,12 @@ struct DevicePlan {
   std::vector<StagedTriple> triples;
   StagedTriple *d_triples = nullptr;
   float *d_bank = nullptr;
+  int *d_stripes = nullptr;
   int xsize = 0, ysize = 0;
   int lmax_out = 0;
+  bool stripes_ok = false;   // the striped backward kernels apply
+  int stripe_cap = 0;        // register rows they need (16 or 32)
+  std::vector<int> stripes;  // host copy of the table
 };
 
 std::mutex g_plan_mutex;
@@ -86,19 +91,60 @@ int get_plan(bool diag, const std::vector<VecTriple> &triples, const std::vector
     plan.lmax_out = std::max(plan.lmax_out, t.l);
     plan.triples.push_back(r);
   }
-  bank.resize(bank.size() + 16, 0.f);  // the coefficient stream may be read a few entries ahead
+  bank.resize(bank.size() + 4 * kWave, 0.f);  // the kernels read the stream up to three registers of lanes ahead
+  // stripes: the triples that feed one x part (resp. one y part)
+  {
+    const int nx = (int)xs.size(), ny = (int)ys.size(), nt = (int)plan.triples.size();
+    std::vector<int> &tb = plan.stripes;
+    tb.assign(3 * (nx + ny) + 2 * nt, 0);
+    bool ok = true;
+    int lown = 0;
+    for (int role = 0; role < 2; role++) {
+      const int np = role == 0 ? nx : ny;
+      int *table = tb.data() + (role == 0 ? 0 : 3 * nx);
+      int *order = tb.data() + 3 * (nx + ny) + (role == 0 ? 0 : nt);
+      int filled = 0;
+      for (int k = 0; k < np; k++) {
+        const int n_own = role == 0 ? xs[k].second : ys[k].second;
+        lown = std::max(lown, role == 0 ? xs[k].first : ys[k].first);
+        table[3 * k] = filled;
+        int n_other = -1;
+        for (int t = 0; t < nt; t++) {
+          const StagedTriple &r = plan.triples[t];
+          if ((role == 0 ? r.xi : r.yi) != k) continue;
+          order[filled++] = t;
+          const int no = role == 0 ? r.n2 : r.n1;
+          if (n_other >= 0 && no != n_other) ok = false;  // a lane's (i, j) would change inside the stripe
+          n_other = no;
+        }
+        table[3 * k + 1] = filled - table[3 * k];
+        const long long U = diag ? n_own : (long long)n_own * std::max(1, n_other);
+        if (!is_pow2(n_own) || (n_other > 0 && !is_pow2(n_other)) || U > (1 << 20)) ok = false;
+        table[3 * k + 2] = ok ? ilog2((int)U) : 0;
+      }
+    }
+    if (!diag)
+      for (auto &v : ys)
+        if (v.second > kWave) ok = false;
+    if (2 * lown + 1 > 32) ok = false;
+    plan.stripes_ok = ok;
+    plan.stripe_cap = 2 * lown + 1 <= 16 ? 16 : 32;
+  }
   const size_t tri_bytes = plan.triples.size() * sizeof(StagedTriple);
   const size_t bank_bytes = bank.size() * sizeof(float);
+  const size_t stripe_bytes = plan.stripes.size() * sizeof(int);
   char *d = nullptr;
-  GELIB_HIP_TRY(hipMalloc((void **)&d, tri_bytes + bank_bytes));
+  GELIB_HIP_TRY(hipMalloc((void **)&d, tri_bytes + bank_bytes + stripe_bytes));
   hipError_t e = hipMemcpy(d, plan.triples.data(), tri_bytes, hipMemcpyHostToDevice);
   if (e == hipSuccess) e = hipMemcpy(d + tri_bytes, bank.data(), bank_bytes, hipMemcpyHostToDevice);
+  if (e == hipSuccess) e = hipMemcpy(d + tri_bytes + bank_bytes, plan.stripes.data(), stripe_bytes, hipMemcpyHostToDevice);
   if (e != hipSuccess) {
     (void)hipFree(d);
     return record_hip_error(e, "hipMemcpy(staged plan)");
   }
   plan.d_triples = (StagedTriple *)d;
   plan.d_bank = (float *)(d + tri_bytes);
+  plan.d_stripes = (int *)(d + tri_bytes + bank_bytes);
   auto ins = g_plans.emplace(key, std::move(plan));
   *out = &ins.first->second;
   return GELIB_HIP_OK;
@@ -124,6 +170,7 @@ void fill_args(StagedArgs &a, const DevicePlan &plan, const FastLists &f, const 
   for (size_t i = 0; i < f.yg.size(); i++) a.yg[i] = f.yg[i];
   a.triples = plan.d_triples;
   a.bank = plan.d_bank;
+  a.stripes = plan.d_stripes;
   a.ncells = ncells;
   a.ntriples = (int)plan.triples.size();
   a.nx = (int)xs.size();
@@ -188,6 +235,37 @@ int run_bwd(bool diag, const std::vector<VecTriple> &triples, const std::vector<
   const DevicePlan *plan = nullptr;
   int rc = get_plan(diag, triples, xs, ys, rls, &plan);
   if (rc) return rc;
+  // The striped kernels win where rows are short (small l: an atomic per handful of terms in the other form); with
+  // 32 register rows for g and 32 for the sums they run at low occupancy and lose to the single-pass form.
+  const bool stripes_wanted = g_bwd_stripes == 2 || (g_bwd_stripes == 1 && plan->stripe_cap == 16);
+  if (stripes_wanted && plan->stripes_ok && 8LL * std::max(plan->xsize, plan->ysize) + 64 <= kLdsLimit) {
+    // one launch per wanted gradient; LDS holds the other operand only
+    StagedArgs a;
+    fill_args(a, *plan, f, xs, ys, ncells, offs_add, accumulate);
+    for (int role = 0; role < 2; role++) {
+      if (role == 0 ? !want_x : !want_y) continue;
+      const long long cell_bytes = 8LL * (role == 0 ? plan->ysize : plan->xsize);
+      const int np = role == 0 ? (int)xs.size() : (int)ys.size();
+      const int *table = plan->stripes.data() + (role == 0 ? 0 : 3 * (int)xs.size());
+      auto units = [&](long long cpb) {
+        long long n = 0;
+        for (int k = 0; k < np; k++) {
+          const int lg = table[3 * k + 2];
+          n += lg >= 6 ? cpb : (((cpb << lg) + kWave - 1) >> 6);
+        }
+        return n;
+      };
+      long long cpb = 1;
+      while (cpb * 2 <= ncells && cell_bytes * cpb * 2 <= g_bwd_lds_target && units(cpb) < 16) cpb *= 2;
+      a.cpb = (int)cpb;
+      const long long nblocks = (ncells + cpb - 1) / cpb;
+      if (nblocks > 0x7fffffffLL) return GELIB_HIP_ERR_ARG;
+      rc = launch_staged_stripe(a, diag, role, plan->stripe_cap, (int)nblocks, (size_t)(cell_bytes * cpb), s);
+      if (rc) return rc;
+    }
+    *used = 1;
+    return GELIB_HIP_OK;
+  }
   const long long cell_bytes = 16LL * (plan->xsize + plan->ysize);  // operands + gradient images
   if (cell_bytes > kLdsLimit) return GELIB_HIP_OK;
   long long cpb = 1;
@@ -278,6 +356,10 @@ int staged_set_option(const char *name, int value) {
   }
   if (!std::strcmp(name, "staged_bwd")) {
     g_bwd_enable = value;
+    return GELIB_HIP_OK;
+  }
+  if (!std::strcmp(name, "staged_bwd_stripes")) {
+    g_bwd_stripes = value;
     return GELIB_HIP_OK;
   }
   if (!std::strcmp(name, "staged_bwd_threads")) {

@@ -1,8 +1,8 @@
 """GPU parity of the any-l ("staged") kernels: operand l above 4, where the unrolled small-l kernels do not apply.
 
 Each case checks the kernel family that ran (gelib_hip_last_path() == 3) and compares with the CPU oracle in
-float32 and float64, as the other GPU tests do.  The backward pass adds partial sums into LDS images with float
-atomics, so its last bits can differ from run to run; the tolerance of assert_parity covers that.
+float32 and float64, as the other GPU tests do.  One of the two backward forms adds partial sums into LDS images with
+float atomics, so its last bits can differ from run to run; the tolerance of assert_parity covers that.
 """
 import numpy as np
 import pytest
@@ -17,14 +17,18 @@ torch = pytest.importorskip("torch")
 STAGED = 3
 
 
-@pytest.fixture(scope="module")
-def cabi():
+@pytest.fixture(scope="module", params=["striped", "atomic"])
+def cabi(request):
+    """Both backward forms of the family: one gradient per launch with sums in registers (the default where its
+    conditions hold), and both gradients in one launch with LDS float atomics."""
     assert torch.cuda.is_available(), "GPU tests need a GPU"
     from gelib_amd import cabi as c
     c.lib()
     c.set_option("force_generic", 0)
+    c.set_option("staged_bwd_stripes", 2 if request.param == "striped" else 0)
     yield c
     c.set_option("staged_bwd_threads", 0)
+    c.set_option("staged_bwd_stripes", 1)
 
 
 def c128(L):
@@ -76,6 +80,8 @@ VEC_CASES = [
     (7, {5: 4, 6: 2}, {0: 2, 7: 4}, -1),                             # l up to 13: 27 rows, the 32-row variant
     (70, {5: 1}, {6: 1}, -1),                                        # one channel: many cells share a run
     (2, {6: 16}, {5: 16}, 8),                                        # 256 slots per cell: several runs per cell
+    (3, {5: 2, 6: 4}, {5: 4, 6: 8}, 7),                              # channel counts differ between parts
+    (2, {12: 2}, {3: 4}, -1),                                        # own l = 12: 25 rows, the 32-row variant
 ]
 
 

@@ -47,7 +47,9 @@ struct StagedArgs {
   int xrows[kMaxParts], yrows[kMaxParts];
 };
 
-int launch_staged_fwd(const StagedArgs &a, bool diag, int nblocks, size_t lds_bytes, hipStream_t s);
+// tile: adjacent output channels per lane (1, 2 or 4); threads: a multiple of 64 up to 1024
+int launch_staged_fwd(const StagedArgs &a, bool diag, int tile, int threads, int nblocks, size_t lds_bytes,
+                      hipStream_t s);
 // cap: rows of g a lane keeps in registers (16 or 32); threads: 256, 512 or 1024 (1024 only with cap 16)
 int launch_staged_bwd(const StagedArgs &a, bool diag, bool want_x, bool want_y, int cap, int threads, int nblocks,
                       size_t lds_bytes, hipStream_t s);

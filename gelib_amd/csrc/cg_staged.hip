@@ -150,8 +150,53 @@ __device__ __forceinline__ void for_coeffs(CoeffStream &cs, int pos, int len, in
 }
 
 // ---- forward ------------------------------------------------------------------------------------------------------
-template <bool DIAG>
-__global__ void __launch_bounds__(256) staged_fwd_kernel(const StagedArgs) {
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+// TILE adjacent complex numbers from LDS / to global memory as 16-byte accesses
+template <int TILE>
+struct CTile {
+  v2f v[TILE];
+};
+
+template <int TILE>
+__device__ __forceinline__ CTile<TILE> lds_tile(LdsC p) {
+  CTile<TILE> t;
+  if constexpr (TILE == 1) {
+    t.v[0] = *p;
+  } else {
+    static_for<TILE / 2>([&](auto hc) __attribute__((always_inline)) {
+      constexpr int h = decltype(hc)::value;
+      const v4f q = ((const __attribute__((address_space(3))) v4f *)p)[h];
+      t.v[2 * h] = v2f{q.x, q.y};
+      t.v[2 * h + 1] = v2f{q.z, q.w};
+    });
+  }
+  return t;
+}
+
+template <int TILE>
+__device__ __forceinline__ void store_tile(GlobalC *dst, const CTile<TILE> &t, bool accumulate) {
+  if constexpr (TILE == 1) {
+    v2f o = t.v[0];
+    if (accumulate) o += *dst;
+    *dst = o;
+  } else {
+    static_for<TILE / 2>([&](auto hc) __attribute__((always_inline)) {
+      constexpr int h = decltype(hc)::value;
+      __attribute__((address_space(1))) v4f *d4 = (__attribute__((address_space(1))) v4f *)dst + h;
+      v4f o = {t.v[2 * h].x, t.v[2 * h].y, t.v[2 * h + 1].x, t.v[2 * h + 1].y};
+      if (accumulate) o += *d4;
+      *d4 = o;
+    });
+  }
+}
+
+// A lane owns TILE adjacent output channels (the same i and TILE adjacent j; for Diag TILE adjacent channels), so
+// the per-row and per-term bookkeeping -- which is most of the instructions when rows are short -- is shared by
+// TILE complex products.  The host picks TILE (1, 2 or 4) so that every channel count and offset is a multiple of
+// it and the output pointers are 8*TILE-byte aligned.
+template <bool DIAG, int TILE>
+__global__ void __launch_bounds__(1024) staged_fwd_kernel(const StagedArgs) {
   const ArgPtr a = kernel_args();
   extern __shared__ float2 staged_lds[];
   const int cpb = a->cpb, xsize = a->xsize, ysize = a->ysize;
@@ -173,7 +218,7 @@ __global__ void __launch_bounds__(256) staged_fwd_kernel(const StagedArgs) {
   int base = 0;
   for (int t = 0; t < ntriples; t++) {
     const TriplePtr tr = triples + t;
-    const int U = tr->u;
+    const int U = tr->u / TILE;  // tile slots per cell
     const int nruns = (cpb * U + kWave - 1) >> 6;
     const int first = first_run(base, wave, W, nruns);
     if (first >= nruns) continue;
@@ -184,7 +229,7 @@ __global__ void __launch_bounds__(256) staged_fwd_kernel(const StagedArgs) {
       const bool live = flat < ncell * U;
       const int fc = live ? flat : 0;  // dead lanes compute on valid data and never store
       const int cl = fc / U;
-      const int u = fc - cl * U;
+      const int u = (fc - cl * U) * TILE;
       const int i = DIAG ? u : u / n2;
       const int j = DIAG ? u : u - i * n2;
       const LdsC xb = (LdsC)xs + (cl * xsize + tr->xoff + i);
@@ -197,24 +242,26 @@ __global__ void __launch_bounds__(256) staged_fwd_kernel(const StagedArgs) {
         const int m1lo = max(-l1, m - l2), m1hi = min(l1, m + l2);
         LdsC xp = xb + (m1lo + l1) * n1;
         LdsC yp = yb + (m - m1lo + l2) * n2;
-        float ar = 0.f, ai = 0.f;
+        CTile<TILE> acc;
+#pragma unroll
+        for (int k = 0; k < TILE; k++) acc.v[k] = v2f{0.f, 0.f};
         for_coeffs(cs, pos, m1hi - m1lo + 1, lane, [&](float c) __attribute__((always_inline)) {
-          const v2f xv = *xp, yv = *yp;
+          const CTile<DIAG ? TILE : 1> xt = lds_tile<DIAG ? TILE : 1>(xp);
+          const CTile<TILE> yt = lds_tile<TILE>(yp);
           xp += n1;
           yp -= n2;
-          const float pr = c * xv.x, pi = c * xv.y;  // (C x) y, the reference's order
-          ar = fmaf(pr, yv.x, ar);
-          ar = fmaf(-pi, yv.y, ar);
-          ai = fmaf(pr, yv.y, ai);
-          ai = fmaf(pi, yv.x, ai);
+#pragma unroll
+          for (int k = 0; k < TILE; k++) {
+            const v2f xv = xt.v[DIAG ? k : 0], yv = yt.v[k];
+            const float pr = c * xv.x, pi = c * xv.y;  // (C x) y, the reference's order
+            acc.v[k].x = fmaf(pr, yv.x, acc.v[k].x);
+            acc.v[k].x = fmaf(-pi, yv.y, acc.v[k].x);
+            acc.v[k].y = fmaf(pr, yv.y, acc.v[k].y);
+            acc.v[k].y = fmaf(pi, yv.x, acc.v[k].y);
+          }
         });
         pos += m1hi - m1lo + 1;
-        if (live) {
-          GlobalC *dst = rp + (long long)(m + l) * R.sm;
-          v2f o = {ar, ai};
-          if (accumulate) o += *dst;
-          *dst = o;
-        }
+        if (live) store_tile<TILE>(rp + (long long)(m + l) * R.sm, acc, accumulate);
       }
     }
   }
@@ -587,11 +634,20 @@ int launch_stripe_cap(const StagedArgs &a, bool diag, int role, int nblocks, siz
 
 }  // namespace
 
-int launch_staged_fwd(const StagedArgs &a, bool diag, int nblocks, size_t lds_bytes, hipStream_t s) {
-  static bool attr_cg = false, attr_diag = false;
-  if (lds_bytes > (size_t)kMaxDynamicLds) return GELIB_HIP_ERR_ARG;
-  if (diag) return launch(staged_fwd_kernel<true>, a, 256, nblocks, lds_bytes, s, &attr_diag);
-  return launch(staged_fwd_kernel<false>, a, 256, nblocks, lds_bytes, s, &attr_cg);
+int launch_staged_fwd(const StagedArgs &a, bool diag, int tile, int threads, int nblocks, size_t lds_bytes,
+                      hipStream_t s) {
+  static bool attr[6] = {false, false, false, false, false, false};
+  if (lds_bytes > (size_t)kMaxDynamicLds || threads < 64 || threads > 1024 || threads % 64) return GELIB_HIP_ERR_ARG;
+  if (diag) {
+    if (tile == 4) return launch(staged_fwd_kernel<true, 4>, a, threads, nblocks, lds_bytes, s, &attr[0]);
+    if (tile == 2) return launch(staged_fwd_kernel<true, 2>, a, threads, nblocks, lds_bytes, s, &attr[1]);
+    if (tile == 1) return launch(staged_fwd_kernel<true, 1>, a, threads, nblocks, lds_bytes, s, &attr[2]);
+  } else {
+    if (tile == 4) return launch(staged_fwd_kernel<false, 4>, a, threads, nblocks, lds_bytes, s, &attr[3]);
+    if (tile == 2) return launch(staged_fwd_kernel<false, 2>, a, threads, nblocks, lds_bytes, s, &attr[4]);
+    if (tile == 1) return launch(staged_fwd_kernel<false, 1>, a, threads, nblocks, lds_bytes, s, &attr[5]);
+  }
+  return GELIB_HIP_ERR_ARG;
 }
 
 int launch_staged_bwd(const StagedArgs &a, bool diag, bool want_x, bool want_y, int cap, int threads, int nblocks,

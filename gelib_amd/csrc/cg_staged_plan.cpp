@@ -1,6 +1,7 @@
 // Host side of the staged (any-l) kernels: eligibility, the per-signature device tables (triples + compact
 // coefficient streams) and the per-call launch shape.
 #include <algorithm>
+#include <cstdint>
 #include <cstring>
 #include <map>
 #include <mutex>
@@ -14,6 +15,8 @@ namespace {
 
 int g_fwd_enable = 1;
 int g_bwd_enable = 1;
+int g_fwd_tile = 0;           // 0 = widest tile that fits, else force 1 / 2 / 4 (still subject to divisibility)
+int g_fwd_threads = 0;        // 0 = choose from the LDS footprint
 int g_bwd_stripes = 1;       // striped (register-accumulating) backward kernels: 0 never, 1 where they pay, 2 wherever they apply
 int g_bwd_threads = 0;       // 0 = choose from the LDS footprint, else force 256 / 512 / 1024
 int g_fwd_lds_target = 32 * 1024;  // LDS up to which a forward block takes more cells to fill its waves
@@ -205,15 +208,51 @@ int run_fwd(bool diag, const std::vector<VecTriple> &triples, const std::vector<
   int rc = get_plan(diag, triples, xs, ys, rls, &plan);
   if (rc) return rc;
   const long long cell_bytes = 8LL * (plan->xsize + plan->ysize);
+  // Channels per lane: the widest tile that divides every channel count and offset and keeps the 16-byte
+  // accesses aligned, provided enough cells fit in LDS to fill a wave with tile slots.
+  auto tile_ok = [&](int tile) {
+    if (tile == 1) return true;
+    if (offs_add % tile || plan->xsize % tile || plan->ysize % tile) return false;  // images stay 16-byte aligned
+    for (auto &t : plan->triples) {
+      if ((diag ? t.n1 : t.n2) % tile || t.offs % tile) return false;
+      if (diag && (t.xoff % tile || t.yoff % tile)) return false;
+      if (t.yoff % tile) return false;
+    }
+    for (auto &r : f.r)
+      if (((uintptr_t)r.ptr % (8 * tile)) || r.sb % tile || r.sm % tile) return false;
+    return true;
+  };
+  int tile = 4, threads = 256;
   long long cpb = 1;
-  // more cells per block while the block's waves would otherwise idle and the image stays small
-  while (cpb * 2 <= ncells && cell_bytes * cpb * 2 <= g_fwd_lds_target && units_per_block(*plan, cpb) < 16) cpb *= 2;
+  if (g_fwd_tile == 1 || g_fwd_tile == 2 || g_fwd_tile == 4) tile = g_fwd_tile;
+  for (;; tile >>= 1) {
+    if (!tile_ok(tile)) continue;
+    long long slots_min = 1 << 30;
+    for (auto &t : plan->triples) slots_min = std::min<long long>(slots_min, t.u / tile);
+    auto units = [&](long long c) {
+      long long n = 0;
+      for (auto &t : plan->triples) n += (c * (t.u / tile) + kWave - 1) / kWave;
+      return n;
+    };
+    cpb = 1;
+    // first fill the lanes of a run, then give the block's waves enough runs
+    while (cpb * 2 <= ncells && cpb * slots_min < kWave && cell_bytes * cpb * 2 <= 110 * 1024) cpb *= 2;
+    while (cpb * 2 <= ncells && cell_bytes * cpb * 2 <= g_fwd_lds_target && units(cpb) < 16) cpb *= 2;
+    if (tile > 1 && cpb * slots_min < kWave && cpb < ncells) continue;  // lanes would idle: try a narrower tile
+    // as many waves per CU as the LDS footprint leaves room for, without more waves than runs
+    const long long blocks_per_cu = std::max<long long>(1, kLdsLimit / std::max<long long>(1, cell_bytes * cpb));
+    long long waves = std::max<long long>(4, std::min<long long>(16, 32 / blocks_per_cu));
+    while (waves > 4 && units(cpb) < 2 * waves) waves >>= 1;
+    threads = (int)waves * kWave;
+    break;
+  }
+  if (g_fwd_threads >= 64 && g_fwd_threads <= 1024 && g_fwd_threads % 64 == 0) threads = g_fwd_threads;
   StagedArgs a;
   fill_args(a, *plan, f, xs, ys, ncells, offs_add, accumulate);
   a.cpb = (int)cpb;
   const long long nblocks = (ncells + cpb - 1) / cpb;
   if (nblocks > 0x7fffffffLL) return GELIB_HIP_ERR_ARG;
-  rc = launch_staged_fwd(a, diag, (int)nblocks, (size_t)(cell_bytes * cpb), s);
+  rc = launch_staged_fwd(a, diag, tile, threads, (int)nblocks, (size_t)(cell_bytes * cpb), s);
   if (rc) return rc;
   *used = 1;
   return GELIB_HIP_OK;
@@ -356,6 +395,14 @@ int staged_set_option(const char *name, int value) {
   }
   if (!std::strcmp(name, "staged_bwd")) {
     g_bwd_enable = value;
+    return GELIB_HIP_OK;
+  }
+  if (!std::strcmp(name, "staged_fwd_tile")) {
+    g_fwd_tile = value;
+    return GELIB_HIP_OK;
+  }
+  if (!std::strcmp(name, "staged_fwd_threads")) {
+    g_fwd_threads = value;
     return GELIB_HIP_OK;
   }
   if (!std::strcmp(name, "staged_bwd_stripes")) {

@@ -105,6 +105,17 @@ def test_backward_block_widths(cabi, threads):
         cabi.set_option("staged_bwd_threads", 0)
 
 
+@pytest.mark.parametrize("tile", [1, 2, 4])
+def test_forward_tile_widths(cabi, tile):
+    cabi.set_option("staged_fwd_tile", tile)
+    try:
+        run_vec(cabi, 37, {5: 8, 6: 8}, {5: 8, 6: 8}, 9, False, seed=650)
+        run_vec(cabi, 37, {5: 8, 6: 8}, {5: 8, 6: 8}, 9, True, seed=651)
+        run_vec(cabi, 3, {6: 64}, {6: 64}, 6, True, seed=652)
+    finally:
+        cabi.set_option("staged_fwd_tile", 0)
+
+
 def test_channel_counts_that_are_not_powers_of_two(cabi):
     # the forward kernel takes any channel count; the backward lane sums need powers of two, so the gradient
     # call falls back to the shape-agnostic kernels
@@ -112,9 +123,10 @@ def test_channel_counts_that_are_not_powers_of_two(cabi):
     run_vec(cabi, 4, {5: 3, 6: 3}, {5: 3, 1: 3}, -1, True, seed=701, expect_bwd=1)
 
 
+@pytest.mark.parametrize("offs", [3, 4])   # odd: one channel per lane; multiple of 4: four adjacent channels per lane
 @pytest.mark.parametrize("diag", [False, True])
-def test_part_level_with_offset(cabi, diag):
-    B, l1, l2, l, n1, n2, offs, extra = 9, 6, 5, 7, 4, (4 if diag else 8), 3, 2
+def test_part_level_with_offset(cabi, diag, offs):
+    B, l1, l2, l, n1, n2, extra = 9, 6, 5, 7, 4, (4 if diag else 8), 4
     nout = n1 if diag else n1 * n2
     x, y = U.seeded(1, B, 2 * l1 + 1, n1), U.seeded(2, B, 2 * l2 + 1, n2)
     g = U.seeded(3, B, 2 * l + 1, offs + nout + extra)

@@ -44,6 +44,7 @@ struct StagedArgs {
   int accumulate;
   int xsize, ysize;  // complex elements of one cell's packed x / y image
   int cpb;           // cells per block
+  int lds_coeffs;    // forward: floats of the coefficient stream staged in LDS behind the operands (0 = read from memory)
   int xrows[kMaxParts], yrows[kMaxParts];
 };
 

@@ -149,6 +149,21 @@ __device__ __forceinline__ void for_coeffs(CoeffStream &cs, int pos, int len, in
   for (; t < len; t++) term(lane_value(cs.nxt, t - first));
 }
 
+// The same over a coefficient stream held in LDS (every lane reads the same address)
+typedef const __attribute__((address_space(3))) float *LdsCoeffs;
+template <class F>
+__device__ __forceinline__ void for_coeffs_lds(LdsCoeffs c, int len, F &&term) {
+  int t = 0;
+  for (; t + 4 <= len; t += 4) {
+    const float c0 = c[t], c1 = c[t + 1], c2 = c[t + 2], c3 = c[t + 3];
+    term(c0);
+    term(c1);
+    term(c2);
+    term(c3);
+  }
+  for (; t < len; t++) term(c[t]);
+}
+
 // ---- forward ------------------------------------------------------------------------------------------------------
 typedef float v4f __attribute__((ext_vector_type(4)));
 
@@ -195,7 +210,8 @@ __device__ __forceinline__ void store_tile(GlobalC *dst, const CTile<TILE> &t, b
 // the per-row and per-term bookkeeping -- which is most of the instructions when rows are short -- is shared by
 // TILE complex products.  The host picks TILE (1, 2 or 4) so that every channel count and offset is a multiple of
 // it and the output pointers are 8*TILE-byte aligned.
-template <bool DIAG, int TILE>
+// LDSC: the coefficient stream has been staged in LDS (it fits); otherwise it is streamed through lane reads.
+template <bool DIAG, int TILE, bool LDSC>
 __global__ void __launch_bounds__(1024) staged_fwd_kernel(const StagedArgs) {
   const ArgPtr a = kernel_args();
   extern __shared__ float2 staged_lds[];
@@ -207,12 +223,17 @@ __global__ void __launch_bounds__(1024) staged_fwd_kernel(const StagedArgs) {
   const int ncell = left < cpb ? (int)left : cpb;
   copy_image<0>(a->x, a->xrows, a->nx, xs, xsize, cell0, ncell);
   copy_image<0>(a->y, a->yrows, a->ny, ys, ysize, cell0, ncell);
+  const float *bank = a->bank;
+  float *coeffs = reinterpret_cast<float *>(ys + cpb * ysize);
+  if (LDSC) {
+    const int n = a->lds_coeffs;
+    for (int e = threadIdx.x; e < n; e += blockDim.x) coeffs[e] = ((const __attribute__((address_space(1))) float *)bank)[e];
+  }
   __syncthreads();
 
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & (kWave - 1);
   const int W = blockDim.x >> 6;
   const TriplePtr triples = (TriplePtr)a->triples;
-  const float *bank = a->bank;
   const int ntriples = a->ntriples, offs_add = a->offs_add;
   const bool accumulate = a->accumulate != 0;
   int base = 0;
@@ -237,7 +258,7 @@ __global__ void __launch_bounds__(1024) staged_fwd_kernel(const StagedArgs) {
       GlobalC *rp = (GlobalC *)R.ptr + (cell0 + cl) * R.sb + (tr->offs + offs_add + u);
       int pos = tr->cg_fwd;
       CoeffStream cs;
-      cs.start(bank, pos, lane);
+      if (!LDSC) cs.start(bank, pos, lane);
       for (int m = -l; m <= l; m++) {
         const int m1lo = max(-l1, m - l2), m1hi = min(l1, m + l2);
         LdsC xp = xb + (m1lo + l1) * n1;
@@ -245,7 +266,7 @@ __global__ void __launch_bounds__(1024) staged_fwd_kernel(const StagedArgs) {
         CTile<TILE> acc;
 #pragma unroll
         for (int k = 0; k < TILE; k++) acc.v[k] = v2f{0.f, 0.f};
-        for_coeffs(cs, pos, m1hi - m1lo + 1, lane, [&](float c) __attribute__((always_inline)) {
+        auto term = [&](float c) __attribute__((always_inline)) {
           const CTile<DIAG ? TILE : 1> xt = lds_tile<DIAG ? TILE : 1>(xp);
           const CTile<TILE> yt = lds_tile<TILE>(yp);
           xp += n1;
@@ -259,7 +280,9 @@ __global__ void __launch_bounds__(1024) staged_fwd_kernel(const StagedArgs) {
             acc.v[k].y = fmaf(pr, yv.y, acc.v[k].y);
             acc.v[k].y = fmaf(pi, yv.x, acc.v[k].y);
           }
-        });
+        };
+        if (LDSC) for_coeffs_lds((LdsCoeffs)coeffs + pos, m1hi - m1lo + 1, term);
+        else for_coeffs(cs, pos, m1hi - m1lo + 1, lane, term);
         pos += m1hi - m1lo + 1;
         if (live) store_tile<TILE>(rp + (long long)(m + l) * R.sm, acc, accumulate);
       }
@@ -634,20 +657,23 @@ int launch_stripe_cap(const StagedArgs &a, bool diag, int role, int nblocks, siz
 
 }  // namespace
 
+template <bool DIAG, bool LDSC>
+static int launch_fwd_tiles(const StagedArgs &a, int tile, int threads, int nblocks, size_t lds, hipStream_t s) {
+  static bool attr[3] = {false, false, false};
+  if (tile == 4) return launch(staged_fwd_kernel<DIAG, 4, LDSC>, a, threads, nblocks, lds, s, &attr[0]);
+  if (tile == 2) return launch(staged_fwd_kernel<DIAG, 2, LDSC>, a, threads, nblocks, lds, s, &attr[1]);
+  if (tile == 1) return launch(staged_fwd_kernel<DIAG, 1, LDSC>, a, threads, nblocks, lds, s, &attr[2]);
+  return GELIB_HIP_ERR_ARG;
+}
+
 int launch_staged_fwd(const StagedArgs &a, bool diag, int tile, int threads, int nblocks, size_t lds_bytes,
                       hipStream_t s) {
-  static bool attr[6] = {false, false, false, false, false, false};
   if (lds_bytes > (size_t)kMaxDynamicLds || threads < 64 || threads > 1024 || threads % 64) return GELIB_HIP_ERR_ARG;
-  if (diag) {
-    if (tile == 4) return launch(staged_fwd_kernel<true, 4>, a, threads, nblocks, lds_bytes, s, &attr[0]);
-    if (tile == 2) return launch(staged_fwd_kernel<true, 2>, a, threads, nblocks, lds_bytes, s, &attr[1]);
-    if (tile == 1) return launch(staged_fwd_kernel<true, 1>, a, threads, nblocks, lds_bytes, s, &attr[2]);
-  } else {
-    if (tile == 4) return launch(staged_fwd_kernel<false, 4>, a, threads, nblocks, lds_bytes, s, &attr[3]);
-    if (tile == 2) return launch(staged_fwd_kernel<false, 2>, a, threads, nblocks, lds_bytes, s, &attr[4]);
-    if (tile == 1) return launch(staged_fwd_kernel<false, 1>, a, threads, nblocks, lds_bytes, s, &attr[5]);
-  }
-  return GELIB_HIP_ERR_ARG;
+  const bool ldsc = a.lds_coeffs > 0;
+  if (diag) return ldsc ? launch_fwd_tiles<true, true>(a, tile, threads, nblocks, lds_bytes, s)
+                        : launch_fwd_tiles<true, false>(a, tile, threads, nblocks, lds_bytes, s);
+  return ldsc ? launch_fwd_tiles<false, true>(a, tile, threads, nblocks, lds_bytes, s)
+              : launch_fwd_tiles<false, false>(a, tile, threads, nblocks, lds_bytes, s);
 }
 
 int launch_staged_bwd(const StagedArgs &a, bool diag, bool want_x, bool want_y, int cap, int threads, int nblocks,

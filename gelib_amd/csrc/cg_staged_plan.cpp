@@ -16,6 +16,7 @@ namespace {
 int g_fwd_enable = 1;
 int g_bwd_enable = 1;
 int g_fwd_tile = 0;           // 0 = widest tile that fits, else force 1 / 2 / 4 (still subject to divisibility)
+int g_fwd_coeffs_lds = 1;     // forward coefficients staged in LDS when they fit
 int g_fwd_threads = 0;        // 0 = choose from the LDS footprint
 int g_bwd_stripes = 1;       // striped (register-accumulating) backward kernels: 0 never, 1 where they pay, 2 wherever they apply
 int g_bwd_threads = 0;       // 0 = choose from the LDS footprint, else force 256 / 512 / 1024
@@ -31,6 +32,7 @@ struct DevicePlan {
   int *d_stripes = nullptr;
   int xsize = 0, ysize = 0;
   int lmax_out = 0;
+  int fwd_len = 0;           // floats of the forward coefficient stream (the first region of the bank)
   bool stripes_ok = false;   // the striped backward kernels apply
   int stripe_cap = 0;        // register rows they need (16 or 32)
   std::vector<int> stripes;  // host copy of the table
@@ -56,7 +58,7 @@ int get_plan(bool diag, const std::vector<VecTriple> &triples, const std::vector
     return GELIB_HIP_OK;
   }
   DevicePlan plan;
-  std::vector<float> bank;
+  std::vector<float> bank, fwd, back0, back1;  // the three streams are laid out one after the other
   std::vector<int> xoff(xs.size()), yoff(ys.size());
   for (size_t i = 0; i < xs.size(); i++) {
     xoff[i] = plan.xsize;
@@ -82,18 +84,26 @@ int get_plan(bool diag, const std::vector<VecTriple> &triples, const std::vector
     full.assign((size_t)L1 * L2, 0.f);
     cg_matrix_host(t.l1, t.l2, t.l, full.data());
     auto C = [&](int m1, int m2) { return full[(size_t)(m1 + t.l1) * L2 + (m2 + t.l2)]; };
-    r.cg_fwd = (int)bank.size();
+    r.cg_fwd = (int)fwd.size();
     for (int m = -t.l; m <= t.l; m++)
-      for (int m1 = std::max(-t.l1, m - t.l2); m1 <= std::min(t.l1, m + t.l2); m1++) bank.push_back(C(m1, m - m1));
-    r.cg_back0 = (int)bank.size();
+      for (int m1 = std::max(-t.l1, m - t.l2); m1 <= std::min(t.l1, m + t.l2); m1++) fwd.push_back(C(m1, m - m1));
+    r.cg_back0 = (int)back0.size();
     for (int m1 = -t.l1; m1 <= t.l1; m1++)
-      for (int m2 = std::max(-t.l2, -t.l - m1); m2 <= std::min(t.l2, t.l - m1); m2++) bank.push_back(C(m1, m2));
-    r.cg_back1 = (int)bank.size();
+      for (int m2 = std::max(-t.l2, -t.l - m1); m2 <= std::min(t.l2, t.l - m1); m2++) back0.push_back(C(m1, m2));
+    r.cg_back1 = (int)back1.size();
     for (int m2 = -t.l2; m2 <= t.l2; m2++)
-      for (int m1 = std::max(-t.l1, -t.l - m2); m1 <= std::min(t.l1, t.l - m2); m1++) bank.push_back(C(m1, m2));
+      for (int m1 = std::max(-t.l1, -t.l - m2); m1 <= std::min(t.l1, t.l - m2); m1++) back1.push_back(C(m1, m2));
     plan.lmax_out = std::max(plan.lmax_out, t.l);
     plan.triples.push_back(r);
   }
+  plan.fwd_len = (int)fwd.size();
+  for (auto &r : plan.triples) {
+    r.cg_back0 += (int)fwd.size();
+    r.cg_back1 += (int)(fwd.size() + back0.size());
+  }
+  bank = fwd;
+  bank.insert(bank.end(), back0.begin(), back0.end());
+  bank.insert(bank.end(), back1.begin(), back1.end());
   bank.resize(bank.size() + 4 * kWave, 0.f);  // the kernels read the stream up to three registers of lanes ahead
   // stripes: the triples that feed one x part (resp. one y part)
   {
@@ -208,6 +218,10 @@ int run_fwd(bool diag, const std::vector<VecTriple> &triples, const std::vector<
   int rc = get_plan(diag, triples, xs, ys, rls, &plan);
   if (rc) return rc;
   const long long cell_bytes = 8LL * (plan->xsize + plan->ysize);
+  // The forward coefficient stream goes into LDS next to the operands when it fits: read from memory it would
+  // share the wave's memory counter with the output stores and every refill would wait for them.
+  const long long coeff_bytes = (g_fwd_coeffs_lds && 4LL * plan->fwd_len <= 64 * 1024 && cell_bytes + 4LL * plan->fwd_len <= kLdsLimit)
+                                    ? 4LL * ((plan->fwd_len + 3) / 4 * 4) : 0;
   // Channels per lane: the widest tile that divides every channel count and offset and keeps the 16-byte
   // accesses aligned, provided enough cells fit in LDS to fill a wave with tile slots.
   auto tile_ok = [&](int tile) {
@@ -236,11 +250,11 @@ int run_fwd(bool diag, const std::vector<VecTriple> &triples, const std::vector<
     };
     cpb = 1;
     // first fill the lanes of a run, then give the block's waves enough runs
-    while (cpb * 2 <= ncells && cpb * slots_min < kWave && cell_bytes * cpb * 2 <= 110 * 1024) cpb *= 2;
-    while (cpb * 2 <= ncells && cell_bytes * cpb * 2 <= g_fwd_lds_target && units(cpb) < 16) cpb *= 2;
+    while (cpb * 2 <= ncells && cpb * slots_min < kWave && cell_bytes * cpb * 2 + coeff_bytes <= 140 * 1024) cpb *= 2;
+    while (cpb * 2 <= ncells && cell_bytes * cpb * 2 + coeff_bytes <= g_fwd_lds_target && units(cpb) < 16) cpb *= 2;
     if (tile > 1 && cpb * slots_min < kWave && cpb < ncells) continue;  // lanes would idle: try a narrower tile
     // as many waves per CU as the LDS footprint leaves room for, without more waves than runs
-    const long long blocks_per_cu = std::max<long long>(1, kLdsLimit / std::max<long long>(1, cell_bytes * cpb));
+    const long long blocks_per_cu = std::max<long long>(1, kLdsLimit / std::max<long long>(1, cell_bytes * cpb + coeff_bytes));
     long long waves = std::max<long long>(4, std::min<long long>(16, 32 / blocks_per_cu));
     while (waves > 4 && units(cpb) < 2 * waves) waves >>= 1;
     threads = (int)waves * kWave;
@@ -250,9 +264,10 @@ int run_fwd(bool diag, const std::vector<VecTriple> &triples, const std::vector<
   StagedArgs a;
   fill_args(a, *plan, f, xs, ys, ncells, offs_add, accumulate);
   a.cpb = (int)cpb;
+  a.lds_coeffs = coeff_bytes ? plan->fwd_len : 0;
   const long long nblocks = (ncells + cpb - 1) / cpb;
   if (nblocks > 0x7fffffffLL) return GELIB_HIP_ERR_ARG;
-  rc = launch_staged_fwd(a, diag, tile, threads, (int)nblocks, (size_t)(cell_bytes * cpb), s);
+  rc = launch_staged_fwd(a, diag, tile, threads, (int)nblocks, (size_t)(cell_bytes * cpb + coeff_bytes), s);
   if (rc) return rc;
   *used = 1;
   return GELIB_HIP_OK;
@@ -399,6 +414,10 @@ int staged_set_option(const char *name, int value) {
   }
   if (!std::strcmp(name, "staged_fwd_tile")) {
     g_fwd_tile = value;
+    return GELIB_HIP_OK;
+  }
+  if (!std::strcmp(name, "staged_fwd_coeffs_lds")) {
+    g_fwd_coeffs_lds = value;
     return GELIB_HIP_OK;
   }
   if (!std::strcmp(name, "staged_fwd_threads")) {

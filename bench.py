@@ -23,7 +23,10 @@ HBM_PEAK = 8.0e12  # B/s, MI355X HBM3E
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs, each scaled by what the
 # counter reads for a plain 1 GiB copy: x2.000 and x1.000); summary in profiles/.
 MEASURED_TRAFFIC = {
-    "so3vec_cg_L4_tau16_B32768_maxl4": {"so3vec_fwd": 26220896459, "so3vec_bwd": 26014461035},
+    "so3vec_cg_L4_tau16_B32768_maxl4": {"so3vec_fwd": 26221108310, "so3vec_bwd": 26008901737},
+    # the backward pass of this type runs as two launches (one per gradient), each reading g: 1.88 x algorithmic
+    "so3vec_diagcg_L6_n64_B131072": {"so3vec_fwd": 102040514571, "so3vec_bwd": 203991472933},
+    "so3part_cg_10x10_all_l_n8_B16384": {"so3vec_fwd": 3746895112, "so3vec_bwd": 3809656495},
 }
 
 WORKLOADS = {
@@ -199,7 +202,7 @@ def main():
                    "fwd_bwd_frac_of_peak": (fwd_bytes + bwd_bytes) / ((fwd_ms + bwd_ms) * 1e-3) / HBM_PEAK},
         "roofline": {"bound": "hbm", "kernel": dom, "achieved": achieved, "peak": HBM_PEAK / 1e9, "unit": "GB/s",
                      "frac": achieved * 1e9 / HBM_PEAK,
-                     "traffic": MEASURED_TRAFFIC.get(name, {}).get(dom) if B == WORKLOADS[name][1] and path == 2 else None,
+                     "traffic": MEASURED_TRAFFIC.get(name, {}).get(dom) if B == WORKLOADS[name][1] and path in (2, 3) else None,
                      "algorithmic_bytes_per_launch": dom_bytes},
     }
     if not args.no_cpu:

@@ -1,0 +1,109 @@
+"""SO3partArr: an array of SO3parts, shape (b, a_1, ..., a_k, 2l+1, n) complex64 -- the class and autograd functions
+of python/src/gelib/SO3partArr.py:18-234 for the CG product path.  The grid dimensions a_1..a_k travel to the kernels
+as the grid dimensions of the part descriptor (core/Gpart.hpp:416-432, 495-531); nothing is reshaped or copied."""
+import torch
+
+from gelib_amd.gelib_common import backend, common_batch
+from gelib_amd.SO3element import SO3element, SO3irrep
+from gelib_amd.SO3part import SO3part
+
+
+class SO3partArr(torch.Tensor):
+
+    @staticmethod
+    def zeros(b, adims, l, n, device='cpu'):
+        return SO3partArr(torch.zeros([b] + list(adims) + [2 * l + 1, n], dtype=torch.complex64, device=device))
+
+    @staticmethod
+    def ones(b, adims, l, n, device='cpu'):
+        return SO3partArr(torch.ones([b] + list(adims) + [2 * l + 1, n], dtype=torch.complex64, device=device))
+
+    @staticmethod
+    def randn(b, adims, l, n, device='cpu'):
+        return SO3partArr(torch.randn([b] + list(adims) + [2 * l + 1, n], dtype=torch.complex64, device=device))
+
+    def zeros_like(self, *args):
+        if not args:
+            return SO3partArr(torch.zeros_like(self))
+        assert len(args) == 2 and isinstance(args[0], int) and isinstance(args[1], int)
+        dims = list(self.size())
+        dims[-2], dims[-1] = 2 * args[0] + 1, args[1]
+        return SO3partArr(torch.zeros(dims, dtype=torch.complex64, device=self.device))
+
+    @classmethod
+    def randn_like(cls, x):
+        return SO3partArr(torch.randn_like(x))
+
+    def backend(self):
+        return backend().SO3part.view(self)
+
+    def collapse(self):
+        return SO3part(self.reshape(self.size(0), -1, self.size(-2), self.size(-1)))
+
+    def getb(self):
+        return self.size(0)
+
+    def get_adims(self):
+        return list(self.size()[1:self.dim() - 2])
+
+    def get_nadims(self):
+        return self.dim() - 3
+
+    def getl(self):
+        return int((self.size(-2) - 1) / 2)
+
+    def getn(self):
+        return self.size(-1)
+
+    def odot(self, y):
+        return torch.Tensor(torch.sum(torch.mul(torch.view_as_real(self), torch.view_as_real(y))))
+
+    def apply(self, R):
+        assert isinstance(R, SO3element)
+        rho = SO3irrep(self.getl())
+        return SO3partArr(torch.matmul(rho.matrix(R).to(self.device), self))
+
+    def CGproduct(self, y, l):
+        return SO3partArr_CGproductFn.apply(self, y, l)
+
+    def DiagCGproduct(self, y, l):
+        return SO3partArr_DiagCGproductFn.apply(self, y, l)
+
+
+def _view(t):
+    return backend().SO3part.view(t)
+
+
+def _part_fn(diag):
+    name = "DiagCGproduct" if diag else "CGproduct"
+
+    class Fn(torch.autograd.Function):
+
+        @staticmethod
+        def forward(ctx, x, y, l):
+            ctx.l = l
+            ctx.save_for_backward(x, y)
+            b = common_batch(x, y)
+            a = x.get_adims() if isinstance(x, SO3partArr) else list(x.size()[1:x.dim() - 2])
+            if diag:
+                assert x.size(-1) == y.size(-1)
+            r = SO3partArr.zeros(b, a, l, x.size(-1) if diag else x.size(-1) * y.size(-1), device=x.device)
+            getattr(_view(r), "add_" + name)(_view(x), _view(y))
+            return r
+
+        @staticmethod
+        def backward(ctx, g):
+            x, y = ctx.saved_tensors
+            g = g.contiguous()
+            xg = torch.zeros_like(x)
+            yg = torch.zeros_like(y)
+            getattr(_view(xg), "add_%s_back0" % name)(_view(g), _view(y))
+            getattr(_view(yg), "add_%s_back1" % name)(_view(g), _view(x))
+            return xg, yg, None
+
+    Fn.__name__ = "SO3partArr_%sFn" % name
+    return Fn
+
+
+SO3partArr_CGproductFn = _part_fn(False)
+SO3partArr_DiagCGproductFn = _part_fn(True)

@@ -90,7 +90,9 @@ class SO3vec:
         return "<SO3vec of type %s [b=%d]>" % (self.tau(), self.getb())
 
 
-def _product_fn(diag):
+def _product_fn(diag, part_cls=SO3part, prefix="SO3vec"):
+    """Autograd function of the fused product; part_cls wraps the output parts.  Works for any number of grid
+    dimensions between the batch and the (2l+1, n) tail (the Arr classes use it too)."""
     gb_type = "DiagCGproduct" if diag else "CGproduct"
 
     class Fn(torch.autograd.Function):
@@ -103,13 +105,14 @@ def _product_fn(diag):
             x = gb.SO3vec.view(list(args[0:k1]))
             y = gb.SO3vec.view(list(args[k1:k1 + k2]))
             b = common_batch(args[0], args[k1])
+            lead = [b] + list(args[0].shape[1:-2])
             tau = getattr(x.get_tau(), gb_type)(y.get_tau(), maxl)
             # uninitialised outputs: every channel of every part is written exactly once by the fused launch
-            rparts = [torch.empty([b, 2 * l + 1, n], dtype=torch.complex64, device=args[0].device)
+            rparts = [torch.empty(lead + [2 * l + 1, n], dtype=torch.complex64, device=args[0].device)
                       for l, n in tau.get_parts().items()]
             r = gb.SO3vec.view(rparts)
             (r.setDiagCGproduct if diag else r.setCGproduct)(x, y)
-            return tuple(SO3part(t) for t in rparts)
+            return tuple(part_cls(t) for t in rparts)
 
         @staticmethod
         def backward(ctx, *gargs):
@@ -122,8 +125,8 @@ def _product_fn(diag):
             g = gb.SO3vec.view([t.contiguous() for t in gargs])
             xg = gb.SO3vec.view(grads[0:k1])
             yg = gb.SO3vec.view(grads[k1:k1 + k2])
-            if any(t.size(0) != gargs[0].size(0) for t in saved):
-                # a batch-broadcast operand: its gradient is a sum over the batch, done by the accumulate path
+            if any(t.shape[:-2] != gargs[0].shape[:-2] for t in saved):
+                # a broadcast operand: its gradient is a sum over the broadcast cells, done by the accumulate path
                 for t in grads:
                     t.zero_()
                 getattr(xg, "add%s_back0" % gb_type)(g, y)
@@ -132,7 +135,7 @@ def _product_fn(diag):
                 getattr(gb.SO3vec, "set%s_back" % gb_type)(xg, yg, g, x, y)
             return tuple([None, None, None] + grads)
 
-    Fn.__name__ = "SO3vec_%sFn" % gb_type
+    Fn.__name__ = "%s_%sFn" % (prefix, gb_type)
     return Fn
 
 

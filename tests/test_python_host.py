@@ -61,3 +61,21 @@ def test_wigner_helper():
         D1, D2, D12 = rho.matrix(R1), rho.matrix(R2), rho.matrix(G.SO3element(R1 @ R2))
         assert torch.allclose(D1 @ D1.conj().t(), torch.eye(2 * l + 1, dtype=torch.complex64), atol=1e-4)
         assert torch.allclose(D1 @ D2, D12, atol=1e-4)      # a representation
+
+
+def test_arr_surface():
+    import gelib_amd as G
+    p = G.SO3partArr.randn(2, [3, 4], 2, 5)
+    assert (p.getb(), p.get_adims(), p.get_nadims(), p.getl(), p.getn()) == (2, [3, 4], 2, 2, 5)
+    assert list(p.zeros_like(1, 7).shape) == [2, 3, 4, 3, 7]
+    assert list(p.collapse().shape) == [2, 12, 5, 5]
+    v = G.SO3vecArr.zeros(2, [3], {0: 2, 2: 1})
+    assert v.tau() == {0: 2, 2: 1} and v.getb() == 2 and v.get_adims() == [3] and v.l_max() == 2
+    w = G.SO3vecArr.randn(2, [3], [2, 1])            # tau given as a list: l = 0, 1
+    assert w.tau() == {0: 2, 1: 1}
+    R = G.SO3element.random()
+    assert list(p.apply(R).shape) == list(p.shape)
+    with pytest.raises(RuntimeError):
+        G.CGproduct(p, p, 2)                          # host tensors are refused, not computed elsewhere
+    with pytest.raises(RuntimeError):
+        G.CGproduct(v, v)

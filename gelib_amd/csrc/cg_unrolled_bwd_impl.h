@@ -37,46 +37,6 @@ typedef const __attribute__((address_space(1))) v2f *GlobalRows;
 // compiler fetches them with scalar loads into SGPRs and they cost neither vector registers nor LDS traffic.
 typedef const __attribute__((address_space(4))) float *CoeffPtr;
 
-template <int ROWS, int KR>
-__device__ __forceinline__ void load_rows(float2 (&buf)[KR], GlobalRows ptr, int sm) {
-#pragma unroll
-  for (int m = 0; m < ROWS; m++) {
-    const v2f t = ptr[m * sm];
-    buf[m] = make_float2(t.x, t.y);
-  }
-}
-
-template <int L1, int L2, int L, int KR, bool WX, bool WY>
-__device__ __forceinline__ void triple_bwd(const float2 (&xv)[2 * L1 + 1], const float2 (&yv)[2 * L2 + 1],
-                                           float2 (&ax)[2 * L1 + 1], float2 (&ay)[2 * L2 + 1],
-                                           CoeffPtr C, const float2 (&g)[KR]) {
-#pragma unroll
-  for (int m1 = -L1; m1 <= L1; m1++) {
-#pragma unroll
-    for (int m2 = -L2; m2 <= L2; m2++) {
-      const int m = m1 + m2;
-      if (m >= -L && m <= L) {
-        const float c = C[(m1 + L1) * (2 * L2 + 1) + (m2 + L2)];
-        const float tr = c * g[m + L].x, ti = c * g[m + L].y;
-        if (WX) {
-          const float2 yc = yv[m2 + L2];
-          ax[m1 + L1].x = fmaf(tr, yc.x, ax[m1 + L1].x);
-          ax[m1 + L1].x = fmaf(ti, yc.y, ax[m1 + L1].x);
-          ax[m1 + L1].y = fmaf(ti, yc.x, ax[m1 + L1].y);
-          ax[m1 + L1].y = fmaf(-tr, yc.y, ax[m1 + L1].y);
-        }
-        if (WY) {
-          const float2 xc = xv[m1 + L1];
-          ay[m2 + L2].x = fmaf(tr, xc.x, ay[m2 + L2].x);
-          ay[m2 + L2].x = fmaf(ti, xc.y, ay[m2 + L2].x);
-          ay[m2 + L2].y = fmaf(ti, xc.x, ay[m2 + L2].y);
-          ay[m2 + L2].y = fmaf(-tr, xc.y, ay[m2 + L2].y);
-        }
-      }
-    }
-  }
-}
-
 // The gradient parts, indexed by their l (the host fills BwdArgs::g that way), copied out of the kernel arguments
 // once so that the unrolled code can name them with compile-time indices.
 template <int LCAP>
@@ -103,14 +63,20 @@ __device__ __forceinline__ LanePos lane_pos(int run, int lane, int log2_u, int n
   return q;
 }
 
-// One run of one pair: every l of the pair that is present, in turn.
-template <int L1, int L2, int LCAP, int KR, bool DIAG, bool WX, bool WY>
-__device__ __forceinline__ void pair_bwd(const GParts<LCAP> &gp, PairPtr pr, CoeffPtr Cs, const float2 *xs,
-                                         const float2 *ys, float2 *xacc, float2 *yacc, int xsize, int ysize,
-                                         long long cell0, int offs_add, const LanePos q) {
+// One run of one pair, all of its l together.  For every row number m = m1 + m2 the lane reads g_l[m] of every l,
+// contracts over l first,
+//     Q[m1,m2] = sum_l C_l[m1,m2] g_l[m1+m2]          (real coefficient times complex: 2 FMA per term)
+// and then feeds both gradients once per (m1,m2):  ax[m1] += Q conj(y[m2]),  ay[m2] += Q conj(x[m1]).
+// That is 2 instructions per term plus 8 per (m1,m2) instead of 10 per term.  An l of the pair whose part is absent
+// reads a row of zeros and a table of zeros (zrows, Zc) instead, so the code has no branches.
+template <int L1, int L2, int LCAP, bool DIAG, bool WX, bool WY>
+__device__ __forceinline__ void pair_bwd(const GParts<LCAP> &gp, PairPtr pr, CoeffPtr Cs, CoeffPtr Zc, GlobalRows zrows,
+                                         const float2 *xs, const float2 *ys, float2 *xacc, float2 *yacc, int xsize,
+                                         int ysize, long long cell0, int offs_add, const LanePos q) {
   constexpr int LMIN = cabs_(L1 - L2);
-  constexpr int NL = 2 * cmin_(L1, L2) + 1;
+  constexpr int LTOP = cmin_(L1 + L2, LCAP);
   if constexpr (LMIN > LCAP) return;  // no l of this pair can be present
+  constexpr int NLP = LTOP - LMIN + 1;
   // scalar loads: the record sits in constant memory and the pointer is uniform
   const __attribute__((address_space(4))) PairRec &p = *pr;
   const int N1 = p.n1, N2 = p.n2;
@@ -136,18 +102,91 @@ __device__ __forceinline__ void pair_bwd(const GParts<LCAP> &gp, PairPtr pr, Coe
 #pragma unroll
   for (int m2 = 0; m2 <= 2 * L2; m2++) ay[m2] = make_float2(0.f, 0.f);
 
-  static_for<NL>([&](auto dl_c) __attribute__((always_inline)) {
+  GlobalRows gptr[NLP];
+  int gsm[NLP];
+  CoeffPtr cl[NLP];
+  static_for<NLP>([&](auto dl_c) __attribute__((always_inline)) {
     constexpr int dl = decltype(dl_c)::value;
-    constexpr int L = LMIN + dl;
-    if constexpr (L <= LCAP) {
-      if (p.ri[dl] >= 0) {
-        float2 gv[KR];
-        const FastPart G = gp.G[L];
-        load_rows<2 * L + 1, KR>(gv, (GlobalRows)G.ptr + cell * G.sb + (p.offs[dl] + offs_add + q.u), G.sm);
-        triple_bwd<L1, L2, L, KR, WX, WY>(xv, yv, ax, ay, Cs + p.cg[dl], gv);
-      }
-    }
+    const bool present = p.ri[dl] >= 0;
+    const FastPart G = gp.G[LMIN + dl];
+    gptr[dl] = present ? (GlobalRows)G.ptr + cell * G.sb + (p.offs[dl] + offs_add + q.u) : zrows;
+    gsm[dl] = present ? G.sm : 0;
+    cl[dl] = present ? Cs + p.cg[dl] : Zc;
   });
+  // rows of one m at a time, the rows of the next m requested before the arithmetic of this one; the scheduling
+  // barrier between steps keeps the compiler from hoisting every load of the pair to the top (twice the registers)
+  auto load_m = [&](auto mc, float2(&dst)[NLP]) __attribute__((always_inline)) {
+    constexpr int m = decltype(mc)::value - LTOP;
+    static_for<NLP>([&](auto dl_c) __attribute__((always_inline)) {
+      constexpr int dl = decltype(dl_c)::value;
+      constexpr int L = LMIN + dl;
+      if constexpr (L >= cabs_(m)) {
+        const v2f t = gptr[dl][(m + L) * gsm[dl]];
+        dst[dl] = make_float2(t.x, t.y);
+      }
+    });
+  };
+  float2 gnext[NLP];
+  load_m(std::integral_constant<int, 0>{}, gnext);
+  static_for<2 * LTOP + 1>([&](auto mc) __attribute__((always_inline)) {
+    constexpr int mi = decltype(mc)::value;
+    constexpr int m = mi - LTOP;
+    constexpr int MABS = cabs_(m);
+    float2 gl[NLP];
+#pragma unroll
+    for (int k = 0; k < NLP; k++) gl[k] = gnext[k];
+    if constexpr (mi + 1 <= 2 * LTOP) load_m(std::integral_constant<int, mi + 1>{}, gnext);
+    constexpr int M1LO = (-L1 > m - L2) ? -L1 : m - L2;
+    constexpr int M1HI = (L1 < m + L2) ? L1 : m + L2;
+    constexpr int NP = M1HI - M1LO + 1;
+    // the coefficients of this m (scalar loads) are requested together; each (m1,m2) then runs as one short
+    // dependent chain, fenced from the next, so only a handful of values are live at any time
+    float cf[NP][NLP];
+    static_for<NP>([&](auto kc) __attribute__((always_inline)) {
+      constexpr int m1 = M1LO + decltype(kc)::value;
+      constexpr int m2 = m - m1;
+      static_for<NLP>([&](auto dl_c) __attribute__((always_inline)) {
+        constexpr int dl = decltype(dl_c)::value;
+        if constexpr (LMIN + dl >= MABS) cf[decltype(kc)::value][dl] = cl[dl][(m1 + L1) * (2 * L2 + 1) + (m2 + L2)];
+      });
+    });
+    __builtin_amdgcn_sched_barrier(0);
+    static_for<NP>([&](auto kc) __attribute__((always_inline)) {
+      constexpr int m1 = M1LO + decltype(kc)::value;
+      constexpr int m2 = m - m1;
+      float qr = 0.f, qi = 0.f;
+      static_for<NLP>([&](auto dl_c) __attribute__((always_inline)) {
+        constexpr int dl = decltype(dl_c)::value;
+        if constexpr (LMIN + dl >= MABS) {
+          const float c = cf[decltype(kc)::value][dl];
+          qr = fmaf(c, gl[dl].x, qr);
+          qi = fmaf(c, gl[dl].y, qi);
+        }
+      });
+      if (WX) {
+        const float2 yc = yv[m2 + L2];
+        ax[m1 + L1].x = fmaf(qr, yc.x, ax[m1 + L1].x);
+        ax[m1 + L1].x = fmaf(qi, yc.y, ax[m1 + L1].x);
+        ax[m1 + L1].y = fmaf(qi, yc.x, ax[m1 + L1].y);
+        ax[m1 + L1].y = fmaf(-qr, yc.y, ax[m1 + L1].y);
+      }
+      if (WY) {
+        const float2 xc = xv[m1 + L1];
+        ay[m2 + L2].x = fmaf(qr, xc.x, ay[m2 + L2].x);
+        ay[m2 + L2].x = fmaf(qi, xc.y, ay[m2 + L2].x);
+        ay[m2 + L2].y = fmaf(qi, xc.x, ay[m2 + L2].y);
+        ay[m2 + L2].y = fmaf(-qr, xc.y, ay[m2 + L2].y);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    });
+    __builtin_amdgcn_sched_barrier(0);
+  });
+  // pin the sums here: without this the optimiser moves the whole chain of ay updates down to its first use after
+  // the ax part, keeping every Q alive until then
+#pragma unroll
+  for (int m1 = 0; m1 <= 2 * L1; m1++) asm volatile("" : "+v"(ax[m1].x), "+v"(ax[m1].y));
+#pragma unroll
+  for (int m2 = 0; m2 <= 2 * L2; m2++) asm volatile("" : "+v"(ay[m2].x), "+v"(ay[m2].y));
 
   if (WX) {
     if (!DIAG) group_sum(ax, N2);
@@ -253,6 +292,8 @@ __global__ void __launch_bounds__(kBlock) unrolled_bwd_kernel(const BwdArgs a) {
   auto runs_of = [&](int k) { return ((cpb << pairs[k].log2_u) + kWave - 1) >> 6; };
   GParts<LCAP> gp;
   static_for<LCAP + 1>([&](auto l) __attribute__((always_inline)) { gp.G[l.value] = a.g[l.value]; });
+  const CoeffPtr Zc = (CoeffPtr)(a.bank + a.zero_off);    // a table of zeros and ...
+  const GlobalRows zrows = (GlobalRows)(a.bank + a.zero_off);  // ... a row of zeros, for parts that are absent
   for (int pidx = 0; pidx < npairs; pidx++) {
     const PairPtr p = pairs + pidx;
     const int nruns = runs_of(pidx);
@@ -262,7 +303,7 @@ __global__ void __launch_bounds__(kBlock) unrolled_bwd_kernel(const BwdArgs a) {
       switch (p->l1 * (kLT + 1) + p->l2) {
 #define GELIB_CASE(A, B)                                                                                      \
   case A * (kLT + 1) + B:                                                                                     \
-    pair_bwd<A, B, LCAP, KR, DIAG, WX, WY>(gp, p, C, xs, ys, xacc, yacc, xsize, ysize, cell0, offs_add, q); \
+    pair_bwd<A, B, LCAP, DIAG, WX, WY>(gp, p, C, Zc, zrows, xs, ys, xacc, yacc, xsize, ysize, cell0, offs_add, q); \
     break;
 #define GELIB_ROW(A) GELIB_CASE(A, 0) GELIB_CASE(A, 1) GELIB_CASE(A, 2) GELIB_CASE(A, 3) GELIB_CASE(A, 4)
         GELIB_ROW(0) GELIB_ROW(1) GELIB_ROW(2) GELIB_ROW(3) GELIB_ROW(4)

@@ -23,6 +23,7 @@ struct DevicePlan {
   PairRec *d_pairs = nullptr;
   float *d_bank = nullptr;
   int bank_len = 0;
+  int zero_off = 0;  // a run of zeros in the bank (stand-in table and stand-in row for absent parts)
   int xsize = 0, ysize = 0;
 };
 
@@ -155,6 +156,9 @@ int get_plan(bool diag, const std::vector<VecTriple> &triples, const std::vector
     cg_matrix_host(t.l1, t.l2, t.l, bank.data() + bank.size() - n);
     p->cg_len = (int)bank.size() - p->cg_base;
   }
+  if (bank.size() % 2) bank.push_back(0.f);
+  plan.zero_off = (int)bank.size();
+  bank.resize(bank.size() + (2 * kLT + 1) * (2 * kLT + 1) + 1, 0.f);
   plan.bank_len = (int)bank.size();
   const size_t pair_bytes = plan.pairs.size() * sizeof(PairRec);
   const size_t bank_bytes = bank.size() * sizeof(float);
@@ -273,6 +277,7 @@ int run_bwd(bool diag, const std::vector<VecTriple> &triples, const std::vector<
   a.want_x = want_x ? 1 : 0;
   a.want_y = want_y ? 1 : 0;
   a.bank_len = plan->bank_len;
+  a.zero_off = plan->zero_off;
   a.xsize = plan->xsize;
   a.ysize = plan->ysize;
   for (size_t i = 0; i < xs.size(); i++) a.xrows[i] = 2 * xs[i].first + 1;

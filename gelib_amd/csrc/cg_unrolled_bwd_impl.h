@@ -139,18 +139,8 @@ __device__ __forceinline__ void pair_bwd(const GParts<LCAP> &gp, PairPtr pr, Coe
     constexpr int M1LO = (-L1 > m - L2) ? -L1 : m - L2;
     constexpr int M1HI = (L1 < m + L2) ? L1 : m + L2;
     constexpr int NP = M1HI - M1LO + 1;
-    // the coefficients of this m (scalar loads) are requested together; each (m1,m2) then runs as one short
-    // dependent chain, fenced from the next, so only a handful of values are live at any time
-    float cf[NP][NLP];
-    static_for<NP>([&](auto kc) __attribute__((always_inline)) {
-      constexpr int m1 = M1LO + decltype(kc)::value;
-      constexpr int m2 = m - m1;
-      static_for<NLP>([&](auto dl_c) __attribute__((always_inline)) {
-        constexpr int dl = decltype(dl_c)::value;
-        if constexpr (LMIN + dl >= MABS) cf[decltype(kc)::value][dl] = cl[dl][(m1 + L1) * (2 * L2 + 1) + (m2 + L2)];
-      });
-    });
-    __builtin_amdgcn_sched_barrier(0);
+    // each (m1,m2) runs as one short dependent chain, fenced from the next, so only a handful of values are live
+    // at any time (left alone, the scheduler interleaves all chains of an m and doubles the register count)
     static_for<NP>([&](auto kc) __attribute__((always_inline)) {
       constexpr int m1 = M1LO + decltype(kc)::value;
       constexpr int m2 = m - m1;
@@ -158,7 +148,7 @@ __device__ __forceinline__ void pair_bwd(const GParts<LCAP> &gp, PairPtr pr, Coe
       static_for<NLP>([&](auto dl_c) __attribute__((always_inline)) {
         constexpr int dl = decltype(dl_c)::value;
         if constexpr (LMIN + dl >= MABS) {
-          const float c = cf[decltype(kc)::value][dl];
+          const float c = cl[dl][(m1 + L1) * (2 * L2 + 1) + (m2 + L2)];
           qr = fmaf(c, gl[dl].x, qr);
           qi = fmaf(c, gl[dl].y, qi);
         }

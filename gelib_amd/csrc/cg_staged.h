@@ -37,6 +37,9 @@ struct StagedArgs {
   // Striped backward kernels: (first, count, log2 of slots per cell) for every x part, then for every y part, then
   // the triple numbers ordered by x part, then ordered by y part; first indexes into the matching order list.
   const int *stripes;
+  // Pair-wise backward kernel: (first triple, count, coefficient stream offset) per (x part, y part) pair.
+  const int *pairs;
+  int npairs;
   long long ncells;
   int ntriples;
   int nx, ny;
@@ -58,6 +61,10 @@ int launch_staged_bwd(const StagedArgs &a, bool diag, bool want_x, bool want_y, 
 // role 0: gradient of x, 1: gradient of y; cap 16 or 32 (own 2l+1 must not exceed it)
 int launch_staged_stripe(const StagedArgs &a, bool diag, int role, int cap, int nblocks, size_t lds_bytes,
                          hipStream_t s);
+
+// both gradients from one pass over g, one (pair, 64 slots) unit at a time; cap 16 or 32
+int launch_staged_pair_bwd(const StagedArgs &a, bool diag, bool want_x, bool want_y, int cap, int nblocks,
+                           size_t lds_bytes, hipStream_t s);
 
 // kind: 0 forward, 1 back0 (destination op.x), 2 back1 (destination op.y).  *used = 1 if a launch was made.
 int staged_part(int kind, const PartOp &op, bool accumulate, hipStream_t s, int *used);

@@ -19,6 +19,8 @@ int g_fwd_tile = 0;           // 0 = widest tile that fits, else force 1 / 2 / 4
 int g_fwd_coeffs_lds = 1;     // forward coefficients staged in LDS when they fit
 int g_fwd_threads = 0;        // 0 = choose from the LDS footprint
 int g_bwd_stripes = 1;       // striped (register-accumulating) backward kernels: 0 never, 1 where they pay, 2 wherever they apply
+int g_bwd_pairs = 0;         // pair-wise single-pass backward kernel where the striped ones are not used: 1 yes, 0 no
+                             // (off: measured slower than the triple-wise kernel, 6.5 vs 5.9 ms at l1 = l2 = 10)
 int g_bwd_threads = 0;       // 0 = choose from the LDS footprint, else force 256 / 512 / 1024
 int g_fwd_lds_target = 32 * 1024;  // LDS up to which a forward block takes more cells to fill its waves
 int g_bwd_lds_target = 40 * 1024;
@@ -36,6 +38,10 @@ struct DevicePlan {
   bool stripes_ok = false;   // the striped backward kernels apply
   int stripe_cap = 0;        // register rows they need (16 or 32)
   std::vector<int> stripes;  // host copy of the table
+  int npairs = 0;            // (x part, y part) pairs; their table follows the stripe tables
+  bool pairs_ok = false;     // the pair-wise backward kernel applies
+  int pair_cap = 0;          // register rows it needs (16 or 32)
+  int pair_off = 0;          // ints from the start of the stripe tables to the pair table
 };
 
 std::mutex g_plan_mutex;
@@ -58,7 +64,7 @@ int get_plan(bool diag, const std::vector<VecTriple> &triples, const std::vector
     return GELIB_HIP_OK;
   }
   DevicePlan plan;
-  std::vector<float> bank, fwd, back0, back1;  // the three streams are laid out one after the other
+  std::vector<float> bank, fwd, back0, back1, pairwise;  // the streams are laid out one after the other
   std::vector<int> xoff(xs.size()), yoff(ys.size());
   for (size_t i = 0; i < xs.size(); i++) {
     xoff[i] = plan.xsize;
@@ -101,9 +107,46 @@ int get_plan(bool diag, const std::vector<VecTriple> &triples, const std::vector
     r.cg_back0 += (int)fwd.size();
     r.cg_back1 += (int)(fwd.size() + back0.size());
   }
+  // Pairs: runs of consecutive triples with the same x part and y part (their l ascending).  The pair-wise backward
+  // kernel reads, for every m and every (m1, m-m1), the coefficients of all l >= |m| of the pair as one run:
+  //   for m: for m1: for the pair's l >= |m| in ascending order: C_l[m1, m-m1]
+  std::vector<int> pair_table;  // (first triple, count, stream offset) per pair
+  {
+    const int pair_base = (int)(fwd.size() + back0.size() + back1.size());
+    bool ok = true;
+    int rows_max = 0;
+    size_t t0 = 0;
+    std::vector<std::vector<float>> tabs;
+    while (t0 < plan.triples.size()) {
+      size_t t1 = t0 + 1;
+      while (t1 < plan.triples.size() && plan.triples[t1].xi == plan.triples[t0].xi && plan.triples[t1].yi == plan.triples[t0].yi) t1++;
+      const StagedTriple &f = plan.triples[t0];
+      pair_table.push_back((int)t0);
+      pair_table.push_back((int)(t1 - t0));
+      pair_table.push_back(pair_base + (int)pairwise.size());
+      rows_max = std::max({rows_max, 2 * f.l1 + 1, 2 * f.l2 + 1, (int)(t1 - t0)});
+      tabs.clear();
+      const int L1 = 2 * f.l1 + 1, L2 = 2 * f.l2 + 1;
+      for (size_t t = t0; t < t1; t++) {
+        if (t > t0 && plan.triples[t].l <= plan.triples[t - 1].l) ok = false;
+        tabs.emplace_back((size_t)L1 * L2, 0.f);
+        cg_matrix_host(f.l1, f.l2, plan.triples[t].l, tabs.back().data());
+      }
+      const int ltop = plan.triples[t1 - 1].l;
+      for (int m = -ltop; m <= ltop; m++)
+        for (int m1 = std::max(-f.l1, m - f.l2); m1 <= std::min(f.l1, m + f.l2); m1++)
+          for (size_t t = t0; t < t1; t++)
+            if (plan.triples[t].l >= std::abs(m)) pairwise.push_back(tabs[t - t0][(size_t)(m1 + f.l1) * L2 + (m - m1 + f.l2)]);
+      t0 = t1;
+    }
+    plan.npairs = (int)pair_table.size() / 3;
+    plan.pair_cap = rows_max <= 16 ? 16 : 32;
+    plan.pairs_ok = ok && rows_max <= 32;
+  }
   bank = fwd;
   bank.insert(bank.end(), back0.begin(), back0.end());
   bank.insert(bank.end(), back1.begin(), back1.end());
+  bank.insert(bank.end(), pairwise.begin(), pairwise.end());
   bank.resize(bank.size() + 4 * kWave, 0.f);  // the kernels read the stream up to three registers of lanes ahead
   // stripes: the triples that feed one x part (resp. one y part)
   {
@@ -142,6 +185,8 @@ int get_plan(bool diag, const std::vector<VecTriple> &triples, const std::vector
     if (2 * lown + 1 > 32) ok = false;
     plan.stripes_ok = ok;
     plan.stripe_cap = 2 * lown + 1 <= 16 ? 16 : 32;
+    plan.pair_off = (int)tb.size();
+    tb.insert(tb.end(), pair_table.begin(), pair_table.end());
   }
   const size_t tri_bytes = plan.triples.size() * sizeof(StagedTriple);
   const size_t bank_bytes = bank.size() * sizeof(float);
@@ -184,6 +229,8 @@ void fill_args(StagedArgs &a, const DevicePlan &plan, const FastLists &f, const 
   a.triples = plan.d_triples;
   a.bank = plan.d_bank;
   a.stripes = plan.d_stripes;
+  a.pairs = plan.d_stripes + plan.pair_off;
+  a.npairs = plan.npairs;
   a.ncells = ncells;
   a.ntriples = (int)plan.triples.size();
   a.nx = (int)xs.size();
@@ -322,6 +369,26 @@ int run_bwd(bool diag, const std::vector<VecTriple> &triples, const std::vector<
   }
   const long long cell_bytes = 16LL * (plan->xsize + plan->ysize);  // operands + gradient images
   if (cell_bytes > kLdsLimit) return GELIB_HIP_OK;
+  // n2 <= 64 and power-of-two channel counts hold here; the pair-wise kernel also needs uniform slots per pair,
+  // which one pair always has
+  if (g_bwd_pairs && plan->pairs_ok) {
+    auto units = [&](long long c) {
+      long long n = 0;
+      for (int k = 0; k < plan->npairs; k++) n += (c * plan->triples[plan->stripes[plan->pair_off + 3 * k]].u + kWave - 1) / kWave;
+      return n;
+    };
+    long long cpb = 1;
+    while (cpb * 2 <= ncells && cell_bytes * cpb * 2 <= g_bwd_lds_target && units(cpb) < 8) cpb *= 2;
+    StagedArgs a;
+    fill_args(a, *plan, f, xs, ys, ncells, offs_add, accumulate);
+    a.cpb = (int)cpb;
+    const long long nblocks = (ncells + cpb - 1) / cpb;
+    if (nblocks > 0x7fffffffLL) return GELIB_HIP_ERR_ARG;
+    rc = launch_staged_pair_bwd(a, diag, want_x, want_y, plan->pair_cap, (int)nblocks, (size_t)(cell_bytes * cpb), s);
+    if (rc) return rc;
+    *used = 1;
+    return GELIB_HIP_OK;
+  }
   long long cpb = 1;
   while (cpb * 2 <= ncells && cell_bytes * cpb * 2 <= g_bwd_lds_target && units_per_block(*plan, cpb) < 16) cpb *= 2;
   const long long lds = cell_bytes * cpb;
@@ -426,6 +493,10 @@ int staged_set_option(const char *name, int value) {
   }
   if (!std::strcmp(name, "staged_bwd_stripes")) {
     g_bwd_stripes = value;
+    return GELIB_HIP_OK;
+  }
+  if (!std::strcmp(name, "staged_bwd_pairs")) {
+    g_bwd_pairs = value;
     return GELIB_HIP_OK;
   }
   if (!std::strcmp(name, "staged_bwd_threads")) {

@@ -143,7 +143,7 @@ int gelib_hip_synchronize(void);
  * "staged_fwd" / "staged_bwd" (1/0: use the family), "fwd_block_bytes", "fwd_lds_bytes", "fwd_tile",
  * "staged_fwd_tile" (1, 2, 4), "staged_fwd_threads", "staged_fwd_coeffs_lds" (1/0), "staged_fwd_lds_target",
  * "staged_bwd_lds_target", "staged_bwd_threads" (256, 512, 1024), "staged_bwd_stripes" (0 never, 1 where they pay,
- * 2 wherever they apply).  Unknown names return GELIB_HIP_ERR_ARG.  Options are process-wide.
+ * 2 wherever they apply), "staged_bwd_pairs" (1/0: pair-wise single-pass backward kernel, off by default).  Unknown names return GELIB_HIP_ERR_ARG.  Options are process-wide.
  * gelib_hip_last_path() tells which kernel family the last call of this thread used
  * (0 = none, 1 = generic, 2 = unrolled small-l kernels, 3 = staged any-l kernels).
  */

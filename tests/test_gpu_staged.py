@@ -17,18 +17,21 @@ torch = pytest.importorskip("torch")
 STAGED = 3
 
 
-@pytest.fixture(scope="module", params=["striped", "atomic"])
+@pytest.fixture(scope="module", params=["striped", "pairwise", "triplewise"])
 def cabi(request):
-    """Both backward forms of the family: one gradient per launch with sums in registers (the default where its
-    conditions hold), and both gradients in one launch with LDS float atomics."""
+    """The three backward forms of the family: one gradient per launch with sums in registers; both gradients in
+    one launch, one (x part, y part) pair at a time, contracting over l first; and both gradients in one launch,
+    one triple at a time.  Each is forced wherever its conditions hold (the library picks one of them by itself)."""
     assert torch.cuda.is_available(), "GPU tests need a GPU"
     from gelib_amd import cabi as c
     c.lib()
     c.set_option("force_generic", 0)
     c.set_option("staged_bwd_stripes", 2 if request.param == "striped" else 0)
+    c.set_option("staged_bwd_pairs", int(request.param == "pairwise"))
     yield c
     c.set_option("staged_bwd_threads", 0)
     c.set_option("staged_bwd_stripes", 1)
+    c.set_option("staged_bwd_pairs", 0)
 
 
 def c128(L):

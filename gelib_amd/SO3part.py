@@ -16,6 +16,15 @@ class SO3part(torch.Tensor):
     def randn(cls, b, l, n, device='cpu'):
         return SO3part(torch.randn([b, 2 * l + 1, n], dtype=torch.complex64, device=device))
 
+    @classmethod
+    def spharm(cls, l, X):
+        """Spherical harmonics of the vectors (x, y, z) in X, shaped (b, 3, n) float32
+        (python/src/gelib/SO3part.py:55-62)."""
+        assert X.dim() == 3
+        R = SO3part.zeros(X.size(0), l, X.size(2), device=X.device)
+        R.backend().add_spharm(X)
+        return R
+
     def zeros_like(self, *args):
         if not args:
             return SO3part(torch.zeros_like(self))

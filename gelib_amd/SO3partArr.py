@@ -22,6 +22,15 @@ class SO3partArr(torch.Tensor):
     def randn(b, adims, l, n, device='cpu'):
         return SO3partArr(torch.randn([b] + list(adims) + [2 * l + 1, n], dtype=torch.complex64, device=device))
 
+    @classmethod
+    def spharm(cls, l, X):
+        """Spherical harmonics of the vectors (x, y, z) in X, shaped (b, a_1..a_k, 3, n) float32
+        (python/src/gelib/SO3partArr.py:59-67)."""
+        assert X.size(-2) == 3
+        R = SO3partArr.zeros(X.size(0), list(X.size())[1:X.dim() - 2], l, X.size(-1), device=X.device)
+        R.backend().add_spharm(X)
+        return R
+
     def zeros_like(self, *args):
         if not args:
             return SO3partArr(torch.zeros_like(self))

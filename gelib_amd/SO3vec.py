@@ -31,6 +31,13 @@ class SO3vec:
         return R
 
     @classmethod
+    def spharm(cls, l, X):
+        """An SO3vec with the single part l holding the spherical harmonics of X (python/src/gelib/SO3vec.py)."""
+        R = SO3vec()
+        R.parts[l] = SO3part.spharm(l, X)
+        return R
+
+    @classmethod
     def zeros_like(cls, x):
         R = SO3vec()
         for l, p in x.parts.items():

@@ -119,6 +119,20 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
              Gpart_add_DiagCGproduct_back1(r, g, x, offs);
            },
            py::arg("g"), py::arg("x"), py::arg("offs") = 0)
+      .def("add_spharm",
+           [](SO3part<float> &r, at::Tensor &X) {
+             TORCH_CHECK(X.scalar_type() == at::kFloat, "GElib: add_spharm takes a float32 tensor of (x, y, z) vectors");
+             cnine::Gdims dims;
+             std::vector<size_t> strides;
+             for (int i = 0; i < X.dim(); i++) {
+               dims.push_back((int)X.size(i));
+               TORCH_CHECK(X.stride(i) >= 0, "GElib: negative strides are not supported");
+               strides.push_back((size_t)X.stride(i));
+             }
+             StreamGuard sg;
+             r.add_spharm(cnine::TensorView<float>(X.data_ptr<float>(), dims, cnine::GstridesB(strides), X.is_cuda() ? 1 : 0));
+           },
+           py::arg("X"))
       .def("getl", &SO3part<float>::getl)
       .def("getn", &SO3part<float>::getn)
       .def("str", &SO3part<float>::str, py::arg("indent") = "")

@@ -16,7 +16,7 @@ SYMBOLS = [
     "gelib_hip_so3part_cg_fwd", "gelib_hip_so3part_cg_back0", "gelib_hip_so3part_cg_back1",
     "gelib_hip_so3part_diagcg_fwd", "gelib_hip_so3part_diagcg_back0", "gelib_hip_so3part_diagcg_back1",
     "gelib_hip_so3vec_cg_fwd", "gelib_hip_so3vec_cg_bwd", "gelib_hip_so3vec_diagcg_fwd",
-    "gelib_hip_so3vec_diagcg_bwd", "gelib_hip_set_option", "gelib_hip_last_path",
+    "gelib_hip_so3vec_diagcg_bwd", "gelib_hip_so3part_spharm", "gelib_hip_set_option", "gelib_hip_last_path",
     "gelib_hip_malloc", "gelib_hip_free", "gelib_hip_memcpy", "gelib_hip_memset", "gelib_hip_synchronize",
 ]
 
@@ -59,6 +59,8 @@ def lib():
         for name in ("gelib_hip_so3vec_cg_bwd", "gelib_hip_so3vec_diagcg_bwd"):
             getattr(L, name).argtypes = [P, P, ctypes.c_int, P, ctypes.c_int, P, ctypes.c_int, P, ctypes.c_int,
                                          ctypes.c_void_p]
+        L.gelib_hip_so3part_spharm.argtypes = [P, ctypes.c_void_p, ctypes.POINTER(ctypes.c_int64),
+                                               ctypes.POINTER(ctypes.c_int64), ctypes.c_int, ctypes.c_void_p]
         L.gelib_hip_set_option.argtypes = [ctypes.c_char_p, ctypes.c_int]
         _lib = L
     return _lib
@@ -164,6 +166,21 @@ def so3vec_bwd(xgparts, ygparts, gparts, xparts, yparts, accumulate=True, diag=F
     fn = lib().gelib_hip_so3vec_diagcg_bwd if diag else lib().gelib_hip_so3vec_cg_bwd
     check(fn(_arr(xgparts), _arr(ygparts), len(gparts), _arr(gparts), len(xparts), _arr(xparts), len(yparts),
              _arr(yparts), int(accumulate), _stream(gparts[0])))
+
+
+def so3part_spharm(r, x, accumulate=True):
+    """r (b, [grid], 2l+1, n) complex64 (+)= spherical harmonics of the float32 vectors x (b or 1, [grid], 3, n)."""
+    import torch
+    if x.dtype != torch.float32:
+        raise TypeError("the vectors are float32")
+    if x.dim() != r.dim() or x.size(-2) != 3:
+        raise ValueError("x is shaped like r with 3 in place of 2l+1")
+    k = x.dim() - 3
+    dims = [x.shape[0]] + list(x.shape[1:1 + k]) + [1] * (2 - k) + list(x.shape[-2:])
+    strs = [x.stride(0)] + list(x.stride()[1:1 + k]) + [0] * (2 - k) + list(x.stride()[-2:])
+    A = ctypes.c_int64 * 5
+    check(lib().gelib_hip_so3part_spharm(ctypes.byref(desc(r)), ctypes.c_void_p(x.data_ptr()), A(*dims), A(*strs),
+                                         int(accumulate), _stream(r)))
 
 
 def set_option(name, value):

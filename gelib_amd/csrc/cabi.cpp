@@ -54,16 +54,16 @@ int check_desc(const gelib_part_desc *d, View &v) {
 
 // The farthest element of the view must lie inside the allocation that holds ptr, and that allocation must be
 // device (or managed) memory: a host pointer or an over-long view would otherwise fault the GPU.
-int check_pointer(const gelib_part_desc *d) {
-  if (!g_check_pointers || !d->ptr) return GELIB_HIP_OK;
+int check_range(const void *ptr, const int64_t dims[5], const int64_t strides[5], size_t elem_bytes) {
+  if (!g_check_pointers || !ptr) return GELIB_HIP_OK;
   long long span = 0;
   for (int k = 0; k < 5; k++) {
-    if (d->dims[k] == 0) return GELIB_HIP_OK;
-    if (d->strides[k] < 0) return GELIB_HIP_ERR_ARG;
-    span += (d->dims[k] - 1) * d->strides[k];
+    if (dims[k] == 0) return GELIB_HIP_OK;
+    if (strides[k] < 0) return GELIB_HIP_ERR_ARG;
+    span += (dims[k] - 1) * strides[k];
   }
   hipPointerAttribute_t attr;
-  hipError_t e = hipPointerGetAttributes(&attr, d->ptr);
+  hipError_t e = hipPointerGetAttributes(&attr, ptr);
   if (e != hipSuccess) {
     (void)hipGetLastError();
     return GELIB_HIP_ERR_DEVICE;
@@ -73,15 +73,17 @@ int check_pointer(const gelib_part_desc *d) {
   if (hipGetDevice(&dev) == hipSuccess && attr.type == hipMemoryTypeDevice && attr.device != dev) return GELIB_HIP_ERR_DEVICE;
   hipDeviceptr_t base = nullptr;
   size_t size = 0;
-  e = hipMemGetAddressRange(&base, &size, (hipDeviceptr_t)d->ptr);
+  e = hipMemGetAddressRange(&base, &size, (hipDeviceptr_t)ptr);
   if (e != hipSuccess) {
     (void)hipGetLastError();
     return GELIB_HIP_OK;  // range unknown (e.g. a suballocator the runtime cannot see): type check above stands
   }
-  const char *end = (const char *)d->ptr + (span + 1) * (long long)sizeof(float2);
+  const char *end = (const char *)ptr + (span + 1) * (long long)elem_bytes;
   if (end > (const char *)base + size) return GELIB_HIP_ERR_DEVICE;
   return GELIB_HIP_OK;
 }
+
+int check_pointer(const gelib_part_desc *d) { return check_range(d->ptr, d->dims, d->strides, sizeof(float2)); }
 
 PartDev to_dev(const gelib_part_desc *d, const long long E[3], long long own[3]) {
   PartDev p;
@@ -465,6 +467,35 @@ int gelib_hip_so3vec_diagcg_bwd(const gelib_part_desc *xg, const gelib_part_desc
                                 const gelib_part_desc *g, int nx, const gelib_part_desc *x, int ny,
                                 const gelib_part_desc *y, int accumulate, void *stream) {
   return vec_bwd_entry(true, xg, yg, ng, g, nx, x, ny, y, accumulate, stream);
+}
+
+int gelib_hip_so3part_spharm(const gelib_part_desc *r, const float *x, const int64_t xdims[5],
+                             const int64_t xstrides[5], int accumulate, void *stream) {
+  t_last_path = kPathNone;
+  View R;
+  int rc = check_desc(r, R);
+  if (rc) return rc;
+  if (!xdims || !xstrides) return GELIB_HIP_ERR_NULL;
+  if (xdims[3] != 3 || xdims[4] != R.n) return GELIB_HIP_ERR_ARG;  // (.., 3, n) vectors, one per channel
+  long long D[3], xs[5];
+  for (int k = 0; k < 3; k++) {
+    D[k] = r->dims[k];
+    if (xdims[k] != r->dims[k] && xdims[k] != 1) return k == 0 ? GELIB_HIP_ERR_BATCH : GELIB_HIP_ERR_GRID;
+    xs[k] = (xdims[k] == r->dims[k] && r->dims[k] > 1) ? xstrides[k] : 0;
+  }
+  xs[3] = xstrides[3];
+  xs[4] = xstrides[4];
+  const bool empty = D[0] * D[1] * D[2] == 0 || R.n == 0;
+  if (empty) return GELIB_HIP_OK;
+  if (!x) return GELIB_HIP_ERR_NULL;
+  for (int k = 0; k < 3; k++)
+    if (r->dims[k] > 1 && r->strides[k] == 0) return GELIB_HIP_ERR_BROADCAST_DEST;
+  if ((rc = check_pointer(r)) || (rc = check_range(x, xdims, xstrides, sizeof(float)))) return rc;
+  long long own[3];
+  const long long E[3] = {D[0], D[1], D[2]};
+  PartDev pr = to_dev(r, E, own);
+  t_last_path = kPathGeneric;
+  return launch_spharm(pr, x, xs, D, R.l, R.n, accumulate != 0, (hipStream_t)stream);
 }
 
 int gelib_hip_malloc(void **ptr, uint64_t bytes) {

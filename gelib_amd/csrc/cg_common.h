@@ -51,4 +51,8 @@ int launch_generic_back0(const PartOp &op, bool accumulate, hipStream_t s);  // 
 int launch_generic_back1(const PartOp &op, bool accumulate, hipStream_t s);  // destination = op.y
 int launch_zero_fill(const PartDev &d, const long long D[3], int M, int n, hipStream_t s);
 
+// ---- spherical harmonics (spharm.hip): xs = strides of x in floats over (batch, grid0, grid1, xyz, channel) ----
+int launch_spharm(const PartDev &r, const float *x, const long long xs[5], const long long D[3], int L, int n,
+                  bool accumulate, hipStream_t s);
+
 }  // namespace gelib_hip

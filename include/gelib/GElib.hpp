@@ -300,6 +300,37 @@ class SO3part : public cnine::BatchedTensor<std::complex<TYPE>>, public GpartBas
     gelib_check(gelib_hip_so3part_diagcg_back1(&YG, &G, &X, offs, 1, gelib_stream()));
   }
 
+  // ---- spherical harmonics (SO3/SO3part.hpp:340-403): x is (.., 3, n) real, leading dims as this part's or 1 ----
+  void add_spharm(const cnine::TensorView<float> &x) const {
+    GELIB_ASSRT(x.get_dev() == dev);
+    if (dev != 1) GELIB_ERROR("SO3part::add_spharm: the operands must be on GPU");
+    const int d = ndims(), xd = x.ndims();
+    if (xd < 2) GELIB_ERROR("x must be at least 2D.");
+    if (x.dim(xd - 2) != 3) GELIB_ERROR("dim(-2) of x must be 3.");
+    gelib_part_desc R = descriptor();
+    // x without leading dimensions is shared by every cell (cuda/SPharm.cu:101-107)
+    int64_t xdims[5] = {1, 1, 1, 3, x.dim(xd - 1)};
+    int64_t xstr[5] = {0, 0, 0, (int64_t)x.strides[xd - 2], (int64_t)x.strides[xd - 1]};
+    if (xd > 2) {
+      if (xd != d) GELIB_ERROR("x must have as many leading dimensions as the part.");
+      xdims[0] = x.dim(0);
+      xstr[0] = (int64_t)x.strides[0];
+      const int ng = xd - 3;
+      if (ng == 1 || ng == 2) {
+        for (int k = 0; k < ng; k++) xdims[1 + k] = x.dim(1 + k), xstr[1 + k] = (int64_t)x.strides[1 + k];
+      } else if (ng > 2) {  // fused like the part's own grid dimensions
+        int64_t tot = 1;
+        for (int k = 1; k <= ng; k++) tot *= x.dim(k);
+        for (int k = 1; k < ng; k++)
+          if (x.strides[k] != (size_t)x.dim(k + 1) * x.strides[k + 1])
+            GELIB_ERROR("the grid dimensions of x must be fusible when there are more than two of them");
+        xdims[1] = tot;
+        xstr[1] = (int64_t)x.strides[ng];
+      }
+    }
+    gelib_check(gelib_hip_so3part_spharm(&R, x.arr, xdims, xstr, 1, gelib_stream()));
+  }
+
   std::string classname() const { return "GElib::SO3part"; }
   std::string repr() const {
     std::ostringstream oss;

@@ -123,6 +123,16 @@ int gelib_hip_so3vec_diagcg_bwd(const gelib_part_desc *xg, const gelib_part_desc
                                 const gelib_part_desc *g, int nx, const gelib_part_desc *x, int ny,
                                 const gelib_part_desc *y, int accumulate, void *stream);
 
+/* ---- producer of the usual second operand: spherical harmonics ----------------------------------------------------------
+ * r[.., l+m, j] += Y_l^m(x[.., :, j] / |x[.., :, j]|), m = -l..l, l read from r's dims[3].  x is float32 viewed 5-D
+ * (batch, grid0, grid1, 3, channels) with strides in floats; leading dimensions of extent 1 broadcast.  A vector on
+ * the polar axis contributes only m = 0, as in the reference.  accumulate == 0 overwrites r.  The Legendre values
+ * are the reference's unnormalised floats, so like the reference the result overflows float32 from l = 30 on.
+ * Replaces addSPharm_cu(r, x, stream) (cuda/SPharm.cu:88-123; CPU form SO3/SO3part.hpp:340-403) without its limits of
+ * 1024 channels and n(l+1)(l+2)/2 floats of shared memory. */
+int gelib_hip_so3part_spharm(const gelib_part_desc *r, const float *x, const int64_t xdims[5],
+                             const int64_t xstrides[5], int accumulate, void *stream);
+
 /*
  * Device memory helpers for host code that does not include the HIP headers itself (the C++ mirror of the
  * reference's classes uses them where the reference relies on cnine's device transport, e.g. the

@@ -15,6 +15,10 @@
  *                                                    stride 0 for a broadcast operand, core/Gpart.hpp:168-185)
  *   vec-level loops       core/Gvec.hpp:311-345, core/Gvec.hpp:358-389 (triple enumeration, running offsets)
  *   type arithmetic       core/Gtype.hpp:115-138, SO3/SO3group.hpp:43-47
+ *   ora_spharm            SO3/SO3part.hpp:340-403   (add_spharm: Legendre table in float, phase recurrence in
+ *                                                    complex<float>; pinned by scipy's spherical harmonics -- the
+ *                                                    reference's own check, python/tests/test_spharm.py -- and the
+ *                                                    printed example python/docs/source/abandoned/SO3part.rst:170-176)
  *
  * How the oracle is pinned (see tests/test_oracle_*.py): coefficients against exact sympy values,
  * the printed table in python/docs/source/SO3CG.rst:51-53, orthogonality and symmetry identities;
@@ -334,6 +338,64 @@ int ora_vec_op(int op, int prec, int nx, const ora_part *xparts, int ny, const o
       }
     }
   }
+  return 0;
+}
+
+/*
+ * r[b, L+m, j] += Y_L^m(x[b,:,j] / |x[b,:,j]|) for every cell b and channel j (SO3/SO3part.hpp:340-403).
+ * x is (B or 1, 3, n) float32 with strides (xsb, xsm, 1) in floats (xsb = 0 broadcasts one set of vectors over the
+ * batch); r is (B, 2L+1, n) complex64, packed.  The arithmetic keeps the reference's types: the associated
+ * Legendre table is float, each entry computed from a double expression; the phase runs in complex<float>.
+ */
+int ora_spharm(int L, long long B, long long n, const float *x, long long xsb, long long xsm, float *r) {
+  if (L < 0 || L > ORA_MAXL) return 1;
+  const int W = L + 1;
+  float *P = (float *)malloc(sizeof(float) * (size_t)W * W);
+  if (!P) return 1;
+  for (long long b = 0; b < B; b++) {
+    float *rb = r + 2 * b * (2 * L + 1) * n;
+    const float *xb = x + b * xsb;
+    for (long long j = 0; j < n; j++) {
+      const float vx = xb[j], vy = xb[xsm + j], vz = xb[2 * xsm + j];
+      const float length = sqrtf(vx * vx + vy * vy + vz * vz);
+      const float len2 = sqrtf(vx * vx + vy * vy);
+      if (len2 == 0 || isnan(vx / len2) || isnan(vy / len2)) {
+        rb[2 * (L * n + j)] += (float)sqrt(((float)(2 * L + 1)) / (M_PI * 4.0));
+        continue;
+      }
+      const float xx = vz / length;
+      memset(P, 0, sizeof(float) * (size_t)W * W);
+      P[0] = 1;
+      const float xfact = (float)sqrt(1.0 - xx * xx);
+      for (int l = 1; l <= L; l++) {
+        P[l * W + l] = (float)(-(2.0 * l - 1.0) * xfact * P[(l - 1) * W + (l - 1)]);
+        P[l * W + l - 1] = (float)((2.0 * l - 1.0) * P[(l - 1) * W + (l - 1)] * xx);
+        for (int m = 0; m < l - 1; m++)
+          P[l * W + m] = (float)(((2.0 * l - 1.0) * P[(l - 1) * W + m] * xx - ((float)(l + m - 1.0)) * (P[(l - 2) * W + m])) /
+                                 ((float)(l - m)));
+      }
+      const float cr = vx / len2, ci = vy / len2;
+      float pr = (float)sqrt((2.0 * L + 1.0) / (M_PI * 4.0)), pi = 0.f;
+      for (int m = 0; m <= L; m++) {
+        const float ar = pr * P[L * W + m], ai = pi * P[L * W + m];
+        rb[2 * ((L + m) * n + j)] += ar;
+        rb[2 * ((L + m) * n + j) + 1] += ai;
+        if (m > 0) {
+          const float sg = (float)(1 - 2 * (m % 2));
+          rb[2 * ((L - m) * n + j)] += sg * ar;
+          rb[2 * ((L - m) * n + j) + 1] += sg * (-ai);
+        }
+        if (m < L) {
+          const float d = sqrtf((float)(L - m) * (L + m + 1));
+          const float qr = cr / d, qi = ci / d;
+          const float nr = pr * qr - pi * qi, ni = pr * qi + pi * qr;
+          pr = nr;
+          pi = ni;
+        }
+      }
+    }
+  }
+  free(P);
   return 0;
 }
 

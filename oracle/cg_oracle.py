@@ -164,3 +164,20 @@ def vec_bwd(gparts, xparts, yparts, diag=False, nthreads=1):
     vec_op(DIAG_BACK0 if diag else CG_BACK0, gparts, xg, yparts, nthreads)
     vec_op(DIAG_BACK1 if diag else CG_BACK1, gparts, xparts, yg, nthreads)
     return xg, yg
+
+
+def spharm(l, x, batch=None):
+    """(B or 1, 3, n) float32 vectors -> (B, 2l+1, n) complex64 spherical harmonics, the reference's add_spharm into zeros."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    assert x.ndim == 3 and x.shape[1] == 3
+    B = batch or x.shape[0]
+    assert x.shape[0] in (1, B)
+    r = np.zeros((B, 2 * l + 1, x.shape[2]), dtype=np.complex64)
+    f = lib().ora_spharm
+    f.restype = ctypes.c_int
+    f.argtypes = [ctypes.c_int, ctypes.c_longlong, ctypes.c_longlong, ctypes.c_void_p, ctypes.c_longlong,
+                  ctypes.c_longlong, ctypes.c_void_p]
+    xsb = 0 if x.shape[0] == 1 else 3 * x.shape[2]   # one set of vectors is shared by the whole batch
+    rc = f(l, B, x.shape[2], x.ctypes.data, xsb, x.shape[2], r.ctypes.data)
+    assert rc == 0
+    return r

@@ -85,6 +85,7 @@ VEC_CASES = [
     (2, {6: 16}, {5: 16}, 8),                                        # 256 slots per cell: several runs per cell
     (3, {5: 2, 6: 4}, {5: 4, 6: 8}, 7),                              # channel counts differ between parts
     (2, {12: 2}, {3: 4}, -1),                                        # own l = 12: 25 rows, the 32-row variant
+    (3, {5: 4, 9: 4}, {5: 4}, 3),                                    # x part l = 9 feeds nothing (l >= 4 is cut): zero gradient
 ]
 
 

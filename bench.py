@@ -23,10 +23,10 @@ HBM_PEAK = 8.0e12  # B/s, MI355X HBM3E
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs, each scaled by what the
 # counter reads for a plain 1 GiB copy: x2.000 and x1.000); summary in profiles/.
 MEASURED_TRAFFIC = {
-    "so3vec_cg_L4_tau16_B32768_maxl4": {"so3vec_fwd": 26221108310, "so3vec_bwd": 26008901737},
+    "so3vec_cg_L4_tau16_B32768_maxl4": {"so3vec_fwd": 26221027505, "so3vec_bwd": 25876776855},
     # the backward pass of this type runs as two launches (one per gradient), each reading g: 1.88 x algorithmic
-    "so3vec_diagcg_L6_n64_B131072": {"so3vec_fwd": 102040514571, "so3vec_bwd": 203991472933},
-    "so3part_cg_10x10_all_l_n8_B16384": {"so3vec_fwd": 3746895112, "so3vec_bwd": 3809656495},
+    "so3vec_diagcg_L6_n64_B131072": {"so3vec_fwd": 102052404553, "so3vec_bwd": 204010468818},
+    "so3part_cg_10x10_all_l_n8_B16384": {"so3vec_fwd": 3747009028, "so3vec_bwd": 3809547747},
 }
 
 WORKLOADS = {

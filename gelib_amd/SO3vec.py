@@ -83,6 +83,10 @@ class SO3vec:
         assert list(self.parts.keys()) == list(y.parts.keys())
         return SO3vec(*[self.parts[l] + y.parts[l] for l in self.parts.keys()])
 
+    def __mul__(self, y):
+        """Multiply every part by the matching weight matrix of an SO3weights (python/src/gelib/SO3vec.py:174-177)."""
+        return SO3vec(*[torch.matmul(p, w) for p, w in zip(self.parts.values(), y.parts)])
+
     def CGproduct(self, y, maxl=-1):
         xparts = list(self.parts.values())
         yparts = list(y.parts.values())

@@ -113,6 +113,10 @@ class SO3vecArr:
     def dtype(self):
         return self.parts[min(self.parts)].dtype if self.parts else torch.cfloat
 
+    def __mul__(self, y):
+        """Multiply every part by the matching weight matrix of an SO3weights (python/src/gelib/SO3vec.py:174-177)."""
+        return SO3vecArr(*[torch.matmul(p, w) for p, w in zip(self.parts.values(), y.parts)])
+
     def CGproduct(self, y, maxl=-1):
         assert isinstance(y, SO3vecArr)
         maxl = -1 if maxl is None else maxl

@@ -9,10 +9,12 @@ gelib_amd.gelib_base; tensors must live on the GPU.  Nothing here falls back to 
 """
 from gelib_amd.gelib_common import common_batch  # noqa: F401
 from gelib_amd.SO3element import SO3element, SO3irrep  # noqa: F401
+from gelib_amd.SO3type import SO3type  # noqa: F401
 from gelib_amd.SO3part import SO3part, SO3part_CGproductFn, SO3part_DiagCGproductFn  # noqa: F401
 from gelib_amd.SO3vec import SO3vec, SO3vec_CGproductFn, SO3vec_DiagCGproductFn  # noqa: F401
 from gelib_amd.SO3partArr import SO3partArr, SO3partArr_CGproductFn, SO3partArr_DiagCGproductFn  # noqa: F401
 from gelib_amd.SO3vecArr import SO3vecArr, SO3vecArr_CGproductFn, SO3vecArr_DiagCGproductFn  # noqa: F401
+from gelib_amd.SO3weights import SO3weights, SO3linear  # noqa: F401
 
 
 def CGproduct(x, y, maxl=-1):

@@ -154,3 +154,30 @@ def test_errors_are_exceptions(G):
         G.DiagCGproduct(xc, G.SO3part.randn(2, 1, 5, device="cuda"), 1)
     with pytest.raises((RuntimeError, AssertionError)):
         G.CGproduct(G.SO3part.randn(3, 1, 4, device="cuda"), xc, 1)
+
+
+def test_product_then_linear_layer(G):
+    """CGproduct followed by the channel-mixing layer (SO3vec * SO3weights), gradients through both: the loss is
+    linear in the weights and bilinear in (x, y), so finite differences are exact up to rounding."""
+    tau = G.SO3type({l: 4 for l in range(3)})
+    x = G.SO3vec.randn(5, tau, device="cuda")
+    y = G.SO3vec.randn(5, tau, device="cuda")
+    x.requires_grad_()
+    tau_mid = tau.CGproduct(tau, 2)
+    tau_out = G.SO3type({l: 3 for l in range(3)})
+    W = G.SO3weights.randn(tau_mid, tau_out, device="cuda").requires_grad_()
+
+    def net(x, y, W):
+        return G.CGproduct(x, y, maxl=2) * W
+
+    out = net(x, y, W)
+    assert out.tau() == dict(tau_out)
+    test_vec = G.SO3vec.randn_like(out)
+    loss = out.odot(test_vec)
+    loss.backward(torch.tensor(1.0, device="cuda"))
+    Weps = G.SO3weights(*[torch.randn_like(w) for w in W.parts])
+    W2 = G.SO3weights(*[w.detach() + e for w, e in zip(W.parts, Weps.parts)])
+    dW = sum(torch.sum(torch.view_as_real(e) * torch.view_as_real(w.grad)) for e, w in zip(Weps.parts, W.parts))
+    assert torch.allclose(net(x, y, W2).odot(test_vec) - loss, dW, rtol=1e-3, atol=1e-2)
+    xeps = G.SO3vec.randn_like(x)
+    assert torch.allclose(net(x + xeps, y, W).odot(test_vec) - loss, xeps.odot(x.get_grad()), rtol=1e-3, atol=1e-2)

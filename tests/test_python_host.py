@@ -79,3 +79,20 @@ def test_arr_surface():
         G.CGproduct(p, p, 2)                          # host tensors are refused, not computed elsewhere
     with pytest.raises(RuntimeError):
         G.CGproduct(v, v)
+
+
+def test_type_and_weights():
+    import gelib_amd as G
+    t = G.SO3type({0: 2, 1: 2})
+    assert t.CGproduct(t) == {0: 8, 1: 12, 2: 4} and isinstance(t.CGproduct(t), G.SO3type)
+    assert G.SO3type({0: 1, 1: 1, 2: 1}).DiagCGproduct(G.SO3type({0: 1, 1: 1, 2: 1}), 1) == {0: 3, 1: 6}
+    tau_in, tau_out = G.SO3type({0: 3, 1: 2}), G.SO3type({0: 5, 1: 4})
+    W = G.SO3weights.randn(tau_in, tau_out)
+    x = G.SO3vec.randn(2, tau_in)
+    y = x * W                                        # plain torch matmuls: also defined on the host
+    assert y.tau() == {0: 5, 1: 4}
+    assert torch.allclose(y.parts[1], torch.matmul(x.parts[1], W.parts[1]))
+    lin = G.SO3linear(tau_in, tau_out)
+    assert len(list(lin.parameters())) == 2 and lin(x).tau() == {0: 5, 1: 4}
+    xa = G.SO3vecArr.randn(2, [3], tau_in)
+    assert (xa * W).tau() == {0: 5, 1: 4} and (xa * W).get_adims() == [3]

@@ -48,7 +48,9 @@ struct PairRec {
   int cg_base;       // offset (floats) of this pair's tables in the bank that follows the pair array
   int cg_len;        // floats of coefficient tables belonging to this pair
   int xoff, yoff;    // offsets (complex elements) of the parts inside a per-cell packed x / y image (backward)
-  int log2_u;        // log2 of the channel slots per cell (n1*n2, or n for Diag) when that is a power of two, else -1
+  int log2_u;        // log2 of the lane slots per cell: n1p*n2p (Diag: n1p) with n1p, n2p the channel counts rounded up
+                     // to powers of two; -1 when that exceeds 2^20
+  int lg_n2p;        // log2 of n2p
 };
 
 // Helpers shared by the kernel families that need contiguous channels and one cell index (cg_unrolled_plan.cpp).

@@ -1,4 +1,4 @@
-// Dispatch of the unrolled backward kernels; the instantiations live in cg_unrolled_bwd_{cg,diag}{4,8}.hip so
+// Dispatch of the unrolled backward kernels; the instantiations live in cg_unrolled_bwd_{cg,diag}{4,8}[_pad].hip so
 // that they compile in parallel.
 #include "cg_unrolled_dev.h"
 
@@ -8,6 +8,10 @@ int launch_unrolled_bwd_cg4(const BwdArgs &a, int nblocks, size_t lds_bytes, hip
 int launch_unrolled_bwd_cg8(const BwdArgs &a, int nblocks, size_t lds_bytes, hipStream_t s);
 int launch_unrolled_bwd_diag4(const BwdArgs &a, int nblocks, size_t lds_bytes, hipStream_t s);
 int launch_unrolled_bwd_diag8(const BwdArgs &a, int nblocks, size_t lds_bytes, hipStream_t s);
+int launch_unrolled_bwd_cg4_pad(const BwdArgs &a, int nblocks, size_t lds_bytes, hipStream_t s);
+int launch_unrolled_bwd_cg8_pad(const BwdArgs &a, int nblocks, size_t lds_bytes, hipStream_t s);
+int launch_unrolled_bwd_diag4_pad(const BwdArgs &a, int nblocks, size_t lds_bytes, hipStream_t s);
+int launch_unrolled_bwd_diag8_pad(const BwdArgs &a, int nblocks, size_t lds_bytes, hipStream_t s);
 
 size_t unrolled_bwd_lds_bytes(int bank_len, int xsize, int ysize, int cells_per_block) {
   const int waves = kBlock / kWave;
@@ -18,6 +22,12 @@ size_t unrolled_bwd_lds_bytes(int bank_len, int xsize, int ysize, int cells_per_
 // lcap: largest l present in the gradient; code for l above 4 is left out when the product is capped there
 int launch_unrolled_bwd(const BwdArgs &a, bool diag, int lcap, int nblocks, size_t lds_bytes, hipStream_t s) {
   if (nblocks <= 0) return GELIB_HIP_OK;
+  if (a.padded) {
+    if (diag) return lcap <= kLT ? launch_unrolled_bwd_diag4_pad(a, nblocks, lds_bytes, s)
+                                 : launch_unrolled_bwd_diag8_pad(a, nblocks, lds_bytes, s);
+    return lcap <= kLT ? launch_unrolled_bwd_cg4_pad(a, nblocks, lds_bytes, s)
+                       : launch_unrolled_bwd_cg8_pad(a, nblocks, lds_bytes, s);
+  }
   if (diag) return lcap <= kLT ? launch_unrolled_bwd_diag4(a, nblocks, lds_bytes, s)
                                : launch_unrolled_bwd_diag8(a, nblocks, lds_bytes, s);
   return lcap <= kLT ? launch_unrolled_bwd_cg4(a, nblocks, lds_bytes, s)

@@ -69,7 +69,9 @@ __device__ __forceinline__ LanePos lane_pos(int run, int lane, int log2_u, int n
 // and then feeds both gradients once per (m1,m2):  ax[m1] += Q conj(y[m2]),  ay[m2] += Q conj(x[m1]).
 // That is 2 instructions per term plus 8 per (m1,m2) instead of 10 per term.  An l of the pair whose part is absent
 // reads a row of zeros and a table of zeros (zrows, Zc) instead, so the code has no branches.
-template <int L1, int L2, int LCAP, bool DIAG, bool WX, bool WY>
+// PAD: channel counts are not all powers of two.  Lane slots are then n1p x n2p with the counts rounded up; a lane
+// whose (i, j) lies beyond the real channels reads channel 0, has its g forced to zero and never writes.
+template <int L1, int L2, int LCAP, bool DIAG, bool WX, bool WY, bool PAD>
 __device__ __forceinline__ void pair_bwd(const GParts<LCAP> &gp, PairPtr pr, CoeffPtr Cs, CoeffPtr Zc, GlobalRows zrows,
                                          const float2 *xs, const float2 *ys, float2 *xacc, float2 *yacc, int xsize,
                                          int ysize, long long cell0, int offs_add, const LanePos q) {
@@ -80,9 +82,13 @@ __device__ __forceinline__ void pair_bwd(const GParts<LCAP> &gp, PairPtr pr, Coe
   // scalar loads: the record sits in constant memory and the pointer is uniform
   const __attribute__((address_space(4))) PairRec &p = *pr;
   const int N1 = p.n1, N2 = p.n2;
-  const int lg_n2 = DIAG ? 0 : 31 - __clz(N2);
-  const int i = DIAG ? q.u : (q.u >> lg_n2);
-  const int j = DIAG ? q.u : (q.u & (N2 - 1));
+  const int lg_n2 = DIAG ? 0 : p.lg_n2p;
+  const int N2P = 1 << lg_n2;  // lanes per group that share i
+  int i = DIAG ? q.u : (q.u >> lg_n2);
+  int j = DIAG ? q.u : (q.u & (N2P - 1));
+  const bool valid = !PAD || (i < N1 && (DIAG || j < N2));
+  if (PAD && !valid) i = 0, j = 0;
+  const int chan = DIAG ? i : (PAD ? i * N2 + j : q.u);  // the lane's channel inside the triple's block
   const int span = p.log2_u < 6 ? (1 << p.log2_u) : kWave;  // lanes of a run that belong to one cell
   const long long cell = cell0 + q.cell_local;
 
@@ -109,7 +115,7 @@ __device__ __forceinline__ void pair_bwd(const GParts<LCAP> &gp, PairPtr pr, Coe
     constexpr int dl = decltype(dl_c)::value;
     const bool present = p.ri[dl] >= 0;
     const FastPart G = gp.G[LMIN + dl];
-    gptr[dl] = present ? (GlobalRows)G.ptr + cell * G.sb + (p.offs[dl] + offs_add + q.u) : zrows;
+    gptr[dl] = present ? (GlobalRows)G.ptr + cell * G.sb + (p.offs[dl] + offs_add + chan) : zrows;
     gsm[dl] = present ? G.sm : 0;
     cl[dl] = present ? Cs + p.cg[dl] : Zc;
   });
@@ -122,7 +128,7 @@ __device__ __forceinline__ void pair_bwd(const GParts<LCAP> &gp, PairPtr pr, Coe
       constexpr int L = LMIN + dl;
       if constexpr (L >= cabs_(m)) {
         const v2f t = gptr[dl][(m + L) * gsm[dl]];
-        dst[dl] = make_float2(t.x, t.y);
+        dst[dl] = (PAD && !valid) ? make_float2(0.f, 0.f) : make_float2(t.x, t.y);
       }
     });
   };
@@ -179,8 +185,8 @@ __device__ __forceinline__ void pair_bwd(const GParts<LCAP> &gp, PairPtr pr, Coe
   for (int m2 = 0; m2 <= 2 * L2; m2++) asm volatile("" : "+v"(ay[m2].x), "+v"(ay[m2].y));
 
   if (WX) {
-    if (!DIAG) group_sum(ax, N2);
-    if (q.live && (DIAG || j == 0)) {
+    if (!DIAG) group_sum(ax, N2P);
+    if (q.live && valid && (DIAG || j == 0)) {
       float2 *xa = xacc + q.cell_local * xsize + p.xoff + i;
 #pragma unroll
       for (int m1 = 0; m1 <= 2 * L1; m1++) {
@@ -192,8 +198,8 @@ __device__ __forceinline__ void pair_bwd(const GParts<LCAP> &gp, PairPtr pr, Coe
     }
   }
   if (WY) {
-    if (!DIAG) stride_sum(ay, N2, span);
-    if (q.live && (DIAG || (q.u & (span - 1)) < N2)) {
+    if (!DIAG) stride_sum(ay, N2P, span);
+    if (q.live && valid && (DIAG || (q.u & (span - 1)) < N2P)) {
       float2 *ya = yacc + q.cell_local * ysize + p.yoff + j;
 #pragma unroll
       for (int m2 = 0; m2 <= 2 * L2; m2++) {
@@ -248,7 +254,7 @@ __device__ __forceinline__ void copy_image(const FastPart (&parts)[kFastIn], con
   });
 }
 
-template <int LCAP, bool DIAG, bool WX, bool WY>
+template <int LCAP, bool DIAG, bool WX, bool WY, bool PAD>
 __global__ void __launch_bounds__(kBlock) unrolled_bwd_kernel(const BwdArgs a) {
   constexpr int KR = 2 * LCAP + 1;
   extern __shared__ float lds[];
@@ -293,7 +299,7 @@ __global__ void __launch_bounds__(kBlock) unrolled_bwd_kernel(const BwdArgs a) {
       switch (p->l1 * (kLT + 1) + p->l2) {
 #define GELIB_CASE(A, B)                                                                                      \
   case A * (kLT + 1) + B:                                                                                     \
-    pair_bwd<A, B, LCAP, DIAG, WX, WY>(gp, p, C, Zc, zrows, xs, ys, xacc, yacc, xsize, ysize, cell0, offs_add, q); \
+    pair_bwd<A, B, LCAP, DIAG, WX, WY, PAD>(gp, p, C, Zc, zrows, xs, ys, xacc, yacc, xsize, ysize, cell0, offs_add, q); \
     break;
 #define GELIB_ROW(A) GELIB_CASE(A, 0) GELIB_CASE(A, 1) GELIB_CASE(A, 2) GELIB_CASE(A, 3) GELIB_CASE(A, 4)
         GELIB_ROW(0) GELIB_ROW(1) GELIB_ROW(2) GELIB_ROW(3) GELIB_ROW(4)
@@ -309,9 +315,9 @@ __global__ void __launch_bounds__(kBlock) unrolled_bwd_kernel(const BwdArgs a) {
   if (WY) copy_image<false>(a.yg, a.yrows, a.ny, yacc_all, ysize, cell0, ncell, kWaves, cpb * ysize, a.accumulate != 0);
 }
 
-template <int LCAP, bool DIAG, bool WX, bool WY>
+template <int LCAP, bool DIAG, bool WX, bool WY, bool PAD>
 int launch_variant(const BwdArgs &a, int nblocks, size_t lds, hipStream_t s) {
-  auto kern = unrolled_bwd_kernel<LCAP, DIAG, WX, WY>;
+  auto kern = unrolled_bwd_kernel<LCAP, DIAG, WX, WY, PAD>;
   static bool attr_set = false;  // benign race: setting the attribute twice is harmless
   if (!attr_set) {
     GELIB_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -324,13 +330,13 @@ int launch_variant(const BwdArgs &a, int nblocks, size_t lds, hipStream_t s) {
 }
 
 // want_x / want_y select which gradients are computed
-template <int LCAP, bool DIAG>
+template <int LCAP, bool DIAG, bool PAD>
 int launch_bwd_variants(const BwdArgs &a, int nblocks, size_t lds_bytes, hipStream_t s) {
   static_assert(kLT == 4, "the case table above lists l1, l2 = 0..4");
   const bool wx = a.want_x != 0, wy = a.want_y != 0;
-  if (wx && wy) return launch_variant<LCAP, DIAG, true, true>(a, nblocks, lds_bytes, s);
-  if (wx) return launch_variant<LCAP, DIAG, true, false>(a, nblocks, lds_bytes, s);
-  return launch_variant<LCAP, DIAG, false, true>(a, nblocks, lds_bytes, s);
+  if (wx && wy) return launch_variant<LCAP, DIAG, true, true, PAD>(a, nblocks, lds_bytes, s);
+  if (wx) return launch_variant<LCAP, DIAG, true, false, PAD>(a, nblocks, lds_bytes, s);
+  return launch_variant<LCAP, DIAG, false, true, PAD>(a, nblocks, lds_bytes, s);
 }
 
 }  // namespace

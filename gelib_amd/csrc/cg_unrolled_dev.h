@@ -37,6 +37,7 @@ struct BwdArgs {
   int accumulate;
   int want_x, want_y;
   int bank_len;     // floats
+  int padded;       // some channel count is not a power of two (lanes beyond the real channels idle)
   int zero_off;     // even offset (floats) in the bank of a run of zeros as long as the largest coefficient table
   int xsize, ysize; // complex elements of one cell's packed x / y image
   int xrows[kFastIn], yrows[kFastIn];  // 2l+1 of each x / y part

@@ -24,6 +24,7 @@ struct DevicePlan {
   float *d_bank = nullptr;
   int bank_len = 0;
   int zero_off = 0;  // a run of zeros in the bank (stand-in table and stand-in row for absent parts)
+  bool padded = false;  // some channel count is not a power of two: the backward pass runs the padded kernels
   int xsize = 0, ysize = 0;
 };
 
@@ -139,8 +140,13 @@ int get_plan(bool diag, const std::vector<VecTriple> &triples, const std::vector
       for (int d = 0; d < kMaxDl; d++) rec.ri[d] = -1;
       rec.cg_base = (int)bank.size();
       {
-        const long long U = diag ? rec.n1 : (long long)rec.n1 * rec.n2;
-        rec.log2_u = (U > 0 && (U & (U - 1)) == 0 && U <= (1 << 20)) ? ilog2((int)U) : -1;
+        // lane slots: channel counts rounded up to powers of two (the backward lane sums need aligned groups);
+        // slots beyond the real channels are idle lanes of the padded kernels
+        const int lg1 = ilog2(std::max(1, rec.n1)), lg2 = ilog2(std::max(1, rec.n2));
+        const int lgu = diag ? lg1 : lg1 + lg2;
+        rec.lg_n2p = lg2;
+        rec.log2_u = lgu <= 20 ? lgu : -1;
+        if (!is_pow2(rec.n1) || (!diag && !is_pow2(rec.n2))) plan.padded = true;
       }
       rec.xoff = xoff[t.xi];
       rec.yoff = yoff[t.yi];
@@ -246,15 +252,16 @@ int run_bwd(bool diag, const std::vector<VecTriple> &triples, const std::vector<
             const std::vector<std::pair<int, int>> &ys, const std::vector<int> &rls, const FastLists &f,
             long long ncells, int offs_add, bool accumulate, bool want_x, bool want_y, hipStream_t s, int *used) {
   *used = 0;
-  // channel counts must be powers of two and the reduced operand must fit a wave
+  // lane slots are the channel counts rounded up to powers of two; the reduced operand must fit a wave
   int u_min = 1 << 30;
   for (auto &t : triples) {
     const int n1 = xs[t.xi].second, n2 = ys[t.yi].second;
-    if (!is_pow2(n1) || !is_pow2(n2)) return GELIB_HIP_OK;
-    if (!diag && n2 > kWave) return GELIB_HIP_OK;
-    const long long U = diag ? n1 : (long long)n1 * n2;
-    if (U > (1 << 20)) return GELIB_HIP_OK;
-    u_min = std::min<int>(u_min, (int)U);
+    if (n1 < 1 || n2 < 1) return GELIB_HIP_OK;
+    const int lg1 = ilog2(n1), lg2 = ilog2(n2);
+    if (!diag && lg2 > 6) return GELIB_HIP_OK;
+    const int lgu = diag ? lg1 : lg1 + lg2;
+    if (lgu > 20) return GELIB_HIP_OK;
+    u_min = std::min<int>(u_min, 1 << lgu);
   }
   const DevicePlan *plan = nullptr;
   int rc = get_plan(diag, triples, xs, ys, rls, &plan);
@@ -278,6 +285,7 @@ int run_bwd(bool diag, const std::vector<VecTriple> &triples, const std::vector<
   a.want_y = want_y ? 1 : 0;
   a.bank_len = plan->bank_len;
   a.zero_off = plan->zero_off;
+  a.padded = plan->padded ? 1 : 0;
   a.xsize = plan->xsize;
   a.ysize = plan->ysize;
   for (size_t i = 0; i < xs.size(); i++) a.xrows[i] = 2 * xs[i].first + 1;

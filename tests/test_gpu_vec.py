@@ -111,3 +111,16 @@ def test_parts_in_any_order(cabi):
     torch.cuda.synchronize()
     for a, b in zip(drs, want):
         assert U.gate_excess(U.host(a), b) <= 1.0
+
+
+@pytest.mark.parametrize("case", [
+    (6, {0: 3, 1: 5, 2: 12}, {1: 6, 2: 7, 4: 3}, -1),      # nothing is a power of two; product l up to 6
+    (33, {l: 12 for l in range(5)}, {l: 12 for l in range(5)}, 4),
+    (70, {1: 1, 3: 3}, {2: 5}, 4),                           # 5 and 15 lane slots per cell: many cells per run
+    (3, {2: 24}, {3: 40}, -1),                               # 24 x 40 channels: several runs per cell, n2 padded to 64
+])
+@pytest.mark.parametrize("diag", [False, True])
+def test_channel_counts_that_are_not_powers_of_two(cabi, case, diag):
+    """The unrolled backward kernels round the channel counts up to powers of two for their lane layout; lanes
+    beyond the real channels idle.  Both gradients still come from the fused kernels (path 2)."""
+    assert run_vec(cabi, *case, diag, seed=500, force_generic=False) == (2, 2)

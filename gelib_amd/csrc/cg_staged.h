@@ -21,7 +21,9 @@ struct StagedTriple {
   int xoff, yoff;   // offsets (complex elements) of the operand parts inside one cell's packed x / y image
   int offs;         // first channel of this triple's block inside the product part
   int u;            // channel slots per cell: n1*n2, or n for Diag
-  int log2_u;       // log2(u) when u is a power of two, else -1
+  int log2_u;       // backward lane slots per cell, as a log2: n1p*n2p (Diag: n1p) with the channel counts rounded up
+                    // to powers of two n1p, n2p (lanes beyond the real channels idle); -1 above 2^20
+  int lg_n2p;       // log2(n2p)
   // Three compact copies of the coefficient table, each holding only the entries with |m1+m2| <= l, in the
   // order the corresponding loop nest visits them, so every kernel reads its coefficients as one stream:
   int cg_fwd;       // m ascending, then m1 ascending            (forward: one output row at a time)

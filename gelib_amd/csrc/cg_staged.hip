@@ -335,15 +335,35 @@ constexpr int bwd_max_threads() {
 // Rows w0 .. w0+CAP-1 of a lane's column of g into the registers.  Rows past the end repeat the last one (never
 // used): the loads stay unconditional, which keeps the register rows one straight chain of writes instead of a
 // merge of alternatives at every row.
+// keep == false (a lane beyond the real channels) stores zeros.
 template <int CAP>
-__device__ __forceinline__ void load_window(RowRegs<CAP> &G, GlobalC *gp, int sm, int w0, int rows) {
+__device__ __forceinline__ void load_window(RowRegs<CAP> &G, GlobalC *gp, int sm, int w0, int rows, bool keep) {
   static_for<CAP>([&](auto mc) __attribute__((always_inline)) {
     constexpr int M = decltype(mc)::value;
     const int row = min(w0 + M, rows - 1);
     const v2f v = gp[(long long)row * sm];
-    G.template set<M>(v.x, v.y);
+    G.template set<M>(keep ? v.x : 0.f, keep ? v.y : 0.f);
   });
 }
+
+// A backward lane's channel pair.  Lane slots are laid out n1p x n2p with the channel counts rounded up to powers
+// of two, so that the lanes sharing i (resp. j) form aligned groups; a slot beyond the real channels reads channel 0,
+// has its g forced to zero and never writes.
+struct LaneChan {
+  int i, j, chan;
+  bool valid;
+};
+template <bool DIAG>
+__device__ __forceinline__ LaneChan lane_chan(int u, int lg_n2p, int n1, int n2) {
+  LaneChan c;
+  c.i = DIAG ? u : (u >> lg_n2p);
+  c.j = DIAG ? u : (u & ((1 << lg_n2p) - 1));
+  c.valid = c.i < n1 && (DIAG || c.j < n2);
+  if (!c.valid) c.i = 0, c.j = 0;
+  c.chan = DIAG ? c.i : c.i * n2 + c.j;
+  return c;
+}
+__device__ __forceinline__ int ceil_log2(int n) { return n > 1 ? 32 - __clz(n - 1) : 0; }
 
 // One gradient's loop nest over the rows of g in the window [wlo, whi] (as values of m = m1 + m2):
 //     for every own row o:   emit(o + lo_own,  sum_q  C[o,q] g[o+q] conj(other[q]))
@@ -426,23 +446,24 @@ __global__ void __launch_bounds__(bwd_max_threads<CAP>()) staged_bwd_kernel(cons
       const int u = flat & ((1 << log2_u) - 1);
       const bool live = cl < ncell;
       if (!live) cl = ncell - 1;  // dead lanes read valid memory and never add
-      const int lg_n2 = DIAG ? 0 : 31 - __clz(n2);
-      const int i = DIAG ? u : (u >> lg_n2);
-      const int j = DIAG ? u : (u & (n2 - 1));
-      GlobalC *gp = (GlobalC *)P.ptr + (cell0 + cl) * P.sb + (tr->offs + offs_add + u);
+      const int n2p = DIAG ? 1 : (1 << tr->lg_n2p);
+      const LaneChan lc = lane_chan<DIAG>(u, tr->lg_n2p, n1, n2);
+      const int i = lc.i, j = lc.j;
+      const bool writer = live && lc.valid;
+      GlobalC *gp = (GlobalC *)P.ptr + (cell0 + cl) * P.sb + (tr->offs + offs_add + lc.chan);
       const int rows = 2 * l + 1;
       // g is taken through the registers in windows of CAP rows (one window unless 2l+1 > CAP); each window adds
       // the terms whose row m1+m2 falls inside it
       for (int w0 = 0; w0 < rows; w0 += CAP) {
-        load_window<CAP>(G, gp, P.sm, w0, rows);
+        load_window<CAP>(G, gp, P.sm, w0, rows, lc.valid);
         const int wlo = w0 - l, whi = w0 + CAP - 1 - l;
         if (WX) {
           LdsF *xa = (LdsF *)(xacc + cl * xsize + tr->xoff + i);
           gradient_pass<CAP>(G, wlo, whi, l1, l2, l, (LdsC)ys + (cl * ysize + tr->yoff + j), n2, bank, tr->cg_back0,
                              lane, [&](int row, float ar, float ai) __attribute__((always_inline)) {
                                float2 acc[1] = {make_float2(ar, ai)};
-                               if (!DIAG) group_sum(acc, n2);
-                               if (live && (DIAG || j == 0)) {
+                               if (!DIAG) group_sum(acc, n2p);
+                               if (writer && (DIAG || j == 0)) {
                                  LdsF *dst = xa + 2 * row * n1;
                                  __hip_atomic_fetch_add(dst, acc[0].x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
                                  __hip_atomic_fetch_add(dst + 1, acc[0].y, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
@@ -454,8 +475,8 @@ __global__ void __launch_bounds__(bwd_max_threads<CAP>()) staged_bwd_kernel(cons
           gradient_pass<CAP>(G, wlo, whi, l2, l1, l, (LdsC)xs + (cl * xsize + tr->xoff + i), n1, bank, tr->cg_back1,
                              lane, [&](int row, float ar, float ai) __attribute__((always_inline)) {
                                float2 acc[1] = {make_float2(ar, ai)};
-                               if (!DIAG) stride_sum(acc, n2, span);
-                               if (live && (DIAG || (u & (span - 1)) < n2)) {
+                               if (!DIAG) stride_sum(acc, n2p, span);
+                               if (writer && (DIAG || (u & (span - 1)) < n2p)) {
                                  LdsF *dst = ya + 2 * row * n2;
                                  __hip_atomic_fetch_add(dst, acc[0].x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
                                  __hip_atomic_fetch_add(dst + 1, acc[0].y, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
@@ -534,9 +555,10 @@ __global__ void __launch_bounds__(256) staged_pair_bwd_kernel(const StagedArgs) 
       const int u = flat & ((1 << log2_u) - 1);
       const bool live = cl < ncell;
       if (!live) cl = ncell - 1;  // dead lanes read valid memory and never add
-      const int lg_n2 = DIAG ? 0 : 31 - __clz(n2);
-      const int i = DIAG ? u : (u >> lg_n2);
-      const int j = DIAG ? u : (u & (n2 - 1));
+      const int n2p = DIAG ? 1 : (1 << tr0->lg_n2p);
+      const LaneChan lc = lane_chan<DIAG>(u, tr0->lg_n2p, n1, n2);
+      const int i = lc.i, j = lc.j;
+      const bool writer = live && lc.valid;
       const LdsC xb = (LdsC)xs + (cl * xsize + tr0->xoff + i);
       const LdsC yb = (LdsC)ys + (cl * ysize + tr0->yoff + j);
       AX.clear();
@@ -557,8 +579,8 @@ __global__ void __launch_bounds__(256) staged_pair_bwd_kernel(const StagedArgs) 
           const int l = tr->l;
           const FastPart P = load_part(a->r + tr->ri);
           const int row = min(max(m + l, 0), 2 * l);
-          const v2f v = ((GlobalC *)P.ptr)[(cell0 + cl) * P.sb + (tr->offs + offs_add + u) + (long long)row * P.sm];
-          G.template set<T>(v.x, v.y);
+          const v2f v = ((GlobalC *)P.ptr)[(cell0 + cl) * P.sb + (tr->offs + offs_add + lc.chan) + (long long)row * P.sm];
+          G.template set<T>(lc.valid ? v.x : 0.f, lc.valid ? v.y : 0.f);
         });
         const int m1lo = max(-l1, m - l2), m1hi = min(l1, m + l2);
         const int len = nt - tlo;
@@ -589,8 +611,8 @@ __global__ void __launch_bounds__(256) staged_pair_bwd_kernel(const StagedArgs) 
       if (WX) {
         float2 out[CAP];
         static_for<CAP>([&](auto mc) __attribute__((always_inline)) { out[decltype(mc)::value] = AX.template row<decltype(mc)::value>(); });
-        if (!DIAG) group_sum(out, n2);
-        if (live && (DIAG || j == 0)) {
+        if (!DIAG) group_sum(out, n2p);
+        if (writer && (DIAG || j == 0)) {
           LdsF *xa = (LdsF *)(xacc + cl * xsize + tr0->xoff + i);
           static_for<CAP>([&](auto mc) __attribute__((always_inline)) {
             constexpr int M = decltype(mc)::value;
@@ -604,8 +626,8 @@ __global__ void __launch_bounds__(256) staged_pair_bwd_kernel(const StagedArgs) 
       if (WY) {
         float2 out[CAP];
         static_for<CAP>([&](auto mc) __attribute__((always_inline)) { out[decltype(mc)::value] = AY.template row<decltype(mc)::value>(); });
-        if (!DIAG) stride_sum(out, n2, span);
-        if (live && (DIAG || (u & (span - 1)) < n2)) {
+        if (!DIAG) stride_sum(out, n2p, span);
+        if (writer && (DIAG || (u & (span - 1)) < n2p)) {
           LdsF *ya = (LdsF *)(yacc + cl * ysize + tr0->yoff + j);
           static_for<CAP>([&](auto mc) __attribute__((always_inline)) {
             constexpr int M = decltype(mc)::value;
@@ -695,7 +717,8 @@ __global__ void __launch_bounds__(256) staged_stripe_kernel(const StagedArgs) {
     }
     const int n_own = OWN.n;
     const int n1 = ROLE == 0 ? n_own : n_other, n2 = ROLE == 0 ? n_other : n_own;
-    const int lg_n2 = DIAG ? 0 : 31 - __clz(n2);
+    const int lg_n2 = DIAG ? 0 : ceil_log2(n2);
+    const int n2p = 1 << lg_n2;
     A.clear();
     for (int sub = 0; sub < nsub; sub++) {
       const int flat = log2_u >= 6 ? ((idx << log2_u) + (sub << 6) + lane) : ((idx << 6) + lane);
@@ -703,16 +726,16 @@ __global__ void __launch_bounds__(256) staged_stripe_kernel(const StagedArgs) {
       const int u = flat & ((1 << log2_u) - 1);
       const bool live = cl < ncell;
       if (!live) cl = ncell - 1;  // dead lanes read valid memory and never store
-      const int i = DIAG ? u : (u >> lg_n2);
-      const int j = DIAG ? u : (u & (n2 - 1));
+      const LaneChan lc = lane_chan<DIAG>(u, lg_n2, n1, n2);
+      const int i = lc.i, j = lc.j;
       for (int t = 0; t < count; t++) {
         const TriplePtr tr = triples + order[first + t];
         const int l1 = tr->l1, l2 = tr->l2, l = tr->l;
         const FastPart P = load_part(a->r + tr->ri);
-        GlobalC *gp = (GlobalC *)P.ptr + (cell0 + cl) * P.sb + (tr->offs + offs_add + u);
+        GlobalC *gp = (GlobalC *)P.ptr + (cell0 + cl) * P.sb + (tr->offs + offs_add + lc.chan);
         const int rows = 2 * l + 1;
         for (int w0 = 0; w0 < rows; w0 += CAP) {
-          load_window<CAP>(G, gp, P.sm, w0, rows);
+          load_window<CAP>(G, gp, P.sm, w0, rows, lc.valid);
           const int wlo = w0 - l, whi = w0 + CAP - 1 - l;
           auto add_row = [&](int row, float ar, float ai) __attribute__((always_inline)) { A.add(row, ar, ai); };
           if (ROLE == 0)
@@ -724,23 +747,27 @@ __global__ void __launch_bounds__(256) staged_stripe_kernel(const StagedArgs) {
         }
       }
       // the gradient of x is complete for this run's i; the gradient of y still sums over the other runs' i
-      if (ROLE == 1 && sub + 1 < nsub) continue;
+      if (ROLE == 1 && !DIAG && sub + 1 < nsub) continue;
       float2 out[CAP];
       static_for<CAP>([&](auto mc) __attribute__((always_inline)) {
         constexpr int M = decltype(mc)::value;
         out[M] = A.template row<M>();
       });
-      bool writer = live;
+      bool writer = live && lc.valid;
+      int column = ROLE == 0 ? i : j;
       if (!DIAG) {
         if (ROLE == 0) {
-          group_sum(out, n2);
-          writer = live && j == 0;
+          group_sum(out, n2p);
+          writer = writer && j == 0;
         } else {
-          stride_sum(out, n2, span);
-          writer = live && (u & (span - 1)) < n2;
+          // the sum over i ran over every run of the cell, so whether this lane writes depends on its j alone
+          // (the same in every run), not on the i of the last run
+          stride_sum(out, n2p, span);
+          column = u & (n2p - 1);
+          writer = live && column < n2 && (u & (span - 1)) < n2p;
         }
       }
-      GlobalC *dst = (GlobalC *)OWN.ptr + (cell0 + cl) * OWN.sb + (ROLE == 0 ? i : j);
+      GlobalC *dst = (GlobalC *)OWN.ptr + (cell0 + cl) * OWN.sb + column;
       if (writer) {
         static_for<CAP>([&](auto mc) __attribute__((always_inline)) {
           constexpr int M = decltype(mc)::value;

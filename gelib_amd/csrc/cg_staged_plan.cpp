@@ -85,7 +85,12 @@ int get_plan(bool diag, const std::vector<VecTriple> &triples, const std::vector
     r.offs = t.offs;
     const long long U = diag ? r.n1 : (long long)r.n1 * r.n2;
     r.u = (int)U;
-    r.log2_u = (U > 0 && (U & (U - 1)) == 0) ? ilog2((int)U) : -1;
+    {
+      const int lg1 = ilog2(std::max(1, r.n1)), lg2 = ilog2(std::max(1, r.n2));
+      const int lgu = diag ? lg1 : lg1 + lg2;
+      r.lg_n2p = lg2;
+      r.log2_u = lgu <= 20 ? lgu : -1;
+    }
     const int L1 = 2 * t.l1 + 1, L2 = 2 * t.l2 + 1;
     full.assign((size_t)L1 * L2, 0.f);
     cg_matrix_host(t.l1, t.l2, t.l, full.data());
@@ -174,9 +179,10 @@ int get_plan(bool diag, const std::vector<VecTriple> &triples, const std::vector
           n_other = no;
         }
         table[3 * k + 1] = filled - table[3 * k];
-        const long long U = diag ? n_own : (long long)n_own * std::max(1, n_other);
-        if (!is_pow2(n_own) || (n_other > 0 && !is_pow2(n_other)) || U > (1 << 20)) ok = false;
-        table[3 * k + 2] = ok ? ilog2((int)U) : 0;
+        // lane slots: channel counts rounded up to powers of two
+        const int lgu = diag ? ilog2(std::max(1, n_own)) : ilog2(std::max(1, n_own)) + ilog2(std::max(1, n_other));
+        if (lgu > 20) ok = false;
+        table[3 * k + 2] = ok ? lgu : 0;
       }
     }
     if (!diag)
@@ -325,13 +331,12 @@ int run_bwd(bool diag, const std::vector<VecTriple> &triples, const std::vector<
             long long ncells, int offs_add, bool accumulate, bool want_x, bool want_y, hipStream_t s, int *used) {
   *used = 0;
   if (!sizes_ok(xs, ys, rls)) return GELIB_HIP_OK;
-  // the lane sums need power-of-two channel counts, and the second operand's channels inside one wave
+  // lane slots are the channel counts rounded up to powers of two; the second operand's must fit one wave
   for (auto &t : triples) {
     const int n1 = xs[t.xi].second, n2 = ys[t.yi].second;
-    if (!is_pow2(n1) || !is_pow2(n2)) return GELIB_HIP_OK;
+    if (n1 < 1 || n2 < 1) return GELIB_HIP_OK;
     if (!diag && n2 > kWave) return GELIB_HIP_OK;
-    const long long U = diag ? n1 : (long long)n1 * n2;
-    if (U > (1 << 20)) return GELIB_HIP_OK;
+    if ((diag ? ilog2(n1) : ilog2(n1) + ilog2(n2)) > 20) return GELIB_HIP_OK;
   }
   const DevicePlan *plan = nullptr;
   int rc = get_plan(diag, triples, xs, ys, rls, &plan);
@@ -374,7 +379,8 @@ int run_bwd(bool diag, const std::vector<VecTriple> &triples, const std::vector<
   if (g_bwd_pairs && plan->pairs_ok) {
     auto units = [&](long long c) {
       long long n = 0;
-      for (int k = 0; k < plan->npairs; k++) n += (c * plan->triples[plan->stripes[plan->pair_off + 3 * k]].u + kWave - 1) / kWave;
+      for (int k = 0; k < plan->npairs; k++)
+        n += ((c << plan->triples[plan->stripes[plan->pair_off + 3 * k]].log2_u) + kWave - 1) / kWave;
       return n;
     };
     long long cpb = 1;

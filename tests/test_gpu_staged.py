@@ -99,6 +99,12 @@ def test_vec(cabi, case, diag):
     run_vec(cabi, B, tx, ty, maxl, diag, seed=500)
 
 
+def test_diag_with_more_channels_than_a_wave(cabi):
+    # 128 and 96 channels: two runs of 64 lane slots per cell, each flushed on its own
+    run_vec(cabi, 3, {5: 128}, {5: 128}, 6, True, seed=520)
+    run_vec(cabi, 3, {5: 96, 6: 96}, {5: 96}, 7, True, seed=521)
+
+
 @pytest.mark.parametrize("threads", [256, 512, 1024])
 def test_backward_block_widths(cabi, threads):
     cabi.set_option("staged_bwd_threads", threads)
@@ -121,10 +127,12 @@ def test_forward_tile_widths(cabi, tile):
 
 
 def test_channel_counts_that_are_not_powers_of_two(cabi):
-    # the forward kernel takes any channel count; the backward lane sums need powers of two, so the gradient
-    # call falls back to the shape-agnostic kernels
-    run_vec(cabi, 4, {5: 3, 6: 5}, {5: 6, 1: 7}, -1, False, seed=700, expect_bwd=1)
-    run_vec(cabi, 4, {5: 3, 6: 3}, {5: 3, 1: 3}, -1, True, seed=701, expect_bwd=1)
+    # the forward kernel takes any channel count; the backward kernels round the counts up to powers of two for their
+    # lane layout and idle the lanes beyond the real channels
+    run_vec(cabi, 4, {5: 3, 6: 5}, {5: 6, 1: 7}, -1, False, seed=700)
+    run_vec(cabi, 4, {5: 3, 6: 3}, {5: 3, 1: 3}, -1, True, seed=701)
+    run_vec(cabi, 9, {6: 12}, {5: 12}, 7, False, seed=702)          # 12 x 12 -> 16 x 16 lane slots, several runs per cell
+    run_vec(cabi, 40, {7: 1}, {5: 3}, -1, False, seed=703)          # 3 -> 4 lane slots per cell, 16 cells per run
 
 
 @pytest.mark.parametrize("offs", [3, 4])   # odd: one channel per lane; multiple of 4: four adjacent channels per lane

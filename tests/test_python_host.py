@@ -96,3 +96,23 @@ def test_type_and_weights():
     assert len(list(lin.parameters())) == 2 and lin(x).tau() == {0: 5, 1: 4}
     xa = G.SO3vecArr.randn(2, [3], tau_in)
     assert (xa * W).tau() == {0: 5, 1: 4} and (xa * W).get_adims() == [3]
+
+
+def test_o3_labels_and_types():
+    import gelib_amd as G
+    t = G.O3type({(1, 1): 2, (2, -1): 2})
+    # (1,+)x(1,+) -> l=0..2 even; (1,+)x(2,-) and (2,-)x(1,+) -> l=1..3 odd; (2,-)x(2,-) -> l=0..4 even
+    assert dict(t.CGproduct(t)) == {(0, 1): 8, (1, 1): 8, (1, -1): 8, (2, 1): 8, (2, -1): 8, (3, 1): 4, (3, -1): 8,
+                                    (4, 1): 4}
+    assert list(t.CGproduct(t)) == sorted(t.CGproduct(t), key=lambda mu: 2 * mu[0] + (mu[1] == -1))
+    assert dict(t.DiagCGproduct(t, 1)) == {(0, 1): 4, (1, 1): 4, (1, -1): 4}
+    p = G.O3part.randn(2, (2, -1), 3)
+    assert (p.getl(), p.getp(), p.getn(), p.getb()) == (2, -1, 3, 2)
+    # the representation property, including reflections: D(R1) D(R2) = D(R1 R2)
+    R1, R2 = G.O3element.random(), G.O3element(-torch.eye(3))
+    for mu in ((1, 1), (1, -1), (3, -1)):
+        rho = G.O3irrep(*mu)
+        assert torch.allclose(rho.matrix(R1) @ rho.matrix(R2), rho.matrix(G.O3element(R1 @ R2)), atol=1e-4)
+    assert torch.allclose(G.O3irrep(2, -1).matrix(R2), -torch.eye(5, dtype=torch.complex64), atol=1e-5)
+    with pytest.raises(AssertionError):
+        G.O3part.randn(1, (1, 1), 2).CGproduct(G.O3part.randn(1, (1, -1), 2), (2, 1))   # parity rule

@@ -115,6 +115,75 @@ def cpu_baseline(torch, xs, ys, gs, rs, xgs, ygs, maxl, diag, nsample):
     return nsample / dt, dt, parity, {"value": nsample / dt_all, "unit": "samples/s", "cores": nth}
 
 
+AUX_WORKLOADS = ("spharm_l4_n16_B1048576", "gather_l2_n16_cells262144_deg8")
+
+
+def aux_bench(torch, args, name):
+    """The two kernels either side of the product: the producer of y (spherical harmonics) and the sum of cells
+    that precedes it in message passing (gather).  Same JSON shape; a step is one launch."""
+    import numpy as np
+    from gelib_amd import cabi
+    from oracle import cg_oracle as ora
+    dev = torch.device("cuda:0")
+    g = torch.Generator().manual_seed(77)
+    if name.startswith("spharm"):
+        l, n, B = 4, 16, args.batch or 1048576
+        X = torch.randn(B, 3, n, generator=g).to(dev)
+        r = torch.empty(B, 2 * l + 1, n, dtype=torch.complex64, device=dev)
+        step = lambda: cabi.so3part_spharm(r, X, accumulate=False)
+        nbytes, units, unit = B * n * (12 + 8 * (2 * l + 1)), B * n, "vectors/s"
+        ns = min(B, 65536)
+
+        def cpu():
+            t0 = time.perf_counter()
+            want = ora.spharm(l, X[:ns].cpu().numpy())
+            return ns * n / (time.perf_counter() - t0), want, r[:ns].cpu().numpy()
+        sample = "first %d of the batch" % ns
+        tol = dict(rtol=1e-5, atol=1e-6)
+    else:
+        l, n, N, deg = 2, 16, args.batch or 262144, 8
+        rng = np.random.default_rng(5)
+        src = rng.integers(0, N, N * deg).astype(np.int32)
+        tgt = rng.integers(0, N, N * deg).astype(np.int32)
+        gm = cabi.GatherMap(src.tolist(), tgt.tolist(), N, N)
+        X = torch.view_as_complex(torch.randn(1, N, 2 * l + 1, n, 2, generator=g)).to(dev)
+        r = torch.empty_like(X)
+        step = lambda: cabi.part_gather(r, X, gm, 1, accumulate=False)
+        cell = 8 * (2 * l + 1) * n
+        nbytes, units, unit = (N * deg + N) * cell, N, "cells/s"   # every pair reads one cell, every target is written once
+
+        def cpu():
+            x = X.cpu().numpy()
+            t0 = time.perf_counter()
+            want = ora.gather(x, src, tgt, N, 1)
+            return N / (time.perf_counter() - t0), want, r.cpu().numpy()
+        sample = "the whole map (%d pairs), numpy slice adds" % (N * deg)
+        tol = dict(rtol=0, atol=0)
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(args.steps):
+        step()
+    e1.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms = e0.elapsed_time(e1) / args.steps
+    out = {"metric": name.split("_")[0] + " " + unit, "value": units / (wall / args.steps), "unit": unit, "n_gpus": 1,
+           "steps": args.steps, "warmup": args.warmup, "ms_per_step": wall * 1e3 / args.steps, "higher_is_better": True,
+           "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic", "config": {"workload": name},
+           "roofline": {"bound": "hbm", "kernel": name.split("_")[0], "achieved": nbytes / (ms * 1e-3) / 1e9,
+                        "peak": HBM_PEAK / 1e9, "unit": "GB/s", "frac": nbytes / (ms * 1e-3) / HBM_PEAK, "traffic": None,
+                        "algorithmic_bytes_per_launch": nbytes}}
+    if not args.no_cpu:
+        rate, want, got = cpu()
+        out["cpu_baseline"] = {"value": rate, "unit": unit, "cores": 1, "kind": "port", "sample": sample}
+        out["parity"] = {"ok": bool(np.allclose(got, want, **tol))}
+    print(json.dumps(out))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -142,6 +211,9 @@ def main():
     cabi.set_option("force_generic", int(args.generic))
     dev = torch.device("cuda:0")
     name = ALIASES.get(args.workload, args.workload)
+    aux = [w for w in AUX_WORKLOADS if w == name or w.split("_")[0] == name]
+    if aux:
+        return aux_bench(torch, args, aux[0])
     kind, B, tx, ty, maxl, diag = WORKLOADS[name]
     if args.batch:
         B = args.batch

@@ -72,6 +72,11 @@ class SO3partArr(torch.Tensor):
         rho = SO3irrep(self.getl())
         return SO3partArr(torch.matmul(rho.matrix(R).to(self.device), self))
 
+    def gather(self, gmap, dim=0):
+        """Sums of cells along grid dimension dim: cell t of the result = sum of the cells s of self over the pairs
+        (s, t) of gmap (python/src/gelib/SO3partArr.py:142-146)."""
+        return SO3partArr_GatherFn.apply(self, gmap, dim)
+
     def CGproduct(self, y, l):
         return SO3partArr_CGproductFn.apply(self, y, l)
 
@@ -116,3 +121,26 @@ def _part_fn(diag):
 
 SO3partArr_CGproductFn = _part_fn(False)
 SO3partArr_DiagCGproductFn = _part_fn(True)
+
+
+class SO3partArr_GatherFn(torch.autograd.Function):
+    """python/src/gelib/SO3partArr.py:236-254: forward add_gather, backward add_gather_back with the same map."""
+
+    @staticmethod
+    def forward(ctx, x, gmap, d):
+        from gelib_amd.gather_map import gather_map
+        assert isinstance(gmap, gather_map)
+        adims = list(x.size()[1:x.dim() - 2])
+        assert 0 <= d < len(adims) and len(adims) <= 2, "gather runs along one of at most two grid dimensions"
+        assert adims[d] == gmap.d_in()
+        ctx.gmap, ctx.d, ctx.adims = gmap, d, list(adims)
+        adims[d] = gmap.d_out()
+        r = SO3partArr.zeros(x.size(0), adims, (x.size(-2) - 1) // 2, x.size(-1), device=x.device)
+        _view(r).add_gather(x, gmap.obj, d)
+        return r
+
+    @staticmethod
+    def backward(ctx, rg):
+        xg = SO3partArr.zeros(rg.size(0), ctx.adims, (rg.size(-2) - 1) // 2, rg.size(-1), device=rg.device)
+        _view(xg).add_gather_back(rg.contiguous(), ctx.gmap.obj, ctx.d)
+        return xg, None, None

@@ -89,6 +89,10 @@ class SO3vecArr:
             r.parts[l] = SO3partArr(p).apply(R)
         return r
 
+    def gather(self, gmap, dim=0):
+        """Part by part (python/src/gelib/SO3vecArr.py:230-234)."""
+        return SO3vecArr(*[SO3partArr(p).gather(gmap, dim) for p in self.parts.values()])
+
     def odot(self, y):
         assert list(self.parts.keys()) == list(y.parts.keys())
         return sum(SO3partArr(self.parts[l]).odot(y.parts[l]) for l in self.parts.keys())

@@ -80,6 +80,32 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("CGproduct", [](const SO3type &x, const SO3type &y) { return x.CGproduct(y, -1); });
   m.def("CGproduct", [](const SO3type &x, const SO3type &y, const int maxl) { return x.CGproduct(y, maxl); });
 
+  // python/bindings/gather_map_py.cpp:15-29
+  py::class_<cnine::GatherMapB>(m, "gather_map", "A list of (source, target) pairs for sums of slices")
+      .def_static("sources_targets",
+                  [](const std::vector<int> sources, const std::vector<int> targets, int n_in, int n_out) {
+                    return cnine::GatherMapB(sources, targets, n_in, n_out);
+                  },
+                  py::arg("sources"), py::arg("targets"), py::arg("n_in") = -1, py::arg("n_out") = -1)
+      .def_static("from_matrix",
+                  [](const at::Tensor &M, const int nin, const int nout) {
+                    TORCH_CHECK(M.scalar_type() == at::kInt && M.dim() == 2 && !M.is_cuda(),
+                                "GElib: a gather map is built from a k x 2 int32 host tensor of (source, target) rows");
+                    cnine::Gdims dims;
+                    std::vector<size_t> strides;
+                    for (int i = 0; i < 2; i++) dims.push_back((int)M.size(i)), strides.push_back((size_t)M.stride(i));
+                    return cnine::GatherMapB(cnine::TensorView<int>(M.data_ptr<int>(), dims, cnine::GstridesB(strides), 0), nin, nout);
+                  })
+      .def_static("random", [](const int n, const int m, const float p, unsigned seed) { return cnine::GatherMapB::random(n, m, p, seed); },
+                  py::arg("n"), py::arg("m"), py::arg("p") = 0.5, py::arg("seed") = 0)
+      .def("inv", &cnine::GatherMapB::inv)
+      .def("d_in", &cnine::GatherMapB::d_in)
+      .def("d_out", &cnine::GatherMapB::d_out)
+      .def("pairs", [](const cnine::GatherMapB &g) { return g.inverted ? std::make_pair(g.targets, g.sources) : std::make_pair(g.sources, g.targets); })
+      .def("str", &cnine::GatherMapB::str, py::arg("indent") = "")
+      .def("__str__", &cnine::GatherMapB::str, py::arg("indent") = "")
+      .def("__repr__", &cnine::GatherMapB::repr);
+
   py::class_<SO3part<float>>(m, "SO3part",
                              "n vectors transforming according to one irreducible representation of SO(3)")
       .def_static("view", [](at::Tensor &x) { return SO3part<float>(view_of(x)); })
@@ -133,6 +159,18 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
              r.add_spharm(cnine::TensorView<float>(X.data_ptr<float>(), dims, cnine::GstridesB(strides), X.is_cuda() ? 1 : 0));
            },
            py::arg("X"))
+      .def("add_gather",
+           [](SO3part<float> &r, at::Tensor &x, const cnine::GatherMapB &gmap, int d) {
+             StreamGuard sg;
+             r.add_gather(SO3part<float>(view_of(x)), gmap, d);
+           },
+           py::arg("x"), py::arg("gmap"), py::arg("d") = 0)
+      .def("add_gather_back",
+           [](SO3part<float> &xg, at::Tensor &rg, const cnine::GatherMapB &gmap, int d) {
+             StreamGuard sg;
+             xg.add_gather_back(SO3part<float>(view_of(rg)), gmap, d);
+           },
+           py::arg("rg"), py::arg("gmap"), py::arg("d") = 0)
       .def("getl", &SO3part<float>::getl)
       .def("getn", &SO3part<float>::getn)
       .def("str", &SO3part<float>::str, py::arg("indent") = "")

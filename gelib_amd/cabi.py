@@ -16,7 +16,8 @@ SYMBOLS = [
     "gelib_hip_so3part_cg_fwd", "gelib_hip_so3part_cg_back0", "gelib_hip_so3part_cg_back1",
     "gelib_hip_so3part_diagcg_fwd", "gelib_hip_so3part_diagcg_back0", "gelib_hip_so3part_diagcg_back1",
     "gelib_hip_so3vec_cg_fwd", "gelib_hip_so3vec_cg_bwd", "gelib_hip_so3vec_diagcg_fwd",
-    "gelib_hip_so3vec_diagcg_bwd", "gelib_hip_so3part_spharm", "gelib_hip_set_option", "gelib_hip_last_path",
+    "gelib_hip_so3vec_diagcg_bwd", "gelib_hip_so3part_spharm", "gelib_hip_gather_map_create",
+    "gelib_hip_gather_map_destroy", "gelib_hip_part_gather", "gelib_hip_set_option", "gelib_hip_last_path",
     "gelib_hip_malloc", "gelib_hip_free", "gelib_hip_memcpy", "gelib_hip_memset", "gelib_hip_synchronize",
 ]
 
@@ -61,6 +62,12 @@ def lib():
                                          ctypes.c_void_p]
         L.gelib_hip_so3part_spharm.argtypes = [P, ctypes.c_void_p, ctypes.POINTER(ctypes.c_int64),
                                                ctypes.POINTER(ctypes.c_int64), ctypes.c_int, ctypes.c_void_p]
+        I32 = ctypes.POINTER(ctypes.c_int32)
+        L.gelib_hip_gather_map_create.argtypes = [I32, I32, ctypes.c_int64, ctypes.c_int, ctypes.c_int,
+                                                  ctypes.POINTER(ctypes.c_void_p)]
+        L.gelib_hip_gather_map_destroy.argtypes = [ctypes.c_void_p]
+        L.gelib_hip_part_gather.argtypes = [P, P, ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                                            ctypes.c_void_p]
         L.gelib_hip_set_option.argtypes = [ctypes.c_char_p, ctypes.c_int]
         _lib = L
     return _lib
@@ -181,6 +188,31 @@ def so3part_spharm(r, x, accumulate=True):
     A = ctypes.c_int64 * 5
     check(lib().gelib_hip_so3part_spharm(ctypes.byref(desc(r)), ctypes.c_void_p(x.data_ptr()), A(*dims), A(*strs),
                                          int(accumulate), _stream(r)))
+
+
+class GatherMap:
+    """Device form of a list of (source, target) pairs; freed with the object."""
+
+    def __init__(self, sources, targets, n_in, n_out):
+        n = len(sources)
+        if len(targets) != n:
+            raise ValueError("as many sources as targets are needed")
+        A = ctypes.c_int32 * max(n, 1)
+        self.handle = ctypes.c_void_p()
+        self.n_in, self.n_out = n_in, n_out
+        check(lib().gelib_hip_gather_map_create(A(*sources), A(*targets), n, n_in, n_out, ctypes.byref(self.handle)))
+
+    def __del__(self):
+        if getattr(self, "handle", None):
+            lib().gelib_hip_gather_map_destroy(self.handle)
+            self.handle = None
+
+
+def part_gather(r, x, gmap, dim, inverse=False, accumulate=True):
+    """r[.., t, ..] (+)= sum over the pairs (s, t) of x[.., s, ..] along dimension dim (0 = batch, 1..2 = grid) of the
+    5-D views; inverse swaps the roles of sources and targets."""
+    check(lib().gelib_hip_part_gather(ctypes.byref(desc(r)), ctypes.byref(desc(x)), gmap.handle, int(dim), int(inverse),
+                                      int(accumulate), _stream(r)))
 
 
 def set_option(name, value):

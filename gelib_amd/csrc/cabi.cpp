@@ -498,6 +498,100 @@ int gelib_hip_so3part_spharm(const gelib_part_desc *r, const float *x, const int
   return launch_spharm(pr, x, xs, D, R.l, R.n, accumulate != 0, (hipStream_t)stream);
 }
 
+// ---- gather maps -------------------------------------------------------------------------------------------
+namespace {
+
+struct GatherMap {  // both directions of a list of (source, target) pairs, compressed by the index that is written
+  int n_in, n_out, device;
+  int *rows[2], *cols[2];  // [0]: by target (forward), [1]: by source (the inverse map, for the gradient)
+};
+
+int upload_compressed(const int32_t *keys, const int32_t *vals, int64_t npairs, int nkeys, int **rows, int **cols) {
+  std::vector<int> ptr((size_t)nkeys + 1, 0), out((size_t)std::max<int64_t>(npairs, 1));
+  for (int64_t k = 0; k < npairs; k++) ptr[(size_t)keys[k] + 1]++;
+  for (int i = 0; i < nkeys; i++) ptr[(size_t)i + 1] += ptr[i];
+  std::vector<int> fill(ptr.begin(), ptr.end() - 1);
+  for (int64_t k = 0; k < npairs; k++) out[(size_t)fill[keys[k]]++] = vals[k];  // stable: pairs keep their order
+  GELIB_HIP_TRY(hipMalloc((void **)rows, ptr.size() * sizeof(int)));
+  GELIB_HIP_TRY(hipMalloc((void **)cols, out.size() * sizeof(int)));
+  GELIB_HIP_TRY(hipMemcpy(*rows, ptr.data(), ptr.size() * sizeof(int), hipMemcpyHostToDevice));
+  GELIB_HIP_TRY(hipMemcpy(*cols, out.data(), out.size() * sizeof(int), hipMemcpyHostToDevice));
+  return GELIB_HIP_OK;
+}
+
+}  // namespace
+
+int gelib_hip_gather_map_create(const int32_t *sources, const int32_t *targets, int64_t npairs, int n_in, int n_out,
+                                void **map) {
+  if (!map) return GELIB_HIP_ERR_NULL;
+  *map = nullptr;
+  if (npairs < 0 || n_in < 0 || n_out < 0 || npairs > 0x7fffffffLL) return GELIB_HIP_ERR_ARG;
+  if (npairs > 0 && (!sources || !targets)) return GELIB_HIP_ERR_NULL;
+  for (int64_t k = 0; k < npairs; k++)
+    if (sources[k] < 0 || sources[k] >= n_in || targets[k] < 0 || targets[k] >= n_out) return GELIB_HIP_ERR_ARG;
+  GatherMap *m = new GatherMap();
+  m->n_in = n_in;
+  m->n_out = n_out;
+  m->rows[0] = m->rows[1] = m->cols[0] = m->cols[1] = nullptr;
+  hipError_t e = hipGetDevice(&m->device);
+  int rc = e == hipSuccess ? GELIB_HIP_OK : record_hip_error(e, "hipGetDevice");
+  if (!rc) rc = upload_compressed(targets, sources, npairs, n_out, &m->rows[0], &m->cols[0]);
+  if (!rc) rc = upload_compressed(sources, targets, npairs, n_in, &m->rows[1], &m->cols[1]);
+  if (rc) {
+    gelib_hip_gather_map_destroy(m);
+    return rc;
+  }
+  *map = m;
+  return GELIB_HIP_OK;
+}
+
+int gelib_hip_gather_map_destroy(void *map) {
+  GatherMap *m = (GatherMap *)map;
+  if (!m) return GELIB_HIP_OK;
+  for (int k = 0; k < 2; k++) {
+    if (m->rows[k]) (void)hipFree(m->rows[k]);
+    if (m->cols[k]) (void)hipFree(m->cols[k]);
+  }
+  delete m;
+  return GELIB_HIP_OK;
+}
+
+int gelib_hip_part_gather(const gelib_part_desc *r, const gelib_part_desc *x, const void *map, int dim, int inverse,
+                          int accumulate, void *stream) {
+  t_last_path = kPathNone;
+  const GatherMap *m = (const GatherMap *)map;
+  if (!m) return GELIB_HIP_ERR_NULL;
+  View R, X;
+  int rc;
+  if ((rc = check_desc(r, R)) || (rc = check_desc(x, X))) return rc;
+  if (dim < 0 || dim > 2) return GELIB_HIP_ERR_ARG;
+  const int dir = inverse ? 1 : 0;
+  const int n_from = inverse ? m->n_out : m->n_in, n_to = inverse ? m->n_in : m->n_out;
+  for (int k = 0; k < 5; k++) {
+    if (k == dim) {
+      if (x->dims[k] != n_from || r->dims[k] != n_to) return k == 0 ? GELIB_HIP_ERR_BATCH : GELIB_HIP_ERR_GRID;
+    } else if (x->dims[k] != r->dims[k]) {
+      return k == 0 ? GELIB_HIP_ERR_BATCH : (k < 3 ? GELIB_HIP_ERR_GRID : GELIB_HIP_ERR_CHANNELS);
+    }
+  }
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev != m->device) return GELIB_HIP_ERR_DEVICE;
+  long long D[5], rs[5], xs[5], total = 1;
+  for (int k = 0; k < 5; k++) {
+    D[k] = r->dims[k];
+    rs[k] = r->strides[k];
+    xs[k] = x->strides[k];
+    total *= D[k];
+    if (r->dims[k] > 1 && r->strides[k] == 0) return GELIB_HIP_ERR_BROADCAST_DEST;
+  }
+  if (total == 0) return GELIB_HIP_OK;
+  if (!r->ptr || (!x->ptr && n_from > 0)) return GELIB_HIP_ERR_NULL;
+  if ((rc = check_pointer(r)) || (rc = check_pointer(x))) return rc;
+  t_last_path = kPathGeneric;
+  return launch_gather((float2 *)r->ptr, (const float2 *)x->ptr, rs, xs, D, dim, m->rows[dir], m->cols[dir],
+                       accumulate != 0, (hipStream_t)stream);
+}
+
 int gelib_hip_malloc(void **ptr, uint64_t bytes) {
   if (!ptr) return GELIB_HIP_ERR_NULL;
   *ptr = nullptr;

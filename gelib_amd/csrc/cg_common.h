@@ -55,4 +55,8 @@ int launch_zero_fill(const PartDev &d, const long long D[3], int M, int n, hipSt
 int launch_spharm(const PartDev &r, const float *x, const long long xs[5], const long long D[3], int L, int n,
                   bool accumulate, hipStream_t s);
 
+// ---- sum of slices along one leading dimension (gather.hip): r[.., t, ..] (+)= sum_{k in row t} x[.., sources[k], ..] ----
+int launch_gather(float2 *r, const float2 *x, const long long rs[5], const long long xs[5], const long long D[5], int dim,
+                  const int *row_ptr, const int *sources, bool accumulate, hipStream_t s);
+
 }  // namespace gelib_hip

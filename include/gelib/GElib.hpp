@@ -19,7 +19,10 @@
 #include <cmath>
 #include <functional>
 #include <map>
+#include <memory>
 #include <mutex>
+#include <sstream>
+#include <stdexcept>
 #include <unordered_map>
 
 #include "cnine_min.hpp"
@@ -31,6 +34,101 @@
     throw std::runtime_error("GElib error in " + std::string(__PRETTY_FUNCTION__) + " : failed assertion " + #condition + ".");
 #define GELIB_ERROR(msg) throw std::runtime_error("GElib error in " + std::string(__PRETTY_FUNCTION__) + " : " + msg + ".");
 #define GELIB_SKIP(msg) throw std::runtime_error("Function " + std::string(__func__) + " skipped: " + msg + ".");
+
+namespace GElib {
+inline void gelib_check(const int rc);
+}
+
+namespace cnine {
+
+// A list of (source, target) pairs: slice `target` of the result collects slice `source` of the argument
+// (the class python/bindings/gather_map_py.cpp:15-29 binds; its definition is in cnine, outside the reference tree).
+// Pairs keep their order within one target, which fixes the order of the float sums.  The device form is made on
+// first use, on the GPU that is current then, and released with the last copy of the map.
+class GatherMapB {
+ public:
+  int n_in = 0, n_out = 0;
+  std::vector<int> sources, targets;
+  bool inverted = false;
+
+  GatherMapB() {}
+  // n_in / n_out default to the largest index + 1
+  GatherMapB(const std::vector<int> &_sources, const std::vector<int> &_targets, const int _n_in = -1, const int _n_out = -1)
+      : sources(_sources), targets(_targets) {
+    if (sources.size() != targets.size()) throw std::invalid_argument("GatherMapB: as many sources as targets are needed.");
+    int ms = -1, mt = -1;
+    for (size_t i = 0; i < sources.size(); i++) ms = std::max(ms, sources[i]), mt = std::max(mt, targets[i]);
+    n_in = _n_in < 0 ? ms + 1 : _n_in;
+    n_out = _n_out < 0 ? mt + 1 : _n_out;
+    for (size_t i = 0; i < sources.size(); i++)
+      if (sources[i] < 0 || sources[i] >= n_in || targets[i] < 0 || targets[i] >= n_out)
+        throw std::out_of_range("GatherMapB: index outside [0, n_in) x [0, n_out).");
+  }
+  // rows of M are (source, target)
+  GatherMapB(const TensorView<int> &M, const int _n_in, const int _n_out) : n_in(_n_in), n_out(_n_out) {
+    if (M.ndims() != 2 || M.dim(1) != 2) throw std::invalid_argument("GatherMapB: the matrix must be k x 2.");
+    if (M.get_dev() != 0) throw std::invalid_argument("GatherMapB: the matrix must be in host memory.");
+    for (int i = 0; i < M.dim(0); i++) {
+      sources.push_back(M.arr[i * M.strides[0]]);
+      targets.push_back(M.arr[i * M.strides[0] + M.strides[1]]);
+    }
+    *this = GatherMapB(sources, targets, n_in, n_out);
+  }
+  // every (source, target) pair independently with probability p
+  static GatherMapB random(const int n_in, const int n_out, const float p, const unsigned seed = 0) {
+    std::vector<int> s, t;
+    unsigned long long state = 0x9E3779B97F4A7C15ull ^ seed;
+    for (int j = 0; j < n_out; j++)
+      for (int i = 0; i < n_in; i++) {
+        state = state * 6364136223846793005ull + 1442695040888963407ull;
+        if ((double)(state >> 11) / 9007199254740992.0 < p) s.push_back(i), t.push_back(j);
+      }
+    return GatherMapB(s, t, n_in, n_out);
+  }
+
+  GatherMapB inv() const {  // same pairs read backwards (core/Gpart.hpp:561)
+    GatherMapB R(*this);
+    R.inverted = !inverted;
+    return R;
+  }
+  int d_in() const { return inverted ? n_out : n_in; }
+  int d_out() const { return inverted ? n_in : n_out; }
+  size_t size() const { return sources.size(); }
+
+  void *device_handle() const {
+    if (!handle) {
+      void *h = nullptr;
+      GElib::gelib_check(gelib_hip_gather_map_create(sources.data(), targets.data(), (int64_t)sources.size(), n_in, n_out, &h));
+      handle = std::shared_ptr<void>(h, [](void *q) { gelib_hip_gather_map_destroy(q); });
+    }
+    return handle.get();
+  }
+
+  std::string str(const std::string indent = "") const {
+    std::ostringstream oss;
+    for (int t = 0; t < d_out(); t++) {
+      oss << indent << t << "<-(";
+      bool first = true;
+      for (size_t k = 0; k < size(); k++)
+        if ((inverted ? sources[k] : targets[k]) == t) {
+          oss << (first ? "" : ",") << (inverted ? targets[k] : sources[k]);
+          first = false;
+        }
+      oss << ")\n";
+    }
+    return oss.str();
+  }
+  std::string repr() const {
+    std::ostringstream oss;
+    oss << "<cnine::GatherMapB n_in=" << d_in() << " n_out=" << d_out() << " pairs=" << size() << ">";
+    return oss.str();
+  }
+
+ private:
+  mutable std::shared_ptr<void> handle;
+};
+
+}  // namespace cnine
 
 namespace GElib {
 
@@ -329,6 +427,21 @@ class SO3part : public cnine::BatchedTensor<std::complex<TYPE>>, public GpartBas
       }
     }
     gelib_check(gelib_hip_so3part_spharm(&R, x.arr, xdims, xstr, 1, gelib_stream()));
+  }
+
+  // ---- sums of slices along grid dimension d (core/Gpart.hpp:556-562) ----
+  void add_gather(const SO3part &x, const cnine::GatherMapB &gmap, const int d = 0) const {
+    GELIB_ASSRT(x.dev == dev);
+    if (dev != 1) GELIB_ERROR("SO3part::add_gather: the operands must be on GPU");
+    GELIB_ASSRT(ndims() <= 5 && x.ndims() == ndims());
+    GELIB_ASSRT(d >= 0 && d < ndims() - 3);
+    GELIB_ASSRT(gmap.d_in() == x.dims[d + 1]);
+    GELIB_ASSRT(gmap.d_out() == dims[d + 1]);
+    auto R = descriptor(), X = x.descriptor();
+    gelib_check(gelib_hip_part_gather(&R, &X, gmap.device_handle(), d + 1, gmap.inverted ? 1 : 0, 1, gelib_stream()));
+  }
+  void add_gather_back(const SO3part &r, const cnine::GatherMapB &gmap, const int d = 0) const {
+    add_gather(r, gmap.inv(), d);
   }
 
   std::string classname() const { return "GElib::SO3part"; }

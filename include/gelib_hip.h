@@ -133,6 +133,27 @@ int gelib_hip_so3vec_diagcg_bwd(const gelib_part_desc *xg, const gelib_part_desc
 int gelib_hip_so3part_spharm(const gelib_part_desc *r, const float *x, const int64_t xdims[5],
                              const int64_t xstrides[5], int accumulate, void *stream);
 
+/* ---- gather: sums of slices along the batch or a grid dimension ---------------------------------------------------------
+ * A gather map is a list of (source, target) pairs with 0 <= source < n_in, 0 <= target < n_out (the arguments of
+ * cnine::GatherMapB(sources, targets), python/bindings/gather_map_py.cpp:17-18).  create() checks the indices, sorts the
+ * pairs by target (and, for the inverse map, by source), keeping their order within one index, and copies both
+ * forms to the current device; the handle is valid on that device until destroy().  Host pointers. */
+int gelib_hip_gather_map_create(const int32_t *sources, const int32_t *targets, int64_t npairs, int n_in, int n_out,
+                                void **map);
+int gelib_hip_gather_map_destroy(void *map);
+/*
+ * r[.., t, ..] += sum over the pairs (s, t) of x[.., s, ..] along dimension dim of the 5-D views (0 = batch,
+ * 1..2 = grid); all other dimensions of r and x agree, dims[dim] is n_out for r and n_in for x.  Replaces
+ * Gpart::add_gather(x, gmap, d) with dim = d + 1 (core/Gpart.hpp:556-558).  inverse != 0 runs the map backwards
+ * (r has n_in slices, x n_out): Gpart::add_gather_back(g, gmap, d) (core/Gpart.hpp:560-562).  Every output element is
+ * summed by one thread in the order of the pairs, so results are reproducible; accumulate == 0 overwrites r,
+ * including slices that no pair targets (they become zero).  The loop the reference calls, cnine::GatherSlices, is
+ * not in its tree: the semantics here are those of its call sites and of python/docs/source/SO3partArr.rst:97-127
+ * with unit weights.
+ */
+int gelib_hip_part_gather(const gelib_part_desc *r, const gelib_part_desc *x, const void *map, int dim, int inverse,
+                          int accumulate, void *stream);
+
 /*
  * Device memory helpers for host code that does not include the HIP headers itself (the C++ mirror of the
  * reference's classes uses them where the reference relies on cnine's device transport, e.g. the

@@ -3,6 +3,8 @@
 Only the test-suite, the smoke check and the ``cpu_baseline`` leg of the benchmark import this
 module; the shipped package never does.  Arrays are numpy ``complex64`` (loop-order-faithful float32
 path) or ``complex128`` (float64 path) of shape ``(B, 2l+1, N)`` with arbitrary strides.
+
+``gather`` is parity unpinned: the loop the reference calls for it (cnine::GatherSlices) is outside its tree.
 """
 import ctypes
 import os
@@ -181,3 +183,18 @@ def spharm(l, x, batch=None):
     rc = f(l, B, x.shape[2], x.ctypes.data, xsb, x.shape[2], r.ctypes.data)
     assert rc == 0
     return r
+
+
+def gather(x, sources, targets, n_out, axis, r=None):
+    """r[.., t, ..] += x[.., s, ..] for every pair (s, t), pairs taken in the order given within one target: the call
+    sites of the reference's gather (core/Gpart.hpp:537-563; the loop itself, cnine::GatherSlices, is not in its
+    tree, so this function is unpinned by the reference and pinned only by its definition as a 0/1 matrix product,
+    see the tests).  float32 adds in pair order, so the result is reproducible bit for bit."""
+    shape = list(x.shape)
+    shape[axis] = n_out
+    out = np.zeros(shape, dtype=x.dtype) if r is None else r
+    xs = np.moveaxis(x, axis, 0)
+    os_ = np.moveaxis(out, axis, 0)
+    for s, t in zip(sources, targets):
+        os_[t] += xs[s]
+    return out

@@ -116,3 +116,21 @@ def test_o3_labels_and_types():
     assert torch.allclose(G.O3irrep(2, -1).matrix(R2), -torch.eye(5, dtype=torch.complex64), atol=1e-5)
     with pytest.raises(AssertionError):
         G.O3part.randn(1, (1, 1), 2).CGproduct(G.O3part.randn(1, (1, -1), 2), (2, 1))   # parity rule
+
+
+def test_gather_map_host_surface():
+    import gelib_amd as G
+    m = G.gather_map.sources_targets([0, 1, 2, 2], [1, 1, 0, 2])
+    assert (m.d_in(), m.d_out()) == (3, 3) and m.pairs() == ([0, 1, 2, 2], [1, 1, 0, 2])
+    assert m.inv().pairs() == ([1, 1, 0, 2], [0, 1, 2, 2]) and str(m).splitlines()[1] == "1<-(0,1)"
+    # the map of python/tests/test_gather_map.py
+    M = torch.tensor([[4, 3, 9, 1], [5, 5, 2, 7]], dtype=torch.int32)
+    f = G.gather_map.from_matrix(M.t(), 10, 10)
+    assert f.pairs() == ([4, 3, 9, 1], [5, 5, 2, 7]) and (f.d_in(), f.d_out()) == (10, 10)
+    r = G.gather_map.random(6, 5, 0.5, seed=1)
+    s, t = r.pairs()
+    assert 0 < len(s) < 30 and max(s) < 6 and max(t) < 5 and r.pairs() == G.gather_map.random(6, 5, 0.5, seed=1).pairs()
+    with pytest.raises(IndexError):
+        G.gather_map.sources_targets([0, 7], [0, 0], 3, 3)
+    with pytest.raises(Exception):                       # host tensors are refused
+        G.SO3partArr.randn(1, [3], 1, 2).gather(m, 0)

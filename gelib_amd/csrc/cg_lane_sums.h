@@ -44,6 +44,28 @@ __device__ __forceinline__ void stride_sum(float2 (&v)[K], int lo, int hi) {
   }
 }
 
+// v_permlane16_swap exchanges the odd 16-lane rows of its first operand with the even rows of its second,
+// v_permlane32_swap the upper half of the first with the lower half of the second.  The two wait states in front
+// cover a vector write of either operand by the instruction just before.
+__device__ __forceinline__ void swap_rows16(float &a, float &b) {
+  asm volatile("s_nop 1\n\tv_permlane16_swap_b32_e32 %0, %1" : "+v"(a), "+v"(b));
+}
+__device__ __forceinline__ void swap_halves32(float &a, float &b) {
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32_e32 %0, %1" : "+v"(a), "+v"(b));
+}
+
+// Sums over the four 16-lane rows of a wave, four values at a time: lane (row k, column c) receives the total of
+// v_k over the four lanes of column c, formed as (row0 + row1) + (row2 + row3).  Six instructions for four values,
+// against eight shuffles through LDS for the same sums as butterflies.
+__device__ __forceinline__ float rows_sum4(float v0, float v1, float v2, float v3) {
+  swap_rows16(v0, v1);
+  float a = v0 + v1;  // rows: v0 (0+1), v1 (0+1), v0 (2+3), v1 (2+3)
+  swap_rows16(v2, v3);
+  float b = v2 + v3;
+  swap_halves32(a, b);
+  return a + b;  // rows: v0, v1, v2, v3
+}
+
 }  // namespace
 
 }  // namespace gelib_hip

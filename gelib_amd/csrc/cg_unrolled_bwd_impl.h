@@ -7,8 +7,8 @@
 // C*g once per (m1,m2) and feeds two complex FMAs,
 //     ax[m1] += (C g) conj(y[m2, j])        ay[m2] += (C g) conj(x[m1, i]),
 // with all m-loops unrolled and x, y, ax, ay, g in registers.  ax is then summed over j inside aligned groups of
-// n2 lanes (DPP butterflies), ay over i with butterflies at lane distance n2 and up, and one lane per group adds
-// the result into the wave's private image of xg / yg in LDS: plain read-add-write in a fixed order, no atomics,
+// n2 lanes (DPP butterflies), ay over i with butterflies at lane distance n2 and up (row swaps when n2 = 16), and
+// the lanes that hold totals add them into the wave's private image of xg / yg in LDS: plain read-add-write in a fixed order, no atomics,
 // no barrier.  After the last pair the four images are summed and written out in contiguous rows.
 //
 // Latency hiding.  A unit (pair, run, l) requests its rows of g and then computes on them; the kernel keeps its
@@ -132,16 +132,25 @@ __device__ __forceinline__ void pair_bwd(const GParts<LCAP> &gp, PairPtr pr, Coe
       }
     });
   };
-  float2 gnext[NLP];
-  load_m(std::integral_constant<int, 0>{}, gnext);
+  // Rows of PF consecutive m are in flight at a time: all rows of the pair when there are at most kRowBudget of
+  // them (the wave then waits once per pair, and 16 waves per compute unit keep enough bytes in flight to cover
+  // the memory latency), otherwise as many m as fit the budget.  The kernels for l up to 8 hold more sums and are
+  // near the register limit of three waves per SIMD already, so their budget is smaller.
+  constexpr int kRowBudget = LCAP <= 4 ? 32 : 14;
+  constexpr int ROWS = (LTOP + 1) * (LTOP + 1) - LMIN * LMIN;  // sum of 2l+1 over the l of the pair
+  constexpr int PF = ROWS <= kRowBudget ? 2 * LTOP + 1 : (kRowBudget / NLP > 1 ? kRowBudget / NLP : 1);
+  float2 gq[PF][NLP];
+  static_for<PF>([&](auto kc) __attribute__((always_inline)) {
+    if constexpr (kc.value <= 2 * LTOP) load_m(kc, gq[kc.value]);
+  });
   static_for<2 * LTOP + 1>([&](auto mc) __attribute__((always_inline)) {
     constexpr int mi = decltype(mc)::value;
     constexpr int m = mi - LTOP;
     constexpr int MABS = cabs_(m);
     float2 gl[NLP];
 #pragma unroll
-    for (int k = 0; k < NLP; k++) gl[k] = gnext[k];
-    if constexpr (mi + 1 <= 2 * LTOP) load_m(std::integral_constant<int, mi + 1>{}, gnext);
+    for (int k = 0; k < NLP; k++) gl[k] = gq[mi % PF][k];
+    if constexpr (mi + PF <= 2 * LTOP) load_m(std::integral_constant<int, mi + PF>{}, gq[mi % PF]);
     constexpr int M1LO = (-L1 > m - L2) ? -L1 : m - L2;
     constexpr int M1HI = (L1 < m + L2) ? L1 : m + L2;
     constexpr int NP = M1HI - M1LO + 1;
@@ -197,7 +206,26 @@ __device__ __forceinline__ void pair_bwd(const GParts<LCAP> &gp, PairPtr pr, Coe
       }
     }
   }
-  if (WY) {
+  if (WY && !DIAG && N2P == 16 && span == kWave) {
+    // four lanes of a run share j (one per 16-lane row): sum them four values at a time; row k of the wave then
+    // holds value 4t + k, a value being one float of ay, and every lane adds its own into the image
+    constexpr int NV = 2 * (2 * L2 + 1);
+    const int row = (q.u >> 4) & 3, col = q.u & 15;
+    float *ya = reinterpret_cast<float *>(yacc + q.cell_local * ysize + p.yoff);
+    const bool writer = q.live && col < N2;
+    static_for<(NV + 3) / 4>([&](auto tc) __attribute__((always_inline)) {
+      constexpr int t = decltype(tc)::value;
+      auto val = [&](auto kc) __attribute__((always_inline)) {
+        constexpr int v = 4 * t + decltype(kc)::value;
+        if constexpr (v < NV) return (v & 1) ? ay[v >> 1].y : ay[v >> 1].x;
+        else return 0.f;
+      };
+      const float total = rows_sum4(val(std::integral_constant<int, 0>{}), val(std::integral_constant<int, 1>{}),
+                                    val(std::integral_constant<int, 2>{}), val(std::integral_constant<int, 3>{}));
+      const int v = 4 * t + row;  // float v of ay: row v / 2 of the part, real or imaginary
+      if (writer && v < NV) ya[((v >> 1) * N2 + col) * 2 + (v & 1)] += total;
+    });
+  } else if (WY) {
     if (!DIAG) stride_sum(ay, N2P, span);
     if (q.live && valid && (DIAG || (q.u & (span - 1)) < N2P)) {
       float2 *ya = yacc + q.cell_local * ysize + p.yoff + j;

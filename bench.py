@@ -194,6 +194,8 @@ def main():
     ap.add_argument("--cpu-samples", type=int, default=2048)
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--generic", action="store_true", help="force the shape-agnostic kernels")
+    ap.add_argument("--option", action="append", default=[], metavar="NAME=VALUE",
+                    help="library tuning option (gelib_hip_set_option), may be repeated")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run one plain 1 GiB device copy (reference dispatch for hardware-counter calibration)")
     args = ap.parse_args()
@@ -209,6 +211,9 @@ def main():
         sys.exit(1)
     cabi.lib()
     cabi.set_option("force_generic", int(args.generic))
+    for kv in args.option:
+        k, v = kv.split("=")
+        cabi.set_option(k, int(v))
     dev = torch.device("cuda:0")
     name = ALIASES.get(args.workload, args.workload)
     aux = [w for w in AUX_WORKLOADS if w == name or w.split("_")[0] == name]

@@ -21,7 +21,9 @@ struct FwdArgs {
   int npairs;
   int offs_add;     // extra channel offset (part-level calls)
   int accumulate;
-  int first_block[kMaxPairs + 1];  // blocks [first_block[p], first_block[p+1]) work on pair p
+  long long tile;                  // cells per tile; the blocks of one tile are consecutive
+  int blocks_per_tile;
+  int first_block[kMaxPairs + 1];  // inside a tile, blocks [first_block[p], first_block[p+1]) work on pair p
   int cpb[kMaxPairs];              // cells per block of pair p
 };
 

@@ -132,17 +132,20 @@ template <int LCAP, bool DIAG, int TI>
 __global__ void __launch_bounds__(kBlock) unrolled_fwd_kernel(const FwdArgs a) {
   extern __shared__ float2 lds_ops[];
   int pidx = 0, first = 0;
+  const int per_tile = a.blocks_per_tile;
+  const int tile_idx = (int)blockIdx.x / per_tile, in_tile = (int)blockIdx.x - tile_idx * per_tile;
   static_for<kMaxPairs>([&](auto k) __attribute__((always_inline)) {
-    if (k.value > 0 && k.value < a.npairs && (int)blockIdx.x >= a.first_block[k.value]) {
+    if (k.value > 0 && k.value < a.npairs && in_tile >= a.first_block[k.value]) {
       pidx = k.value;
       first = a.first_block[k.value];
     }
   });
   const PairPtr p = (PairPtr)a.pairs + pidx;
   const int cpb = pick_int(a.cpb, pidx);
-  const long long cell0 = (long long)((int)blockIdx.x - first) * cpb;
-  const long long left = a.ncells - cell0;
-  const int ncell = left < cpb ? (int)left : cpb;
+  const long long tile_end = (tile_idx + 1) * a.tile < a.ncells ? (tile_idx + 1) * a.tile : a.ncells;
+  const long long cell0 = tile_idx * a.tile + (long long)(in_tile - first) * cpb;
+  const long long left = tile_end - cell0;  // <= 0 for the surplus blocks of a short last tile
+  const int ncell = left < cpb ? (int)(left > 0 ? left : 0) : cpb;
   const int l1 = p->l1, l2 = p->l2, n1 = p->n1, n2 = p->n2;
 
   float2 *xs = lds_ops;

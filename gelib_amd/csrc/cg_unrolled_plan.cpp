@@ -12,8 +12,9 @@ namespace gelib_hip {
 
 namespace {
 
-int g_fwd_block_bytes = 384 * 1024;  // product bytes one forward block aims to write
+int g_fwd_block_bytes = 96 * 1024;   // product bytes one forward block aims to write
 int g_fwd_lds_bytes = 16 * 1024;     // LDS one forward block may use for its staged operands
+int g_fwd_cell_tile = 64;             // cells per tile of the forward launch (0 = all cells in one tile)
 int g_fwd_ti = 0;                    // 0 = widest tile that divides every n1, else force 1 / 2 / 4
 int g_bwd_enable = 1;
 int g_fwd_enable = 1;
@@ -222,6 +223,9 @@ int run_fwd(bool diag, const std::vector<VecTriple> &triples, const std::vector<
   size_t lds_bytes = 0;
   int lcap = 0;
   for (auto &t : triples) lcap = std::max(lcap, t.l);
+  // The cells are cut into tiles; the blocks of a tile (every pair, every run of cells inside the tile) have
+  // consecutive indices, so blocks that run at the same time write into the same neighbourhood of every product part.
+  const long long tile = g_fwd_cell_tile > 0 ? std::min<long long>(g_fwd_cell_tile, ncells) : ncells;
   for (int i = 0; i < a.npairs; i++) {
     const PairRec &p = plan->pairs[i];
     long long rows = 0;
@@ -234,14 +238,19 @@ int run_fwd(bool diag, const std::vector<VecTriple> &triples, const std::vector<
     const long long op_bytes = 8LL * ((2 * p.l1 + 1) * (long long)p.n1 + (2 * p.l2 + 1) * (long long)p.n2);
     cpb = std::min(cpb, std::max<long long>(1, g_fwd_lds_bytes / op_bytes));
     cpb = std::min<long long>(cpb, std::max<long long>(1, (1LL << 28) / std::max<long long>(1, U)));
-    cpb = std::min(cpb, ncells);
+    cpb = std::min(cpb, tile);
+    cpb = (tile + (tile + cpb - 1) / cpb - 1) / ((tile + cpb - 1) / cpb);  // equal shares of the tile, not a short last block
     a.cpb[i] = (int)cpb;
     lds_bytes = std::max(lds_bytes, (size_t)(cpb * op_bytes));
     a.first_block[i] = (int)nblocks;
-    nblocks += (ncells + cpb - 1) / cpb;
+    nblocks += (tile + cpb - 1) / cpb;
     if (nblocks > 0x7fffffffLL) return GELIB_HIP_ERR_ARG;
   }
-  a.first_block[a.npairs] = (int)nblocks;
+  a.first_block[a.npairs] = (int)nblocks;  // blocks of one tile
+  a.tile = tile;
+  a.blocks_per_tile = (int)nblocks;
+  nblocks *= (ncells + tile - 1) / tile;
+  if (nblocks > 0x7fffffffLL) return GELIB_HIP_ERR_ARG;
   rc = launch_unrolled_fwd(a, diag, ti, lcap, (int)nblocks, lds_bytes, s);
   if (rc) return rc;
   *used = 1;
@@ -401,6 +410,11 @@ int unrolled_set_option(const char *name, int value) {
   if (!std::strcmp(name, "fwd_lds_bytes")) {
     if (value < 1024 || value > 60 * 1024) return GELIB_HIP_ERR_ARG;
     g_fwd_lds_bytes = value;
+    return GELIB_HIP_OK;
+  }
+  if (!std::strcmp(name, "fwd_cell_tile")) {
+    if (value < 0) return GELIB_HIP_ERR_ARG;
+    g_fwd_cell_tile = value;
     return GELIB_HIP_OK;
   }
   if (!std::strcmp(name, "fwd_tile")) {

@@ -23,7 +23,7 @@ HBM_PEAK = 8.0e12  # B/s, MI355X HBM3E
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs, each scaled by what the
 # counter reads for a plain 1 GiB copy: x2.000 and x1.000); summary in profiles/.
 MEASURED_TRAFFIC = {
-    "so3vec_cg_L4_tau16_B32768_maxl4": {"so3vec_fwd": 26221027505, "so3vec_bwd": 25876776855},
+    "so3vec_cg_L4_tau16_B32768_maxl4": {"so3vec_fwd": 27148781681, "so3vec_bwd": 25959930442},
     # the backward pass of this type runs as two launches (one per gradient), each reading g: 1.88 x algorithmic
     "so3vec_diagcg_L6_n64_B131072": {"so3vec_fwd": 102052404553, "so3vec_bwd": 204010468818},
     "so3part_cg_10x10_all_l_n8_B16384": {"so3vec_fwd": 3747009028, "so3vec_bwd": 3809547747},
@@ -264,6 +264,7 @@ def main():
     ms_per_step = wall * 1e3 / args.steps
     path = cabi.last_path()
 
+
     if bwd_ms >= fwd_ms:
         dom, dom_ms, dom_bytes = "so3vec_bwd", bwd_ms, bwd_bytes
     else:
@@ -295,6 +296,21 @@ def main():
                                "sample": "first %d samples of the same batch, fwd+bwd, %.1f s" % (ns, dt),
                                "all_cores": allc}
         out["parity"] = parity
+
+    # What a plain streaming kernel reaches on these very buffers (outside the timed region): torch's fill over the
+    # product parts.  Write bandwidth on this GPU depends on where a buffer lies in memory (about 5.6 or 6.6 TB/s
+    # for one and the same kernel), so this is the yardstick beside the nominal peak.
+    def timed(fn):
+        fn()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        fn()
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b) * 1e-3
+    rbytes = sum(t.numel() * 8 for t in rs)
+    fill_GBps = rbytes / timed(lambda: [t.fill_(1.0) for t in rs]) / 1e9
+    out["config"]["streaming_reference"] = {"torch_fill_of_product_GBps": fill_GBps}
     print(json.dumps(out))
 
 

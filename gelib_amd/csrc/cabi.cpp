@@ -281,6 +281,12 @@ int vec_fwd_entry(bool diag, int nr, const gelib_part_desc *r, int nx, const gel
       t_last_path = kPathUnrolled;
       return GELIB_HIP_OK;
     }
+    rc = diag6_vec_fwd(plan, rd, xd, yd, accumulate != 0, s, &used);
+    if (rc) return rc;
+    if (used) {
+      t_last_path = kPathDiag6;
+      return GELIB_HIP_OK;
+    }
     rc = staged_vec_fwd(plan, rd, xd, yd, accumulate != 0, s, &used);
     if (rc) return rc;
     if (used) {
@@ -341,6 +347,12 @@ int vec_bwd_entry(bool diag, const gelib_part_desc *xg, const gelib_part_desc *y
     if (rc) return rc;
     if (used) {
       t_last_path = kPathUnrolled;
+      return GELIB_HIP_OK;
+    }
+    rc = diag6_vec_bwd(plan, gd, xd, yd, xgd, ygd, accumulate != 0, s, &used);
+    if (rc) return rc;
+    if (used) {
+      t_last_path = kPathDiag6;
       return GELIB_HIP_OK;
     }
     rc = staged_vec_bwd(plan, gd, xd, yd, xgd, ygd, accumulate != 0, s, &used);
@@ -633,6 +645,7 @@ int gelib_hip_set_option(const char *name, int value) {
     return GELIB_HIP_OK;
   }
   if (!std::strncmp(name, "staged_", 7)) return staged_set_option(name, value);
+  if (!std::strncmp(name, "diag6", 5)) return diag6_set_option(name, value);
   return unrolled_set_option(name, value);
 }
 

@@ -1,0 +1,55 @@
+// Argument block and table layout of the lane-per-channel Diag kernels (internal).
+#pragma once
+
+#include "cg_unrolled.h"
+
+namespace gelib_hip {
+
+constexpr int kL6 = 6;
+constexpr int kNP = kL6 + 1;      // operand parts l = 0..6
+constexpr int kNR = 2 * kL6 + 1;  // product parts l = 0..12
+constexpr int kImgRows = kNP * kNP;  // rows of all operand parts together: sum of 2l+1 = 49; part l starts at row l*l
+constexpr int kZeroFloats = 16384;   // zeros behind the tables: a row of zeros for up to 8192 channels
+constexpr int kMaxChannels = kZeroFloats / 2;
+
+constexpr int iabs(int a) { return a < 0 ? -a : a; }
+constexpr int imin(int a, int b) { return a < b ? a : b; }
+constexpr int imax(int a, int b) { return a > b ? a : b; }
+
+// Offsets (floats) of the (2l1+1) x (2l2+1) tables of all (l1,l2,l) in the bank, and its total length.
+struct TableOffsets {
+  int v[kNP][kNP][kNR];
+  int total;
+};
+constexpr TableOffsets make_table_offsets() {
+  TableOffsets t{};
+  int off = 0;
+  for (int a = 0; a <= kL6; a++)
+    for (int b = 0; b <= kL6; b++)
+      for (int c = iabs(a - b); c <= a + b; c++) {
+        t.v[a][b][c] = off;
+        off += (2 * a + 1) * (2 * b + 1);
+      }
+  t.total = off;
+  return t;
+}
+constexpr TableOffsets kTables = make_table_offsets();
+constexpr int table_off(int l1, int l2, int l) { return kTables.v[l1][l2][l]; }
+constexpr int kBankFloats = (kTables.total + 1) & ~1;  // even, so that the zeros behind it are 8-byte aligned
+
+struct Diag6Args {
+  FastPart x[kNP], y[kNP], xg[kNP], yg[kNP];  // by l; ptr == nullptr: no such part
+  FastPart r[kNR];                            // product (forward) or its gradient (backward), by l
+  const int *offs;    // device, [kNP][kNP][kNR]: first channel of the triple's block in part l, -1 = no such triple
+  const float *bank;  // device, kBankFloats coefficients followed by kZeroFloats zeros
+  long long nwaves;   // cells * groups
+  int groups;         // 64-channel groups per cell
+  int n;              // channels of every part
+  int offs_add;
+  int accumulate;
+};
+
+int launch_diag6_fwd_l6(const Diag6Args &a, hipStream_t s);  // product l up to 6
+int launch_diag6_bwd_l6(const Diag6Args &a, hipStream_t s);
+
+}  // namespace gelib_hip

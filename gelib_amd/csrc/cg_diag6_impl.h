@@ -1,0 +1,292 @@
+// DiagCGproduct of SO3vecs whose parts have l <= 6 and more than 32 channels: forward, and both gradients from one
+// pass over g, every loop over l1, l2, l, m unrolled at compile time.
+//
+// A Diag product pairs channel c of x with channel c of y, so nothing is ever summed across channels.  A wave takes
+// one cell and 64 consecutive channels, lane = channel, and walks through all (l1,l2) pairs:
+//   forward   P[m1,m2] = x[m1] y[m2] once per (m1,m2), then r_l[m1+m2] += C_l[m1,m2] P for every l of the pair; the rows
+//             of one m are complete after its m1-loop and are stored as 512 contiguous bytes each;
+//   backward  Q[m1,m2] = sum_l C_l[m1,m2] g_l[m1+m2], then ax[m1] += Q conj(y[m2]) and ay[m2] += Q conj(x[m1]).  The
+//             x-gradient of part l1 stays in registers while l2 runs and is written once; the y-gradient is kept in
+//             a wave-private image in LDS (49 rows of 64 lanes), each lane adding into its own column: no atomics, no
+//             barrier, a fixed order of additions.
+// The cell of a wave is uniform, so every row address is a scalar base plus the lane's channel: loads and stores use
+// the scalar-base form and need no address arithmetic on the vector unit.  Coefficients of all (l1,l2,l) with
+// l1, l2 <= 6 live in one table with compile-time offsets and are read with scalar loads.
+#pragma once
+
+#include "cg_diag6.h"
+#include "cg_unrolled_dev.h"
+
+namespace gelib_hip {
+
+namespace {
+
+constexpr int kRowBudget = 28;  // rows of g a lane keeps in flight
+
+typedef float v2f __attribute__((ext_vector_type(2)));
+typedef const __attribute__((address_space(1))) v2f *GlobalIn;
+typedef __attribute__((address_space(1))) v2f *GlobalOut;
+typedef const __attribute__((address_space(4))) float *CoeffPtr;
+typedef const __attribute__((address_space(4))) int *OffsPtr;
+
+struct WavePos {
+  long long cell;
+  int ch;     // the lane's channel (clamped to a valid one for lanes beyond n)
+  bool live;
+};
+
+__device__ __forceinline__ WavePos wave_pos(const Diag6Args &a, long long w) {
+  WavePos q;
+  q.cell = w / a.groups;
+  const int grp = (int)(w - q.cell * a.groups);
+  const int ch = grp * 64 + (int)(threadIdx.x & 63);
+  q.live = ch < a.n;
+  q.ch = q.live ? ch : 0;
+  return q;
+}
+
+template <int L>
+__device__ __forceinline__ void load_rows(float2 (&v)[2 * L + 1], const FastPart P, const WavePos q) {
+  GlobalIn base = (GlobalIn)P.ptr + q.cell * P.sb;
+#pragma unroll
+  for (int m = 0; m <= 2 * L; m++) {
+    const v2f t = (base + m * P.sm)[q.ch];
+    v[m] = make_float2(t.x, t.y);
+  }
+}
+
+template <int L1, int L2, int LCAP>
+__device__ __forceinline__ void fwd_pair(const Diag6Args &a, const float2 (&xv)[2 * L1 + 1], const float2 (&yv)[2 * L2 + 1],
+                                         const WavePos q) {
+  constexpr int LMIN = iabs(L1 - L2);
+  constexpr int LTOP = imin(L1 + L2, LCAP);
+  if constexpr (LMIN <= LCAP) {
+    constexpr int NL = LTOP - LMIN + 1;
+    const OffsPtr offs = (OffsPtr)a.offs + (L1 * kNP + L2) * kNR;
+    const CoeffPtr C = (CoeffPtr)a.bank;
+    const bool accumulate = a.accumulate != 0;
+    static_for<2 * LTOP + 1>([&](auto mc) __attribute__((always_inline)) {
+      constexpr int m = decltype(mc)::value - LTOP;
+      constexpr int MABS = iabs(m);
+      constexpr int M1LO = imax(-L1, m - L2), M1HI = imin(L1, m + L2);
+      float2 acc[NL];
+#pragma unroll
+      for (int k = 0; k < NL; k++) acc[k] = make_float2(0.f, 0.f);
+      static_for<M1HI - M1LO + 1>([&](auto kc) __attribute__((always_inline)) {
+        constexpr int m1 = M1LO + decltype(kc)::value;
+        constexpr int m2 = m - m1;
+        const float2 xa = xv[m1 + L1], yb = yv[m2 + L2];
+        const float pr = fmaf(-xa.y, yb.y, xa.x * yb.x), pi = fmaf(xa.y, yb.x, xa.x * yb.y);
+        static_for<NL>([&](auto dc) __attribute__((always_inline)) {
+          constexpr int dl = decltype(dc)::value;
+          constexpr int L = LMIN + dl;
+          if constexpr (L >= MABS) {
+            const float c = C[table_off(L1, L2, L) + (m1 + L1) * (2 * L2 + 1) + (m2 + L2)];
+            acc[dl].x = fmaf(c, pr, acc[dl].x);
+            acc[dl].y = fmaf(c, pi, acc[dl].y);
+          }
+        });
+      });
+      static_for<NL>([&](auto dc) __attribute__((always_inline)) {
+        constexpr int dl = decltype(dc)::value;
+        constexpr int L = LMIN + dl;
+        if constexpr (L >= MABS) {
+          const int off = offs[L];
+          if (off >= 0) {  // uniform
+            const FastPart R = a.r[L];
+            GlobalOut row = (GlobalOut)R.ptr + (q.cell * R.sb + (long long)(m + L) * R.sm + (off + a.offs_add));
+            if (q.live) {
+              v2f v = {acc[dl].x, acc[dl].y};
+              if (accumulate) v += row[q.ch];
+              row[q.ch] = v;
+            }
+          }
+        }
+      });
+    });
+  }
+}
+
+template <int LCAP>
+__global__ void __launch_bounds__(256) diag6_fwd_kernel(const Diag6Args a) {
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const long long w = (long long)blockIdx.x * 4 + wave;
+  if (w >= a.nwaves) return;
+  const WavePos q = wave_pos(a, w);
+  static_for<kNP>([&](auto l1c) __attribute__((always_inline)) {
+    constexpr int L1 = decltype(l1c)::value;
+    const FastPart X = a.x[L1];
+    if (X.ptr != nullptr) {
+      float2 xv[2 * L1 + 1];
+      load_rows<L1>(xv, X, q);
+      static_for<kNP>([&](auto l2c) __attribute__((always_inline)) {
+        constexpr int L2 = decltype(l2c)::value;
+        const FastPart Y = a.y[L2];
+        if (Y.ptr != nullptr) {
+          float2 yv[2 * L2 + 1];
+          load_rows<L2>(yv, Y, q);
+          fwd_pair<L1, L2, LCAP>(a, xv, yv, q);
+        }
+      });
+    }
+  });
+}
+
+// One pair of the backward pass: every l of the pair together, one row number m = m1 + m2 at a time.
+template <int L1, int L2, int LCAP>
+__device__ __forceinline__ void bwd_pair(const Diag6Args &a, const float2 (&xv)[2 * L1 + 1], const float2 (&yv)[2 * L2 + 1],
+                                         float2 (&ax)[2 * L1 + 1], float2 *yimg, const WavePos q) {
+  constexpr int LMIN = iabs(L1 - L2);
+  constexpr int LTOP = imin(L1 + L2, LCAP);
+  if constexpr (LMIN <= LCAP) {
+    constexpr int NL = LTOP - LMIN + 1;
+    constexpr int ROWS = (LTOP + 1) * (LTOP + 1) - LMIN * LMIN;
+    constexpr int PF = ROWS <= kRowBudget ? 2 * LTOP + 1 : (kRowBudget / NL > 1 ? kRowBudget / NL : 1);
+    const OffsPtr offs = (OffsPtr)a.offs + (L1 * kNP + L2) * kNR;
+    const CoeffPtr C = (CoeffPtr)a.bank;
+    // a triple that is not there reads rows of zeros against a table of zeros, so the arithmetic has no branches
+    GlobalIn gbase[NL];
+    int gsm[NL];
+    int coff[NL];
+    static_for<NL>([&](auto dc) __attribute__((always_inline)) {
+      constexpr int dl = decltype(dc)::value;
+      constexpr int L = LMIN + dl;
+      const int off = offs[L];
+      const FastPart G = a.r[L];
+      const bool present = off >= 0;
+      gbase[dl] = present ? (GlobalIn)G.ptr + (q.cell * G.sb + (off + a.offs_add)) : (GlobalIn)(a.bank + kBankFloats);
+      gsm[dl] = present ? G.sm : 0;
+      coff[dl] = present ? table_off(L1, L2, L) : kBankFloats;
+    });
+    float2 ay[2 * L2 + 1];
+#pragma unroll
+    for (int m2 = 0; m2 <= 2 * L2; m2++) ay[m2] = make_float2(0.f, 0.f);
+    auto load_m = [&](auto mc, float2(&dst)[NL]) __attribute__((always_inline)) {
+      constexpr int m = decltype(mc)::value - LTOP;
+      static_for<NL>([&](auto dc) __attribute__((always_inline)) {
+        constexpr int dl = decltype(dc)::value;
+        constexpr int L = LMIN + dl;
+        if constexpr (L >= iabs(m)) {
+          const v2f t = (gbase[dl] + (m + L) * gsm[dl])[q.ch];
+          dst[dl] = make_float2(t.x, t.y);
+        }
+      });
+    };
+    float2 gq[PF][NL];
+    static_for<PF>([&](auto kc) __attribute__((always_inline)) {
+      if constexpr (kc.value <= 2 * LTOP) load_m(kc, gq[kc.value]);
+    });
+    static_for<2 * LTOP + 1>([&](auto mc) __attribute__((always_inline)) {
+      constexpr int mi = decltype(mc)::value;
+      constexpr int m = mi - LTOP;
+      constexpr int MABS = iabs(m);
+      float2 gl[NL];
+#pragma unroll
+      for (int k = 0; k < NL; k++) gl[k] = gq[mi % PF][k];
+      if constexpr (mi + PF <= 2 * LTOP) load_m(std::integral_constant<int, mi + PF>{}, gq[mi % PF]);
+      constexpr int M1LO = imax(-L1, m - L2), M1HI = imin(L1, m + L2);
+      static_for<M1HI - M1LO + 1>([&](auto kc) __attribute__((always_inline)) {
+        constexpr int m1 = M1LO + decltype(kc)::value;
+        constexpr int m2 = m - m1;
+        float qr = 0.f, qi = 0.f;
+        static_for<NL>([&](auto dc) __attribute__((always_inline)) {
+          constexpr int dl = decltype(dc)::value;
+          if constexpr (LMIN + dl >= MABS) {
+            const float c = C[coff[dl] + (m1 + L1) * (2 * L2 + 1) + (m2 + L2)];
+            qr = fmaf(c, gl[dl].x, qr);
+            qi = fmaf(c, gl[dl].y, qi);
+          }
+        });
+        const float2 yc = yv[m2 + L2], xc = xv[m1 + L1];
+        ax[m1 + L1].x = fmaf(qr, yc.x, ax[m1 + L1].x);
+        ax[m1 + L1].x = fmaf(qi, yc.y, ax[m1 + L1].x);
+        ax[m1 + L1].y = fmaf(qi, yc.x, ax[m1 + L1].y);
+        ax[m1 + L1].y = fmaf(-qr, yc.y, ax[m1 + L1].y);
+        ay[m2 + L2].x = fmaf(qr, xc.x, ay[m2 + L2].x);
+        ay[m2 + L2].x = fmaf(qi, xc.y, ay[m2 + L2].x);
+        ay[m2 + L2].y = fmaf(qi, xc.x, ay[m2 + L2].y);
+        ay[m2 + L2].y = fmaf(-qr, xc.y, ay[m2 + L2].y);
+        __builtin_amdgcn_sched_barrier(0);
+      });
+      __builtin_amdgcn_sched_barrier(0);
+    });
+#pragma unroll
+    for (int m1 = 0; m1 <= 2 * L1; m1++) asm volatile("" : "+v"(ax[m1].x), "+v"(ax[m1].y));
+    float2 *col = yimg + (L2 * L2) * 64 + (threadIdx.x & 63);
+#pragma unroll
+    for (int m2 = 0; m2 <= 2 * L2; m2++) {
+      float2 o = col[m2 * 64];
+      o.x += ay[m2].x;
+      o.y += ay[m2].y;
+      col[m2 * 64] = o;
+    }
+  }
+}
+
+template <int L>
+__device__ __forceinline__ void store_rows(const float2 *v, int vstride, const FastPart P, const WavePos q, bool accumulate) {
+  GlobalOut base = (GlobalOut)P.ptr + q.cell * P.sb;
+  if (!q.live) return;
+#pragma unroll
+  for (int m = 0; m <= 2 * L; m++) {
+    v2f o = {v[m * vstride].x, v[m * vstride].y};
+    GlobalOut row = base + m * P.sm;
+    if (accumulate) o += row[q.ch];
+    row[q.ch] = o;
+  }
+}
+
+template <int LCAP>
+__global__ void __launch_bounds__(64) diag6_bwd_kernel(const Diag6Args a) {
+  __shared__ float2 yimg[kImgRows * 64];
+  const long long w = blockIdx.x;
+  const WavePos q = wave_pos(a, w);
+  const int lane = threadIdx.x & 63;
+  const bool accumulate = a.accumulate != 0;
+#pragma unroll
+  for (int r = 0; r < kImgRows; r++) yimg[r * 64 + lane] = make_float2(0.f, 0.f);
+  static_for<kNP>([&](auto l1c) __attribute__((always_inline)) {
+    constexpr int L1 = decltype(l1c)::value;
+    const FastPart X = a.x[L1];
+    if (X.ptr != nullptr) {
+      float2 xv[2 * L1 + 1], ax[2 * L1 + 1];
+      load_rows<L1>(xv, X, q);
+#pragma unroll
+      for (int m1 = 0; m1 <= 2 * L1; m1++) ax[m1] = make_float2(0.f, 0.f);
+      static_for<kNP>([&](auto l2c) __attribute__((always_inline)) {
+        constexpr int L2 = decltype(l2c)::value;
+        const FastPart Y = a.y[L2];
+        if (Y.ptr != nullptr) {
+          float2 yv[2 * L2 + 1];
+          load_rows<L2>(yv, Y, q);
+          bwd_pair<L1, L2, LCAP>(a, xv, yv, ax, yimg, q);
+        }
+      });
+      store_rows<L1>(ax, 1, a.xg[L1], q, accumulate);
+    }
+  });
+  static_for<kNP>([&](auto l2c) __attribute__((always_inline)) {
+    constexpr int L2 = decltype(l2c)::value;
+    const FastPart YG = a.yg[L2];
+    if (YG.ptr != nullptr) store_rows<L2>(yimg + (L2 * L2) * 64 + lane, 64, YG, q, accumulate);
+  });
+}
+
+template <int LCAP>
+int launch_diag6_fwd_variant(const Diag6Args &a, hipStream_t s) {
+  const unsigned nblocks = (unsigned)((a.nwaves + 3) / 4);
+  hipLaunchKernelGGL((diag6_fwd_kernel<LCAP>), dim3(nblocks), dim3(256), 0, s, a);
+  GELIB_HIP_TRY(hipGetLastError());
+  return GELIB_HIP_OK;
+}
+
+template <int LCAP>
+int launch_diag6_bwd_variant(const Diag6Args &a, hipStream_t s) {
+  hipLaunchKernelGGL((diag6_bwd_kernel<LCAP>), dim3((unsigned)a.nwaves), dim3(64), 0, s, a);
+  GELIB_HIP_TRY(hipGetLastError());
+  return GELIB_HIP_OK;
+}
+
+}  // namespace
+
+}  // namespace gelib_hip

@@ -1,0 +1,146 @@
+// Host side of the lane-per-channel Diag kernels: which products they take, the coefficient table with its fixed
+// layout, the per-type offset table (both cached on the device), and the argument block.
+#include <cstring>
+#include <map>
+#include <mutex>
+#include <vector>
+
+#include "cg_diag6.h"
+
+namespace gelib_hip {
+
+namespace {
+
+// ---- host side ---------------------------------------------------------------------------------------------------
+
+std::mutex g_mutex;
+std::map<int, float *> g_banks;                     // device -> coefficient table
+std::map<std::pair<int, std::vector<int>>, int *> g_offs;  // (device, offsets) -> device copy
+int g_enable = 1;
+
+int device_bank(const float **out) {
+  int dev = 0;
+  GELIB_HIP_TRY(hipGetDevice(&dev));
+  std::lock_guard<std::mutex> lock(g_mutex);
+  auto it = g_banks.find(dev);
+  if (it == g_banks.end()) {
+    std::vector<float> h((size_t)kBankFloats + kZeroFloats, 0.f);
+    for (int a = 0; a <= kL6; a++)
+      for (int b = 0; b <= kL6; b++)
+        for (int c = iabs(a - b); c <= a + b; c++) cg_matrix_host(a, b, c, h.data() + table_off(a, b, c));
+    float *d = nullptr;
+    GELIB_HIP_TRY(hipMalloc((void **)&d, h.size() * sizeof(float)));
+    GELIB_HIP_TRY(hipMemcpy(d, h.data(), h.size() * sizeof(float), hipMemcpyHostToDevice));
+    it = g_banks.emplace(dev, d).first;
+  }
+  *out = it->second;
+  return GELIB_HIP_OK;
+}
+
+int device_offs(const std::vector<int> &h, const int **out) {
+  int dev = 0;
+  GELIB_HIP_TRY(hipGetDevice(&dev));
+  std::lock_guard<std::mutex> lock(g_mutex);
+  auto key = std::make_pair(dev, h);
+  auto it = g_offs.find(key);
+  if (it == g_offs.end()) {
+    int *d = nullptr;
+    GELIB_HIP_TRY(hipMalloc((void **)&d, h.size() * sizeof(int)));
+    GELIB_HIP_TRY(hipMemcpy(d, h.data(), h.size() * sizeof(int), hipMemcpyHostToDevice));
+    it = g_offs.emplace(key, d).first;
+  }
+  *out = it->second;
+  return GELIB_HIP_OK;
+}
+
+// Fills the argument block; *ok = false when the product is not one this family takes.
+int make_args(const VecPlan &plan, const std::vector<const gelib_part_desc *> &r,
+              const std::vector<const gelib_part_desc *> &x, const std::vector<const gelib_part_desc *> &y,
+              const std::vector<const gelib_part_desc *> *xg, const std::vector<const gelib_part_desc *> *yg,
+              bool r_is_dest, Diag6Args *a, int *lcap, bool *ok) {
+  *ok = false;
+  if (!g_enable || !plan.diag) return GELIB_HIP_OK;
+  std::vector<FastPart> fx, fy, fr, fxg, fyg;
+  std::vector<std::pair<int, int>> lx, ly, lr;
+  if (!lists_to_fast(x, plan.E, false, &fx, &lx) || !lists_to_fast(y, plan.E, false, &fy, &ly) ||
+      !lists_to_fast(r, plan.E, r_is_dest, &fr, &lr))
+    return GELIB_HIP_OK;
+  if (xg && !lists_to_fast(*xg, plan.E, true, &fxg, nullptr)) return GELIB_HIP_OK;
+  if (yg && !lists_to_fast(*yg, plan.E, true, &fyg, nullptr)) return GELIB_HIP_OK;
+  const int n = lx[0].second;
+  if (n <= 32 || n > kMaxChannels) return GELIB_HIP_OK;
+  for (auto &p : lx)
+    if (p.first > kL6 || p.second != n) return GELIB_HIP_OK;
+  for (auto &p : ly)
+    if (p.first > kL6 || p.second != n) return GELIB_HIP_OK;
+  for (auto &p : lr)
+    if (p.first > 2 * kL6) return GELIB_HIP_OK;
+  std::memset(a, 0, sizeof(*a));
+  for (size_t i = 0; i < fx.size(); i++) a->x[lx[i].first] = fx[i];
+  for (size_t i = 0; i < fy.size(); i++) a->y[ly[i].first] = fy[i];
+  for (size_t i = 0; i < fr.size(); i++) a->r[lr[i].first] = fr[i];
+  for (size_t i = 0; i < fxg.size(); i++) a->xg[lx[i].first] = fxg[i];
+  for (size_t i = 0; i < fyg.size(); i++) a->yg[ly[i].first] = fyg[i];
+  std::vector<int> offs((size_t)kNP * kNP * kNR, -1);
+  *lcap = 0;
+  for (auto &t : plan.triples) {
+    offs[((size_t)t.l1 * kNP + t.l2) * kNR + t.l] = t.offs;
+    *lcap = std::max(*lcap, t.l);
+  }
+  int rc = device_offs(offs, &a->offs);
+  if (rc) return rc;
+  if ((rc = device_bank(&a->bank))) return rc;
+  const long long ncells = plan.E[0] * plan.E[1] * plan.E[2];
+  a->groups = (n + 63) / 64;
+  a->n = n;
+  a->nwaves = ncells * a->groups;
+  if (a->nwaves > 0x7fffffffLL) return GELIB_HIP_OK;
+  *ok = true;
+  return GELIB_HIP_OK;
+}
+
+}  // namespace
+
+int diag6_vec_fwd(const VecPlan &plan, const std::vector<const gelib_part_desc *> &r,
+                  const std::vector<const gelib_part_desc *> &x, const std::vector<const gelib_part_desc *> &y,
+                  bool accumulate, hipStream_t s, int *used) {
+  *used = 0;
+  Diag6Args a;
+  int lcap = 0;
+  bool ok = false;
+  int rc = make_args(plan, r, x, y, nullptr, nullptr, true, &a, &lcap, &ok);
+  if (rc || !ok) return rc;
+  if (lcap > kL6) return GELIB_HIP_OK;  // kernels are built for products capped at l = 6
+  a.accumulate = accumulate ? 1 : 0;
+  if ((rc = launch_diag6_fwd_l6(a, s))) return rc;
+  *used = 1;
+  return GELIB_HIP_OK;
+}
+
+int diag6_vec_bwd(const VecPlan &plan, const std::vector<const gelib_part_desc *> &g,
+                  const std::vector<const gelib_part_desc *> &x, const std::vector<const gelib_part_desc *> &y,
+                  const std::vector<const gelib_part_desc *> &xg, const std::vector<const gelib_part_desc *> &yg,
+                  bool accumulate, hipStream_t s, int *used) {
+  *used = 0;
+  if (xg.empty() || yg.empty()) return GELIB_HIP_OK;  // one gradient alone goes to the other kernel families
+  Diag6Args a;
+  int lcap = 0;
+  bool ok = false;
+  int rc = make_args(plan, g, x, y, &xg, &yg, false, &a, &lcap, &ok);
+  if (rc || !ok) return rc;
+  if (lcap > kL6) return GELIB_HIP_OK;
+  a.accumulate = accumulate ? 1 : 0;
+  if ((rc = launch_diag6_bwd_l6(a, s))) return rc;
+  *used = 1;
+  return GELIB_HIP_OK;
+}
+
+int diag6_set_option(const char *name, int value) {
+  if (!std::strcmp(name, "diag6")) {
+    g_enable = value;
+    return GELIB_HIP_OK;
+  }
+  return GELIB_HIP_ERR_ARG;
+}
+
+}  // namespace gelib_hip

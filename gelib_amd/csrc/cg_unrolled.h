@@ -76,4 +76,14 @@ int unrolled_vec_bwd(const VecPlan &plan, const std::vector<const gelib_part_des
                      bool accumulate, hipStream_t s, int *used);
 int unrolled_set_option(const char *name, int value);
 
+// Diag products of parts with l <= 6 and more than 32 channels, one lane per channel (cg_diag6.hip).
+int diag6_vec_fwd(const VecPlan &plan, const std::vector<const gelib_part_desc *> &r,
+                  const std::vector<const gelib_part_desc *> &x, const std::vector<const gelib_part_desc *> &y,
+                  bool accumulate, hipStream_t s, int *used);
+int diag6_vec_bwd(const VecPlan &plan, const std::vector<const gelib_part_desc *> &g,
+                  const std::vector<const gelib_part_desc *> &x, const std::vector<const gelib_part_desc *> &y,
+                  const std::vector<const gelib_part_desc *> &xg, const std::vector<const gelib_part_desc *> &yg,
+                  bool accumulate, hipStream_t s, int *used);
+int diag6_set_option(const char *name, int value);
+
 }  // namespace gelib_hip

@@ -1,0 +1,102 @@
+"""GPU parity of the lane-per-channel Diag kernels (operand l up to 6, more than 32 channels, product l up to 6):
+gelib_hip_last_path() == 4, results against the CPU oracle in float32 and float64."""
+import numpy as np
+import pytest
+
+from oracle import cg_oracle as ora
+from tests import gpu_util as U
+
+pytestmark = pytest.mark.gpu
+
+torch = pytest.importorskip("torch")
+
+DIAG6 = 4
+
+
+@pytest.fixture(scope="module")
+def cabi():
+    assert torch.cuda.is_available(), "GPU tests need a GPU"
+    from gelib_amd import cabi as c
+    c.lib()
+    c.set_option("force_generic", 0)
+    c.set_option("diag6", 1)
+    return c
+
+
+def c128(L):
+    return [a.astype(np.complex128) for a in L]
+
+
+CASES = [
+    # (B, tau_x, tau_y, maxl)
+    (5, {l: 64 for l in range(7)}, {l: 64 for l in range(7)}, 6),      # the benchmark type, small batch
+    (3, {l: 96 for l in range(6)}, {l: 96 for l in range(6)}, 5),      # two channel groups, the second half empty
+    (4, {0: 40, 5: 40}, {1: 40, 6: 40}, 6),                            # parts missing, 40 of 64 lanes live
+    (2, {6: 64}, {6: 64}, 6),                                          # one pair, l from 0 to 6 of 0..12
+    (3, {2: 64, 6: 64}, {3: 64, 5: 64}, 4),                            # capped below the largest operand l
+    (1, {l: 200 for l in range(7)}, {l: 200 for l in range(7)}, 6),    # four groups, one cell
+    (70, {5: 33}, {4: 33}, 6),                                         # the smallest channel count the family takes
+]
+
+
+@pytest.mark.parametrize("B,tx,ty,maxl", CASES)
+def test_diag6_vec(cabi, B, tx, ty, maxl):
+    seed = 900 + B
+    xs = [U.seeded(seed + l, B, 2 * l + 1, n) for l, n in sorted(tx.items())]
+    ys = [U.seeded(seed + 50 + l, B, 2 * l + 1, n) for l, n in sorted(ty.items())]
+    r32 = ora.vec_fwd(xs, ys, maxl, True)
+    r64 = ora.vec_fwd(c128(xs), c128(ys), maxl, True)
+    gs = [U.seeded(seed + 100 + i, *p.shape) for i, p in enumerate(r32)]
+    xg32, yg32 = ora.vec_bwd(gs, xs, ys, True)
+    xg64, yg64 = ora.vec_bwd(c128(gs), c128(xs), c128(ys), True)
+    dxs, dys, dgs = [U.dev(a) for a in xs], [U.dev(a) for a in ys], [U.dev(a) for a in gs]
+    drs = [torch.full(p.shape, 7.0 + 1j, dtype=torch.complex64, device="cuda") for p in r32]
+    cabi.so3vec_fwd(drs, dxs, dys, accumulate=False, diag=True)
+    assert cabi.last_path() == DIAG6
+    dxg = [torch.full(a.shape, 3.0 - 2j, dtype=torch.complex64, device="cuda") for a in xs]
+    dyg = [torch.full(a.shape, 3.0 - 2j, dtype=torch.complex64, device="cuda") for a in ys]
+    cabi.so3vec_bwd(dxg, dyg, dgs, dxs, dys, accumulate=False, diag=True)
+    assert cabi.last_path() == DIAG6
+    torch.cuda.synchronize()
+    tag = "B%d %s x %s maxl %d" % (B, tx, ty, maxl)
+    for a, b, c in zip(drs, r32, r64):
+        U.assert_parity(U.host(a), b, c, "fwd " + tag)
+    for a, b, c in zip(dxg, xg32, xg64):
+        U.assert_parity(U.host(a), b, c, "xg " + tag, slack=4.0)
+    for a, b, c in zip(dyg, yg32, yg64):
+        U.assert_parity(U.host(a), b, c, "yg " + tag, slack=4.0)
+    # accumulate mode adds on top of what is there
+    drs2 = [a.clone() for a in drs]
+    cabi.so3vec_fwd(drs2, dxs, dys, accumulate=True, diag=True)
+    dxg2, dyg2 = [a.clone() for a in dxg], [a.clone() for a in dyg]
+    cabi.so3vec_bwd(dxg2, dyg2, dgs, dxs, dys, accumulate=True, diag=True)
+    assert cabi.last_path() == DIAG6
+    torch.cuda.synchronize()
+    for a, b in zip(drs2, drs):
+        assert U.gate_excess(U.host(a), 2 * U.host(b)) <= 1.0
+    for a, b in zip(dxg2 + dyg2, dxg + dyg):
+        assert U.gate_excess(U.host(a), 2 * U.host(b), rtol=2e-5, atol=2e-5) <= 1.0
+
+
+def test_diag6_declines_what_it_cannot_do(cabi):
+    # a broadcast operand whose gradient is wanted, a product above l = 6, 32 channels or fewer: other families run
+    x = [U.dev(U.seeded(1, 1, 13, 64))]
+    y = [U.dev(U.seeded(2, 4, 13, 64))]
+    r = [torch.zeros(4, 2 * l + 1, 64, dtype=torch.complex64, device="cuda") for l in range(13)]
+    cabi.so3vec_fwd(r, x, y, accumulate=False, diag=True)
+    assert cabi.last_path() != DIAG6          # product l up to 12
+    want = ora.vec_fwd([U.host(x[0])], [U.host(y[0])], -1, True)
+    for a, b in zip(r, want):
+        assert U.gate_excess(U.host(a), b) <= 1.0
+    r6 = r[:7]
+    cabi.so3vec_fwd(r6, x, y, accumulate=False, diag=True)
+    assert cabi.last_path() == DIAG6          # a broadcast x is fine going forward
+    for a, b in zip(r6, want[:7]):
+        assert U.gate_excess(U.host(a), b) <= 1.0
+    xg, yg = [torch.zeros_like(x[0])], [torch.zeros_like(y[0])]
+    cabi.so3vec_bwd(xg, yg, r6, x, y, accumulate=False, diag=True)
+    assert cabi.last_path() != DIAG6          # its gradient needs a sum over the batch
+    x32 = [U.dev(U.seeded(3, 2, 11, 32))]
+    r32 = [torch.zeros(2, 2 * l + 1, 32, dtype=torch.complex64, device="cuda") for l in range(7)]
+    cabi.so3vec_fwd(r32, x32, x32, accumulate=False, diag=True)
+    assert cabi.last_path() != DIAG6

@@ -29,9 +29,31 @@ typedef __attribute__((address_space(1))) v2f *GlobalOut;
 typedef const __attribute__((address_space(4))) float *CoeffPtr;
 typedef const __attribute__((address_space(4))) int *OffsPtr;
 
+// Rows are addressed as a wave-uniform byte pointer plus the lane's byte offset (32 bits, unsigned): the form the
+// scalar-base load/store instructions take, so no address arithmetic runs on the vector unit.
+typedef __attribute__((address_space(1))) char *RowPtr;
+
+// (The empty asm keeps the widening of the offset next to its use; hoisted out of the block, the instruction selector
+// no longer sees base + 32-bit offset and falls back to a 64-bit vector add per access.)
+__device__ __forceinline__ float2 row_load(RowPtr row, unsigned lane_off) {
+  asm volatile("" : "+v"(lane_off));
+  const v2f t = *(GlobalIn)(row + lane_off);
+  return make_float2(t.x, t.y);
+}
+__device__ __forceinline__ void row_store(RowPtr row, unsigned lane_off, float2 v, bool accumulate) {
+  v2f o = {v.x, v.y};
+  if (accumulate) {
+    unsigned lo = lane_off;
+    asm volatile("" : "+v"(lo));
+    o += *(GlobalOut)(row + lo);
+  }
+  asm volatile("" : "+v"(lane_off));
+  *(GlobalOut)(row + lane_off) = o;
+}
+
 struct WavePos {
   long long cell;
-  int ch;     // the lane's channel (clamped to a valid one for lanes beyond n)
+  unsigned lane_off;  // byte offset of the lane's channel in a row (a valid channel also for lanes beyond n)
   bool live;
 };
 
@@ -41,23 +63,26 @@ __device__ __forceinline__ WavePos wave_pos(const Diag6Args &a, long long w) {
   const int grp = (int)(w - q.cell * a.groups);
   const int ch = grp * 64 + (int)(threadIdx.x & 63);
   q.live = ch < a.n;
-  q.ch = q.live ? ch : 0;
+  q.lane_off = q.live ? (unsigned)ch * 8u : 0u;
   return q;
 }
 
+// Row 0 of a part in the wave's cell, and the distance between its rows in bytes.
+__device__ __forceinline__ RowPtr cell_row0(const FastPart P, long long cell) { return (RowPtr)P.ptr + cell * P.sb * 8; }
+__device__ __forceinline__ long long row_step(const FastPart P) { return (long long)P.sm * 8; }
+
 template <int L>
-__device__ __forceinline__ void load_rows(float2 (&v)[2 * L + 1], const FastPart P, const WavePos q) {
-  GlobalIn base = (GlobalIn)P.ptr + q.cell * P.sb;
+__device__ __forceinline__ void load_rows(float2 (&v)[2 * L + 1], RowPtr row, long long step, const WavePos q) {
 #pragma unroll
   for (int m = 0; m <= 2 * L; m++) {
-    const v2f t = (base + m * P.sm)[q.ch];
-    v[m] = make_float2(t.x, t.y);
+    v[m] = row_load(row, q.lane_off);
+    row += step;
   }
 }
 
 template <int L1, int L2, int LCAP>
-__device__ __forceinline__ void fwd_pair(const Diag6Args &a, const float2 (&xv)[2 * L1 + 1], const float2 (&yv)[2 * L2 + 1],
-                                         const WavePos q) {
+__device__ __forceinline__ void fwd_pair(const Diag6Args &a, const float2 (&xv)[2 * L1 + 1],
+                                         const float2 (&yv)[2 * L2 + 1], const WavePos q) {
   constexpr int LMIN = iabs(L1 - L2);
   constexpr int LTOP = imin(L1 + L2, LCAP);
   if constexpr (LMIN <= LCAP) {
@@ -65,6 +90,15 @@ __device__ __forceinline__ void fwd_pair(const Diag6Args &a, const float2 (&xv)[
     const OffsPtr offs = (OffsPtr)a.offs + (L1 * kNP + L2) * kNR;
     const CoeffPtr C = (CoeffPtr)a.bank;
     const bool accumulate = a.accumulate != 0;
+    // the row of part l that the next m of that part is stored to; a triple that is not there is never stored
+    RowPtr row[NL];
+    bool present[NL];
+    static_for<NL>([&](auto dc) __attribute__((always_inline)) {
+      constexpr int dl = decltype(dc)::value;
+      const int off = offs[LMIN + dl];
+      present[dl] = off >= 0;
+      row[dl] = cell_row0(a.r[LMIN + dl], q.cell) + (long long)(off + a.offs_add) * 8;
+    });
     static_for<2 * LTOP + 1>([&](auto mc) __attribute__((always_inline)) {
       constexpr int m = decltype(mc)::value - LTOP;
       constexpr int MABS = iabs(m);
@@ -91,16 +125,8 @@ __device__ __forceinline__ void fwd_pair(const Diag6Args &a, const float2 (&xv)[
         constexpr int dl = decltype(dc)::value;
         constexpr int L = LMIN + dl;
         if constexpr (L >= MABS) {
-          const int off = offs[L];
-          if (off >= 0) {  // uniform
-            const FastPart R = a.r[L];
-            GlobalOut row = (GlobalOut)R.ptr + (q.cell * R.sb + (long long)(m + L) * R.sm + (off + a.offs_add));
-            if (q.live) {
-              v2f v = {acc[dl].x, acc[dl].y};
-              if (accumulate) v += row[q.ch];
-              row[q.ch] = v;
-            }
-          }
+          if (present[dl] && q.live) row_store(row[dl], q.lane_off, acc[dl], accumulate);
+          row[dl] += row_step(a.r[L]);
         }
       });
     });
@@ -115,16 +141,14 @@ __global__ void __launch_bounds__(256) diag6_fwd_kernel(const Diag6Args a) {
   const WavePos q = wave_pos(a, w);
   static_for<kNP>([&](auto l1c) __attribute__((always_inline)) {
     constexpr int L1 = decltype(l1c)::value;
-    const FastPart X = a.x[L1];
-    if (X.ptr != nullptr) {
+    if (a.x[L1].ptr != nullptr) {
       float2 xv[2 * L1 + 1];
-      load_rows<L1>(xv, X, q);
+      load_rows<L1>(xv, cell_row0(a.x[L1], q.cell), row_step(a.x[L1]), q);
       static_for<kNP>([&](auto l2c) __attribute__((always_inline)) {
         constexpr int L2 = decltype(l2c)::value;
-        const FastPart Y = a.y[L2];
-        if (Y.ptr != nullptr) {
+        if (a.y[L2].ptr != nullptr) {
           float2 yv[2 * L2 + 1];
-          load_rows<L2>(yv, Y, q);
+          load_rows<L2>(yv, cell_row0(a.y[L2], q.cell), row_step(a.y[L2]), q);
           fwd_pair<L1, L2, LCAP>(a, xv, yv, q);
         }
       });
@@ -134,8 +158,9 @@ __global__ void __launch_bounds__(256) diag6_fwd_kernel(const Diag6Args a) {
 
 // One pair of the backward pass: every l of the pair together, one row number m = m1 + m2 at a time.
 template <int L1, int L2, int LCAP>
-__device__ __forceinline__ void bwd_pair(const Diag6Args &a, const float2 (&xv)[2 * L1 + 1], const float2 (&yv)[2 * L2 + 1],
-                                         float2 (&ax)[2 * L1 + 1], float2 *yimg, const WavePos q) {
+__device__ __forceinline__ void bwd_pair(const Diag6Args &a, const float2 (&xv)[2 * L1 + 1],
+                                         const float2 (&yv)[2 * L2 + 1], float2 (&ax)[2 * L1 + 1], float2 *yimg,
+                                         const WavePos q) {
   constexpr int LMIN = iabs(L1 - L2);
   constexpr int LTOP = imin(L1 + L2, LCAP);
   if constexpr (LMIN <= LCAP) {
@@ -144,19 +169,17 @@ __device__ __forceinline__ void bwd_pair(const Diag6Args &a, const float2 (&xv)[
     constexpr int PF = ROWS <= kRowBudget ? 2 * LTOP + 1 : (kRowBudget / NL > 1 ? kRowBudget / NL : 1);
     const OffsPtr offs = (OffsPtr)a.offs + (L1 * kNP + L2) * kNR;
     const CoeffPtr C = (CoeffPtr)a.bank;
-    // a triple that is not there reads rows of zeros against a table of zeros, so the arithmetic has no branches
-    GlobalIn gbase[NL];
-    int gsm[NL];
-    int coff[NL];
+    // a triple that is not there reads a row of zeros (its coefficients then do not matter), so the arithmetic has
+    // no branches; row[dl] is the row of part l that the next m of that part is read from
+    RowPtr row[NL];
+    long long step[NL];
     static_for<NL>([&](auto dc) __attribute__((always_inline)) {
       constexpr int dl = decltype(dc)::value;
       constexpr int L = LMIN + dl;
       const int off = offs[L];
-      const FastPart G = a.r[L];
       const bool present = off >= 0;
-      gbase[dl] = present ? (GlobalIn)G.ptr + (q.cell * G.sb + (off + a.offs_add)) : (GlobalIn)(a.bank + kBankFloats);
-      gsm[dl] = present ? G.sm : 0;
-      coff[dl] = present ? table_off(L1, L2, L) : kBankFloats;
+      row[dl] = present ? cell_row0(a.r[L], q.cell) + (long long)(off + a.offs_add) * 8 : (RowPtr)(a.bank + kBankFloats);
+      step[dl] = present ? row_step(a.r[L]) : 0;
     });
     float2 ay[2 * L2 + 1];
 #pragma unroll
@@ -165,10 +188,9 @@ __device__ __forceinline__ void bwd_pair(const Diag6Args &a, const float2 (&xv)[
       constexpr int m = decltype(mc)::value - LTOP;
       static_for<NL>([&](auto dc) __attribute__((always_inline)) {
         constexpr int dl = decltype(dc)::value;
-        constexpr int L = LMIN + dl;
-        if constexpr (L >= iabs(m)) {
-          const v2f t = (gbase[dl] + (m + L) * gsm[dl])[q.ch];
-          dst[dl] = make_float2(t.x, t.y);
+        if constexpr (LMIN + dl >= iabs(m)) {
+          dst[dl] = row_load(row[dl], q.lane_off);
+          row[dl] += step[dl];
         }
       });
     };
@@ -191,8 +213,9 @@ __device__ __forceinline__ void bwd_pair(const Diag6Args &a, const float2 (&xv)[
         float qr = 0.f, qi = 0.f;
         static_for<NL>([&](auto dc) __attribute__((always_inline)) {
           constexpr int dl = decltype(dc)::value;
-          if constexpr (LMIN + dl >= MABS) {
-            const float c = C[coff[dl] + (m1 + L1) * (2 * L2 + 1) + (m2 + L2)];
+          constexpr int L = LMIN + dl;
+          if constexpr (L >= MABS) {
+            const float c = C[table_off(L1, L2, L) + (m1 + L1) * (2 * L2 + 1) + (m2 + L2)];
             qr = fmaf(c, gl[dl].x, qr);
             qi = fmaf(c, gl[dl].y, qi);
           }
@@ -224,15 +247,13 @@ __device__ __forceinline__ void bwd_pair(const Diag6Args &a, const float2 (&xv)[
 }
 
 template <int L>
-__device__ __forceinline__ void store_rows(const float2 *v, int vstride, const FastPart P, const WavePos q, bool accumulate) {
-  GlobalOut base = (GlobalOut)P.ptr + q.cell * P.sb;
+__device__ __forceinline__ void store_rows(const float2 *v, int vstride, RowPtr row, long long step, const WavePos q,
+                                           bool accumulate) {
   if (!q.live) return;
 #pragma unroll
   for (int m = 0; m <= 2 * L; m++) {
-    v2f o = {v[m * vstride].x, v[m * vstride].y};
-    GlobalOut row = base + m * P.sm;
-    if (accumulate) o += row[q.ch];
-    row[q.ch] = o;
+    row_store(row, q.lane_off, v[m * vstride], accumulate);
+    row += step;
   }
 }
 
@@ -247,28 +268,28 @@ __global__ void __launch_bounds__(64) diag6_bwd_kernel(const Diag6Args a) {
   for (int r = 0; r < kImgRows; r++) yimg[r * 64 + lane] = make_float2(0.f, 0.f);
   static_for<kNP>([&](auto l1c) __attribute__((always_inline)) {
     constexpr int L1 = decltype(l1c)::value;
-    const FastPart X = a.x[L1];
-    if (X.ptr != nullptr) {
+    if (a.x[L1].ptr != nullptr) {
       float2 xv[2 * L1 + 1], ax[2 * L1 + 1];
-      load_rows<L1>(xv, X, q);
+      load_rows<L1>(xv, cell_row0(a.x[L1], q.cell), row_step(a.x[L1]), q);
 #pragma unroll
       for (int m1 = 0; m1 <= 2 * L1; m1++) ax[m1] = make_float2(0.f, 0.f);
       static_for<kNP>([&](auto l2c) __attribute__((always_inline)) {
         constexpr int L2 = decltype(l2c)::value;
-        const FastPart Y = a.y[L2];
-        if (Y.ptr != nullptr) {
+        if (a.y[L2].ptr != nullptr) {
           float2 yv[2 * L2 + 1];
-          load_rows<L2>(yv, Y, q);
+          load_rows<L2>(yv, cell_row0(a.y[L2], q.cell), row_step(a.y[L2]), q);
           bwd_pair<L1, L2, LCAP>(a, xv, yv, ax, yimg, q);
         }
       });
-      store_rows<L1>(ax, 1, a.xg[L1], q, accumulate);
+      const FastPart XG = a.xg[L1];
+      store_rows<L1>(ax, 1, cell_row0(XG, q.cell), row_step(XG), q, accumulate);
     }
   });
   static_for<kNP>([&](auto l2c) __attribute__((always_inline)) {
     constexpr int L2 = decltype(l2c)::value;
     const FastPart YG = a.yg[L2];
-    if (YG.ptr != nullptr) store_rows<L2>(yimg + (L2 * L2) * 64 + lane, 64, YG, q, accumulate);
+    if (YG.ptr != nullptr)
+      store_rows<L2>(yimg + (L2 * L2) * 64 + lane, 64, cell_row0(YG, q.cell), row_step(YG), q, accumulate);
   });
 }
 

@@ -133,11 +133,12 @@ __device__ __forceinline__ void fwd_pair(const Diag6Args &a, const float2 (&xv)[
   }
 }
 
+// The four waves of a block work on the same cell and channel group and take every fourth pair: pairs that follow
+// each other write neighbouring 512-byte blocks of the same product rows, so the rows fill in 2 KB at a time.
 template <int LCAP>
 __global__ void __launch_bounds__(256) diag6_fwd_kernel(const Diag6Args a) {
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const long long w = (long long)blockIdx.x * 4 + wave;
-  if (w >= a.nwaves) return;
+  const long long w = blockIdx.x;
   const WavePos q = wave_pos(a, w);
   static_for<kNP>([&](auto l1c) __attribute__((always_inline)) {
     constexpr int L1 = decltype(l1c)::value;
@@ -146,7 +147,7 @@ __global__ void __launch_bounds__(256) diag6_fwd_kernel(const Diag6Args a) {
       load_rows<L1>(xv, cell_row0(a.x[L1], q.cell), row_step(a.x[L1]), q);
       static_for<kNP>([&](auto l2c) __attribute__((always_inline)) {
         constexpr int L2 = decltype(l2c)::value;
-        if (a.y[L2].ptr != nullptr) {
+        if (((L1 * kNP + L2) & 3) == wave && a.y[L2].ptr != nullptr) {
           float2 yv[2 * L2 + 1];
           load_rows<L2>(yv, cell_row0(a.y[L2], q.cell), row_step(a.y[L2]), q);
           fwd_pair<L1, L2, LCAP>(a, xv, yv, q);
@@ -229,7 +230,6 @@ __device__ __forceinline__ void bwd_pair(const Diag6Args &a, const float2 (&xv)[
         ay[m2 + L2].x = fmaf(qi, xc.y, ay[m2 + L2].x);
         ay[m2 + L2].y = fmaf(qi, xc.x, ay[m2 + L2].y);
         ay[m2 + L2].y = fmaf(-qr, xc.y, ay[m2 + L2].y);
-        __builtin_amdgcn_sched_barrier(0);
       });
       __builtin_amdgcn_sched_barrier(0);
     });
@@ -295,8 +295,7 @@ __global__ void __launch_bounds__(64) diag6_bwd_kernel(const Diag6Args a) {
 
 template <int LCAP>
 int launch_diag6_fwd_variant(const Diag6Args &a, hipStream_t s) {
-  const unsigned nblocks = (unsigned)((a.nwaves + 3) / 4);
-  hipLaunchKernelGGL((diag6_fwd_kernel<LCAP>), dim3(nblocks), dim3(256), 0, s, a);
+  hipLaunchKernelGGL((diag6_fwd_kernel<LCAP>), dim3((unsigned)a.nwaves), dim3(256), 0, s, a);
   GELIB_HIP_TRY(hipGetLastError());
   return GELIB_HIP_OK;
 }

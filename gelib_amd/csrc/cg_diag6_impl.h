@@ -257,38 +257,68 @@ __device__ __forceinline__ void store_rows(const float2 *v, int vstride, RowPtr 
   }
 }
 
+// Which of the four waves of a block owns the pairs with this l2: {6}, {5,0}, {4,1}, {3,2} -- 13, 12, 12 and 12 rows
+// of y, so the waves finish every l1 at about the same time.
+constexpr int owner_of(int l2) { return l2 == 6 ? 0 : (l2 == 5 || l2 == 0) ? 1 : (l2 == 4 || l2 == 1) ? 2 : 3; }
+
+// The four waves of a block share one cell and channel group.  Each owns the pairs of its l2 set, so its rows of the
+// y-gradient image are its own (plain read-add-write).  The x-gradient of part l1 gets a partial sum from every
+// wave; the partials meet in LDS after the last pair of l1, are added in the order of the waves and written out, the
+// rows dealt round-robin to the waves.  Pairs (l1, l2) and (l1, l2 +- 1) read neighbouring 512-byte blocks of the same
+// rows of g, and they are in flight at about the same time.
 template <int LCAP>
-__global__ void __launch_bounds__(64) diag6_bwd_kernel(const Diag6Args a) {
+__global__ void __launch_bounds__(256) diag6_bwd_kernel(const Diag6Args a) {
+  constexpr int kXRows = 2 * kL6 + 1;
   __shared__ float2 yimg[kImgRows * 64];
+  __shared__ float2 xpart[4 * kXRows * 64];  // [wave][row][lane]
   const long long w = blockIdx.x;
   const WavePos q = wave_pos(a, w);
-  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const bool accumulate = a.accumulate != 0;
-#pragma unroll
-  for (int r = 0; r < kImgRows; r++) yimg[r * 64 + lane] = make_float2(0.f, 0.f);
+  for (int e = threadIdx.x; e < kImgRows * 64; e += 256) yimg[e] = make_float2(0.f, 0.f);
+  __syncthreads();
   static_for<kNP>([&](auto l1c) __attribute__((always_inline)) {
     constexpr int L1 = decltype(l1c)::value;
-    if (a.x[L1].ptr != nullptr) {
+    if (a.x[L1].ptr != nullptr) {  // the same for the whole block
       float2 xv[2 * L1 + 1], ax[2 * L1 + 1];
       load_rows<L1>(xv, cell_row0(a.x[L1], q.cell), row_step(a.x[L1]), q);
 #pragma unroll
       for (int m1 = 0; m1 <= 2 * L1; m1++) ax[m1] = make_float2(0.f, 0.f);
       static_for<kNP>([&](auto l2c) __attribute__((always_inline)) {
-        constexpr int L2 = decltype(l2c)::value;
-        if (a.y[L2].ptr != nullptr) {
+        constexpr int L2 = kL6 - decltype(l2c)::value;  // descending, so that neighbours in l2 run at the same time
+        if (owner_of(L2) == wave && a.y[L2].ptr != nullptr) {
           float2 yv[2 * L2 + 1];
           load_rows<L2>(yv, cell_row0(a.y[L2], q.cell), row_step(a.y[L2]), q);
           bwd_pair<L1, L2, LCAP>(a, xv, yv, ax, yimg, q);
         }
       });
+      float2 *mine = xpart + wave * kXRows * 64 + lane;
+#pragma unroll
+      for (int m1 = 0; m1 <= 2 * L1; m1++) mine[m1 * 64] = ax[m1];
+      __syncthreads();
       const FastPart XG = a.xg[L1];
-      store_rows<L1>(ax, 1, cell_row0(XG, q.cell), row_step(XG), q, accumulate);
+      RowPtr row0 = cell_row0(XG, q.cell);
+      const long long step = row_step(XG);
+      static_for<2 * L1 + 1>([&](auto rc) __attribute__((always_inline)) {
+        constexpr int r = decltype(rc)::value;
+        if ((r & 3) == wave && q.live) {
+          float2 t = xpart[(0 * kXRows + r) * 64 + lane];
+#pragma unroll
+          for (int k = 1; k < 4; k++) {
+            const float2 u = xpart[(k * kXRows + r) * 64 + lane];
+            t.x += u.x;
+            t.y += u.y;
+          }
+          row_store(row0 + r * step, q.lane_off, t, accumulate);
+        }
+      });
+      __syncthreads();
     }
   });
   static_for<kNP>([&](auto l2c) __attribute__((always_inline)) {
     constexpr int L2 = decltype(l2c)::value;
     const FastPart YG = a.yg[L2];
-    if (YG.ptr != nullptr)
+    if (owner_of(L2) == wave && YG.ptr != nullptr)
       store_rows<L2>(yimg + (L2 * L2) * 64 + lane, 64, cell_row0(YG, q.cell), row_step(YG), q, accumulate);
   });
 }
@@ -302,7 +332,7 @@ int launch_diag6_fwd_variant(const Diag6Args &a, hipStream_t s) {
 
 template <int LCAP>
 int launch_diag6_bwd_variant(const Diag6Args &a, hipStream_t s) {
-  hipLaunchKernelGGL((diag6_bwd_kernel<LCAP>), dim3((unsigned)a.nwaves), dim3(64), 0, s, a);
+  hipLaunchKernelGGL((diag6_bwd_kernel<LCAP>), dim3((unsigned)a.nwaves), dim3(256), 0, s, a);
   GELIB_HIP_TRY(hipGetLastError());
   return GELIB_HIP_OK;
 }

@@ -24,8 +24,8 @@ HBM_PEAK = 8.0e12  # B/s, MI355X HBM3E
 # counter reads for a plain 1 GiB copy: x2.000 and x1.000); summary in profiles/.
 MEASURED_TRAFFIC = {
     "so3vec_cg_L4_tau16_B32768_maxl4": {"so3vec_fwd": 27148781681, "so3vec_bwd": 25959930442},
-    # the backward pass of this type runs as two launches (one per gradient), each reading g: 1.88 x algorithmic
-    "so3vec_diagcg_L6_n64_B131072": {"so3vec_fwd": 102052404553, "so3vec_bwd": 204010468818},
+    # x and y are re-read by the waves that share a cell (mostly from the memory-side cache): 1.25 / 1.23 x algorithmic
+    "so3vec_diagcg_L6_n64_B131072": {"so3vec_fwd": 127684806967, "so3vec_bwd": 133009610533},
     "so3part_cg_10x10_all_l_n8_B16384": {"so3vec_fwd": 3747009028, "so3vec_bwd": 3809547747},
 }
 

@@ -275,16 +275,17 @@ int vec_fwd_entry(bool diag, int nr, const gelib_part_desc *r, int nx, const gel
     for (auto &v : X) xd.push_back(v.d);
     for (auto &v : Y) yd.push_back(v.d);
     int used = 0;
-    rc = unrolled_vec_fwd(plan, rd, xd, yd, accumulate != 0, s, &used);
-    if (rc) return rc;
-    if (used) {
-      t_last_path = kPathUnrolled;
-      return GELIB_HIP_OK;
-    }
+    // Diag products with more than 32 channels: one lane per channel beats the lane-per-channel-pair kernels
     rc = diag6_vec_fwd(plan, rd, xd, yd, accumulate != 0, s, &used);
     if (rc) return rc;
     if (used) {
       t_last_path = kPathDiag6;
+      return GELIB_HIP_OK;
+    }
+    rc = unrolled_vec_fwd(plan, rd, xd, yd, accumulate != 0, s, &used);
+    if (rc) return rc;
+    if (used) {
+      t_last_path = kPathUnrolled;
       return GELIB_HIP_OK;
     }
     rc = staged_vec_fwd(plan, rd, xd, yd, accumulate != 0, s, &used);
@@ -343,16 +344,16 @@ int vec_bwd_entry(bool diag, const gelib_part_desc *xg, const gelib_part_desc *y
     for (auto &v : XG) xgd.push_back(v.d);
     for (auto &v : YG) ygd.push_back(v.d);
     int used = 0;
-    rc = unrolled_vec_bwd(plan, gd, xd, yd, xgd, ygd, accumulate != 0, s, &used);
-    if (rc) return rc;
-    if (used) {
-      t_last_path = kPathUnrolled;
-      return GELIB_HIP_OK;
-    }
     rc = diag6_vec_bwd(plan, gd, xd, yd, xgd, ygd, accumulate != 0, s, &used);
     if (rc) return rc;
     if (used) {
       t_last_path = kPathDiag6;
+      return GELIB_HIP_OK;
+    }
+    rc = unrolled_vec_bwd(plan, gd, xd, yd, xgd, ygd, accumulate != 0, s, &used);
+    if (rc) return rc;
+    if (used) {
+      t_last_path = kPathUnrolled;
       return GELIB_HIP_OK;
     }
     rc = staged_vec_bwd(plan, gd, xd, yd, xgd, ygd, accumulate != 0, s, &used);

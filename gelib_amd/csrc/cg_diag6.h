@@ -42,8 +42,10 @@ struct Diag6Args {
   FastPart r[kNR];                            // product (forward) or its gradient (backward), by l
   const int *offs;    // device, [kNP][kNP][kNR]: first channel of the triple's block in part l, -1 = no such triple
   const float *bank;  // device, kBankFloats coefficients followed by kZeroFloats zeros
-  long long nwaves;   // cells * groups
-  int groups;         // 64-channel groups per cell
+  long long nwaves;   // cells * groups, or cells / (64 >> lg_npad) rounded up
+  long long ncells;
+  int groups;         // 64-channel groups per cell (more than 32 channels)
+  int lg_npad;        // log2 of the channel count rounded up to a power of two, at most 6
   int n;              // channels of every part
   int offs_add;
   int accumulate;
@@ -51,5 +53,7 @@ struct Diag6Args {
 
 int launch_diag6_fwd_l6(const Diag6Args &a, hipStream_t s);  // product l up to 6
 int launch_diag6_bwd_l6(const Diag6Args &a, hipStream_t s);
+int launch_diag6_fwd_l6_packed(const Diag6Args &a, hipStream_t s);  // several cells per wave (lg_npad < 6)
+int launch_diag6_bwd_l6_packed(const Diag6Args &a, hipStream_t s);
 
 }  // namespace gelib_hip

@@ -51,36 +51,59 @@ __device__ __forceinline__ void row_store(RowPtr row, unsigned lane_off, float2 
   *(GlobalOut)(row + lane_off) = o;
 }
 
+// A wave covers 64 channels of one cell, or -- when a part has 32 channels or fewer -- all channels of 64 / n_pad
+// consecutive cells (n_pad = the channel count rounded up to a power of two).  `cell` is the first cell of the wave and
+// uniform; `cell_local` and `ch` are the lane's own.
 struct WavePos {
   long long cell;
-  unsigned lane_off;  // byte offset of the lane's channel in a row (a valid channel also for lanes beyond n)
+  int cell_local;
+  int ch;     // a valid channel of a valid cell also for lanes that have nothing to do (they never store)
   bool live;
 };
 
 __device__ __forceinline__ WavePos wave_pos(const Diag6Args &a, long long w) {
   WavePos q;
-  q.cell = w / a.groups;
-  const int grp = (int)(w - q.cell * a.groups);
-  const int ch = grp * 64 + (int)(threadIdx.x & 63);
-  q.live = ch < a.n;
-  q.lane_off = q.live ? (unsigned)ch * 8u : 0u;
+  const int lane = (int)(threadIdx.x & 63);
+  if (a.lg_npad < 6) {
+    q.cell = w << (6 - a.lg_npad);
+    q.cell_local = lane >> a.lg_npad;
+    q.ch = lane & ((1 << a.lg_npad) - 1);
+    q.live = q.ch < a.n && q.cell + q.cell_local < a.ncells;
+  } else {
+    q.cell = w / a.groups;
+    q.cell_local = 0;
+    q.ch = (int)(w - q.cell * a.groups) * 64 + lane;
+    q.live = q.ch < a.n;
+  }
+  if (!q.live) q.cell_local = 0, q.ch = 0;
   return q;
+}
+
+// Byte offset of the lane's element from row 0 of the wave's first cell; 32 bits (the host checks the range).
+// PACKED: several cells per wave, so the offset depends on the part's cell stride; otherwise it is the channel alone.
+template <bool PACKED>
+__device__ __forceinline__ unsigned lane_offset(const FastPart P, const WavePos q) {
+  if constexpr (PACKED) return ((unsigned)q.cell_local * (unsigned)P.sb + (unsigned)q.ch) * 8u;
+  else return (unsigned)q.ch * 8u;
 }
 
 // Row 0 of a part in the wave's cell, and the distance between its rows in bytes.
 __device__ __forceinline__ RowPtr cell_row0(const FastPart P, long long cell) { return (RowPtr)P.ptr + cell * P.sb * 8; }
 __device__ __forceinline__ long long row_step(const FastPart P) { return (long long)P.sm * 8; }
 
-template <int L>
-__device__ __forceinline__ void load_rows(float2 (&v)[2 * L + 1], RowPtr row, long long step, const WavePos q) {
+template <int L, bool PACKED>
+__device__ __forceinline__ void load_rows(float2 (&v)[2 * L + 1], const FastPart P, const WavePos q) {
+  RowPtr row = cell_row0(P, q.cell);
+  const long long step = row_step(P);
+  const unsigned lo = lane_offset<PACKED>(P, q);
 #pragma unroll
   for (int m = 0; m <= 2 * L; m++) {
-    v[m] = row_load(row, q.lane_off);
+    v[m] = row_load(row, lo);
     row += step;
   }
 }
 
-template <int L1, int L2, int LCAP>
+template <int L1, int L2, int LCAP, bool PACKED>
 __device__ __forceinline__ void fwd_pair(const Diag6Args &a, const float2 (&xv)[2 * L1 + 1],
                                          const float2 (&yv)[2 * L2 + 1], const WavePos q) {
   constexpr int LMIN = iabs(L1 - L2);
@@ -92,12 +115,14 @@ __device__ __forceinline__ void fwd_pair(const Diag6Args &a, const float2 (&xv)[
     const bool accumulate = a.accumulate != 0;
     // the row of part l that the next m of that part is stored to; a triple that is not there is never stored
     RowPtr row[NL];
+    unsigned lo[NL];
     bool present[NL];
     static_for<NL>([&](auto dc) __attribute__((always_inline)) {
       constexpr int dl = decltype(dc)::value;
       const int off = offs[LMIN + dl];
       present[dl] = off >= 0;
       row[dl] = cell_row0(a.r[LMIN + dl], q.cell) + (long long)(off + a.offs_add) * 8;
+      lo[dl] = lane_offset<PACKED>(a.r[LMIN + dl], q);
     });
     static_for<2 * LTOP + 1>([&](auto mc) __attribute__((always_inline)) {
       constexpr int m = decltype(mc)::value - LTOP;
@@ -125,7 +150,7 @@ __device__ __forceinline__ void fwd_pair(const Diag6Args &a, const float2 (&xv)[
         constexpr int dl = decltype(dc)::value;
         constexpr int L = LMIN + dl;
         if constexpr (L >= MABS) {
-          if (present[dl] && q.live) row_store(row[dl], q.lane_off, acc[dl], accumulate);
+          if (present[dl] && q.live) row_store(row[dl], lo[dl], acc[dl], accumulate);
           row[dl] += row_step(a.r[L]);
         }
       });
@@ -135,7 +160,7 @@ __device__ __forceinline__ void fwd_pair(const Diag6Args &a, const float2 (&xv)[
 
 // The four waves of a block work on the same cell and channel group and take every fourth pair: pairs that follow
 // each other write neighbouring 512-byte blocks of the same product rows, so the rows fill in 2 KB at a time.
-template <int LCAP>
+template <int LCAP, bool PACKED>
 __global__ void __launch_bounds__(256) diag6_fwd_kernel(const Diag6Args a) {
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const long long w = blockIdx.x;
@@ -144,13 +169,13 @@ __global__ void __launch_bounds__(256) diag6_fwd_kernel(const Diag6Args a) {
     constexpr int L1 = decltype(l1c)::value;
     if (a.x[L1].ptr != nullptr) {
       float2 xv[2 * L1 + 1];
-      load_rows<L1>(xv, cell_row0(a.x[L1], q.cell), row_step(a.x[L1]), q);
+      load_rows<L1, PACKED>(xv, a.x[L1], q);
       static_for<kNP>([&](auto l2c) __attribute__((always_inline)) {
         constexpr int L2 = decltype(l2c)::value;
         if (((L1 * kNP + L2) & 3) == wave && a.y[L2].ptr != nullptr) {
           float2 yv[2 * L2 + 1];
-          load_rows<L2>(yv, cell_row0(a.y[L2], q.cell), row_step(a.y[L2]), q);
-          fwd_pair<L1, L2, LCAP>(a, xv, yv, q);
+          load_rows<L2, PACKED>(yv, a.y[L2], q);
+          fwd_pair<L1, L2, LCAP, PACKED>(a, xv, yv, q);
         }
       });
     }
@@ -158,7 +183,7 @@ __global__ void __launch_bounds__(256) diag6_fwd_kernel(const Diag6Args a) {
 }
 
 // One pair of the backward pass: every l of the pair together, one row number m = m1 + m2 at a time.
-template <int L1, int L2, int LCAP>
+template <int L1, int L2, int LCAP, bool PACKED>
 __device__ __forceinline__ void bwd_pair(const Diag6Args &a, const float2 (&xv)[2 * L1 + 1],
                                          const float2 (&yv)[2 * L2 + 1], float2 (&ax)[2 * L1 + 1], float2 *yimg,
                                          const WavePos q) {
@@ -174,6 +199,7 @@ __device__ __forceinline__ void bwd_pair(const Diag6Args &a, const float2 (&xv)[
     // no branches; row[dl] is the row of part l that the next m of that part is read from
     RowPtr row[NL];
     long long step[NL];
+    unsigned lo[NL];
     static_for<NL>([&](auto dc) __attribute__((always_inline)) {
       constexpr int dl = decltype(dc)::value;
       constexpr int L = LMIN + dl;
@@ -181,6 +207,7 @@ __device__ __forceinline__ void bwd_pair(const Diag6Args &a, const float2 (&xv)[
       const bool present = off >= 0;
       row[dl] = present ? cell_row0(a.r[L], q.cell) + (long long)(off + a.offs_add) * 8 : (RowPtr)(a.bank + kBankFloats);
       step[dl] = present ? row_step(a.r[L]) : 0;
+      lo[dl] = present ? lane_offset<PACKED>(a.r[L], q) : (unsigned)q.ch * 8u;
     });
     float2 ay[2 * L2 + 1];
 #pragma unroll
@@ -190,7 +217,7 @@ __device__ __forceinline__ void bwd_pair(const Diag6Args &a, const float2 (&xv)[
       static_for<NL>([&](auto dc) __attribute__((always_inline)) {
         constexpr int dl = decltype(dc)::value;
         if constexpr (LMIN + dl >= iabs(m)) {
-          dst[dl] = row_load(row[dl], q.lane_off);
+          dst[dl] = row_load(row[dl], lo[dl]);
           row[dl] += step[dl];
         }
       });
@@ -246,13 +273,15 @@ __device__ __forceinline__ void bwd_pair(const Diag6Args &a, const float2 (&xv)[
   }
 }
 
-template <int L>
-__device__ __forceinline__ void store_rows(const float2 *v, int vstride, RowPtr row, long long step, const WavePos q,
-                                           bool accumulate) {
+template <int L, bool PACKED>
+__device__ __forceinline__ void store_rows(const float2 *v, int vstride, const FastPart P, const WavePos q, bool accumulate) {
   if (!q.live) return;
+  RowPtr row = cell_row0(P, q.cell);
+  const long long step = row_step(P);
+  const unsigned lo = lane_offset<PACKED>(P, q);
 #pragma unroll
   for (int m = 0; m <= 2 * L; m++) {
-    row_store(row, q.lane_off, v[m * vstride], accumulate);
+    row_store(row, lo, v[m * vstride], accumulate);
     row += step;
   }
 }
@@ -266,8 +295,10 @@ constexpr int owner_of(int l2) { return l2 == 6 ? 0 : (l2 == 5 || l2 == 0) ? 1 :
 // wave; the partials meet in LDS after the last pair of l1, are added in the order of the waves and written out, the
 // rows dealt round-robin to the waves.  Pairs (l1, l2) and (l1, l2 +- 1) read neighbouring 512-byte blocks of the same
 // rows of g, and they are in flight at about the same time.
-template <int LCAP>
-__global__ void __launch_bounds__(256) diag6_bwd_kernel(const Diag6Args a) {
+// Three waves per SIMD (168 registers) is what the LDS of a block lets a compute unit hold.  The one-cell form fits by
+// itself; the packed form is one register over and is capped (capping the other one too changes its schedule for the worse).
+template <int LCAP, bool PACKED>
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(PACKED ? 3 : 1))) diag6_bwd_kernel(const Diag6Args a) {
   constexpr int kXRows = 2 * kL6 + 1;
   __shared__ float2 yimg[kImgRows * 64];
   __shared__ float2 xpart[4 * kXRows * 64];  // [wave][row][lane]
@@ -281,15 +312,15 @@ __global__ void __launch_bounds__(256) diag6_bwd_kernel(const Diag6Args a) {
     constexpr int L1 = decltype(l1c)::value;
     if (a.x[L1].ptr != nullptr) {  // the same for the whole block
       float2 xv[2 * L1 + 1], ax[2 * L1 + 1];
-      load_rows<L1>(xv, cell_row0(a.x[L1], q.cell), row_step(a.x[L1]), q);
+      load_rows<L1, PACKED>(xv, a.x[L1], q);
 #pragma unroll
       for (int m1 = 0; m1 <= 2 * L1; m1++) ax[m1] = make_float2(0.f, 0.f);
       static_for<kNP>([&](auto l2c) __attribute__((always_inline)) {
         constexpr int L2 = kL6 - decltype(l2c)::value;  // descending, so that neighbours in l2 run at the same time
         if (owner_of(L2) == wave && a.y[L2].ptr != nullptr) {
           float2 yv[2 * L2 + 1];
-          load_rows<L2>(yv, cell_row0(a.y[L2], q.cell), row_step(a.y[L2]), q);
-          bwd_pair<L1, L2, LCAP>(a, xv, yv, ax, yimg, q);
+          load_rows<L2, PACKED>(yv, a.y[L2], q);
+          bwd_pair<L1, L2, LCAP, PACKED>(a, xv, yv, ax, yimg, q);
         }
       });
       float2 *mine = xpart + wave * kXRows * 64 + lane;
@@ -299,6 +330,7 @@ __global__ void __launch_bounds__(256) diag6_bwd_kernel(const Diag6Args a) {
       const FastPart XG = a.xg[L1];
       RowPtr row0 = cell_row0(XG, q.cell);
       const long long step = row_step(XG);
+      const unsigned xlo = lane_offset<PACKED>(XG, q);
       static_for<2 * L1 + 1>([&](auto rc) __attribute__((always_inline)) {
         constexpr int r = decltype(rc)::value;
         if ((r & 3) == wave && q.live) {
@@ -309,7 +341,7 @@ __global__ void __launch_bounds__(256) diag6_bwd_kernel(const Diag6Args a) {
             t.x += u.x;
             t.y += u.y;
           }
-          row_store(row0 + r * step, q.lane_off, t, accumulate);
+          row_store(row0 + r * step, xlo, t, accumulate);
         }
       });
       __syncthreads();
@@ -319,20 +351,20 @@ __global__ void __launch_bounds__(256) diag6_bwd_kernel(const Diag6Args a) {
     constexpr int L2 = decltype(l2c)::value;
     const FastPart YG = a.yg[L2];
     if (owner_of(L2) == wave && YG.ptr != nullptr)
-      store_rows<L2>(yimg + (L2 * L2) * 64 + lane, 64, cell_row0(YG, q.cell), row_step(YG), q, accumulate);
+      store_rows<L2, PACKED>(yimg + (L2 * L2) * 64 + lane, 64, YG, q, accumulate);
   });
 }
 
-template <int LCAP>
+template <int LCAP, bool PACKED>
 int launch_diag6_fwd_variant(const Diag6Args &a, hipStream_t s) {
-  hipLaunchKernelGGL((diag6_fwd_kernel<LCAP>), dim3((unsigned)a.nwaves), dim3(256), 0, s, a);
+  hipLaunchKernelGGL((diag6_fwd_kernel<LCAP, PACKED>), dim3((unsigned)a.nwaves), dim3(256), 0, s, a);
   GELIB_HIP_TRY(hipGetLastError());
   return GELIB_HIP_OK;
 }
 
-template <int LCAP>
+template <int LCAP, bool PACKED>
 int launch_diag6_bwd_variant(const Diag6Args &a, hipStream_t s) {
-  hipLaunchKernelGGL((diag6_bwd_kernel<LCAP>), dim3((unsigned)a.nwaves), dim3(256), 0, s, a);
+  hipLaunchKernelGGL((diag6_bwd_kernel<LCAP, PACKED>), dim3((unsigned)a.nwaves), dim3(256), 0, s, a);
   GELIB_HIP_TRY(hipGetLastError());
   return GELIB_HIP_OK;
 }

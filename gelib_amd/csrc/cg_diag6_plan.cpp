@@ -68,7 +68,7 @@ int make_args(const VecPlan &plan, const std::vector<const gelib_part_desc *> &r
   if (xg && !lists_to_fast(*xg, plan.E, true, &fxg, nullptr)) return GELIB_HIP_OK;
   if (yg && !lists_to_fast(*yg, plan.E, true, &fyg, nullptr)) return GELIB_HIP_OK;
   const int n = lx[0].second;
-  if (n <= 32 || n > kMaxChannels) return GELIB_HIP_OK;
+  if (n < 1 || n > kMaxChannels) return GELIB_HIP_OK;
   for (auto &p : lx)
     if (p.first > kL6 || p.second != n) return GELIB_HIP_OK;
   for (auto &p : ly)
@@ -91,9 +91,26 @@ int make_args(const VecPlan &plan, const std::vector<const gelib_part_desc *> &r
   if (rc) return rc;
   if ((rc = device_bank(&a->bank))) return rc;
   const long long ncells = plan.E[0] * plan.E[1] * plan.E[2];
-  a->groups = (n + 63) / 64;
+  a->ncells = ncells;
   a->n = n;
-  a->nwaves = ncells * a->groups;
+  int lg = 0;
+  while ((1 << lg) < n && lg < 6) lg++;
+  a->lg_npad = lg;
+  if (lg < 6) {
+    // several cells per wave: the lane's offset from the wave's first cell must fit 32 bits in every part
+    const long long cpw = 64 >> lg;
+    auto fits = [&](const std::vector<FastPart> &v) {
+      for (auto &p : v)
+        if (p.sb < 0 || ((cpw - 1) * p.sb + n) * 8 >= (1LL << 31)) return false;
+      return true;
+    };
+    if (!fits(fx) || !fits(fy) || !fits(fr) || !fits(fxg) || !fits(fyg)) return GELIB_HIP_OK;
+    a->groups = 1;
+    a->nwaves = (ncells + cpw - 1) / cpw;
+  } else {
+    a->groups = (n + 63) / 64;
+    a->nwaves = ncells * a->groups;
+  }
   if (a->nwaves > 0x7fffffffLL) return GELIB_HIP_OK;
   *ok = true;
   return GELIB_HIP_OK;
@@ -112,7 +129,7 @@ int diag6_vec_fwd(const VecPlan &plan, const std::vector<const gelib_part_desc *
   if (rc || !ok) return rc;
   if (lcap > kL6) return GELIB_HIP_OK;  // kernels are built for products capped at l = 6
   a.accumulate = accumulate ? 1 : 0;
-  if ((rc = launch_diag6_fwd_l6(a, s))) return rc;
+  if ((rc = a.lg_npad < 6 ? launch_diag6_fwd_l6_packed(a, s) : launch_diag6_fwd_l6(a, s))) return rc;
   *used = 1;
   return GELIB_HIP_OK;
 }
@@ -130,7 +147,7 @@ int diag6_vec_bwd(const VecPlan &plan, const std::vector<const gelib_part_desc *
   if (rc || !ok) return rc;
   if (lcap > kL6) return GELIB_HIP_OK;
   a.accumulate = accumulate ? 1 : 0;
-  if ((rc = launch_diag6_bwd_l6(a, s))) return rc;
+  if ((rc = a.lg_npad < 6 ? launch_diag6_bwd_l6_packed(a, s) : launch_diag6_bwd_l6(a, s))) return rc;
   *used = 1;
   return GELIB_HIP_OK;
 }

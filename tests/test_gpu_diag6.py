@@ -35,7 +35,11 @@ CASES = [
     (2, {6: 64}, {6: 64}, 6),                                          # one pair, l from 0 to 6 of 0..12
     (3, {2: 64, 6: 64}, {3: 64, 5: 64}, 4),                            # capped below the largest operand l
     (1, {l: 200 for l in range(7)}, {l: 200 for l in range(7)}, 6),    # four groups, one cell
-    (70, {5: 33}, {4: 33}, 6),                                         # the smallest channel count the family takes
+    (70, {5: 33}, {4: 33}, 6),                                         # 33 channels: one group, 31 lanes idle
+    (37, {l: 16 for l in range(5)}, {l: 16 for l in range(5)}, 4),     # four cells per wave, the last wave one cell
+    (130, {0: 1, 3: 1}, {2: 1, 3: 1}, 6),                              # one channel: 64 cells per wave
+    (9, {l: 24 for l in range(7)}, {l: 24 for l in range(7)}, 6),      # two cells per wave, 8 lanes of each idle
+    (5, {1: 32, 6: 32}, {6: 32}, 5),                                   # exactly half a wave per cell
 ]
 
 
@@ -79,7 +83,7 @@ def test_diag6_vec(cabi, B, tx, ty, maxl):
 
 
 def test_diag6_declines_what_it_cannot_do(cabi):
-    # a broadcast operand whose gradient is wanted, a product above l = 6, 32 channels or fewer: other families run
+    # a broadcast operand whose gradient is wanted, a product above l = 6: other families run
     x = [U.dev(U.seeded(1, 1, 13, 64))]
     y = [U.dev(U.seeded(2, 4, 13, 64))]
     r = [torch.zeros(4, 2 * l + 1, 64, dtype=torch.complex64, device="cuda") for l in range(13)]
@@ -96,7 +100,12 @@ def test_diag6_declines_what_it_cannot_do(cabi):
     xg, yg = [torch.zeros_like(x[0])], [torch.zeros_like(y[0])]
     cabi.so3vec_bwd(xg, yg, r6, x, y, accumulate=False, diag=True)
     assert cabi.last_path() != DIAG6          # its gradient needs a sum over the batch
-    x32 = [U.dev(U.seeded(3, 2, 11, 32))]
-    r32 = [torch.zeros(2, 2 * l + 1, 32, dtype=torch.complex64, device="cuda") for l in range(7)]
-    cabi.so3vec_fwd(r32, x32, x32, accumulate=False, diag=True)
-    assert cabi.last_path() != DIAG6
+    # a broadcast operand with several cells per wave
+    x8 = [U.dev(U.seeded(3, 1, 11, 8))]
+    y8 = [U.dev(U.seeded(4, 21, 11, 8))]
+    r8 = [torch.zeros(21, 2 * l + 1, 8, dtype=torch.complex64, device="cuda") for l in range(7)]
+    cabi.so3vec_fwd(r8, x8, y8, accumulate=False, diag=True)
+    assert cabi.last_path() == DIAG6
+    want8 = ora.vec_fwd([U.host(x8[0])], [U.host(y8[0])], 6, True)
+    for a, b in zip(r8, want8):
+        assert U.gate_excess(U.host(a), b) <= 1.0

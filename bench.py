@@ -282,14 +282,14 @@ def main():
         "config": {"workload": name, "batch": B, "tau_x": {str(k): v for k, v in tx.items()},
                    "tau_y": {str(k): v for k, v in ty.items()}, "maxl": maxl, "diag": diag,
                    "triples": sum(1 for l1 in tx for l2 in ty for l in range(abs(l1 - l2), l1 + l2 + 1) if l in tr),
-                   "kernel_path": {1: "generic", 2: "unrolled", 3: "staged", 4: "diag6"}.get(path, str(path)),
+                   "kernel_path": {1: "generic", 2: "unrolled", 3: "staged", 4: "diag6", 5: "onepair"}.get(path, str(path)),
                    "fwd_ms": fwd_ms, "bwd_ms": bwd_ms,
                    "fwd_GBps": fwd_bytes / (fwd_ms * 1e-3) / 1e9, "bwd_GBps": bwd_bytes / (bwd_ms * 1e-3) / 1e9,
                    "fwd_bwd_GBps": (fwd_bytes + bwd_bytes) / ((fwd_ms + bwd_ms) * 1e-3) / 1e9,
                    "fwd_bwd_frac_of_peak": (fwd_bytes + bwd_bytes) / ((fwd_ms + bwd_ms) * 1e-3) / HBM_PEAK},
         "roofline": {"bound": "hbm", "kernel": dom, "achieved": achieved, "peak": HBM_PEAK / 1e9, "unit": "GB/s",
                      "frac": achieved * 1e9 / HBM_PEAK,
-                     "traffic": MEASURED_TRAFFIC.get(name, {}).get(dom) if B == WORKLOADS[name][1] and path in (2, 3, 4) else None,
+                     "traffic": MEASURED_TRAFFIC.get(name, {}).get(dom) if B == WORKLOADS[name][1] and path in (2, 3, 4, 5) else None,
                      "algorithmic_bytes_per_launch": dom_bytes},
     }
     if not args.no_cpu:

@@ -356,6 +356,12 @@ int vec_bwd_entry(bool diag, const gelib_part_desc *xg, const gelib_part_desc *y
       t_last_path = kPathUnrolled;
       return GELIB_HIP_OK;
     }
+    rc = onepair_vec_bwd(plan, gd, xd, yd, xgd, ygd, accumulate != 0, s, &used);
+    if (rc) return rc;
+    if (used) {
+      t_last_path = kPathOnePair;
+      return GELIB_HIP_OK;
+    }
     rc = staged_vec_bwd(plan, gd, xd, yd, xgd, ygd, accumulate != 0, s, &used);
     if (rc) return rc;
     if (used) {
@@ -647,6 +653,7 @@ int gelib_hip_set_option(const char *name, int value) {
   }
   if (!std::strncmp(name, "staged_", 7)) return staged_set_option(name, value);
   if (!std::strncmp(name, "diag6", 5)) return diag6_set_option(name, value);
+  if (!std::strncmp(name, "onepair", 7)) return onepair_set_option(name, value);
   return unrolled_set_option(name, value);
 }
 

@@ -79,4 +79,11 @@ int staged_vec_bwd(const VecPlan &plan, const std::vector<const gelib_part_desc 
                    bool accumulate, hipStream_t s, int *used);
 int staged_set_option(const char *name, int value);
 
+// Backward pass of a product of ONE x part with ONE y part, any l with l1 + l2 <= 21 (cg_onepair.hip).
+int onepair_vec_bwd(const VecPlan &plan, const std::vector<const gelib_part_desc *> &g,
+                    const std::vector<const gelib_part_desc *> &x, const std::vector<const gelib_part_desc *> &y,
+                    const std::vector<const gelib_part_desc *> &xg, const std::vector<const gelib_part_desc *> &yg,
+                    bool accumulate, hipStream_t s, int *used);
+int onepair_set_option(const char *name, int value);
+
 }  // namespace gelib_hip

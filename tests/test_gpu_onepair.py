@@ -1,0 +1,83 @@
+"""GPU parity of the backward kernel for products of ONE x part with ONE y part of large l (l1 + l2 <= 21, at most 64
+channel slots per cell): gelib_hip_last_path() == 5, gradients against the CPU oracle in float32 and float64."""
+import numpy as np
+import pytest
+
+from oracle import cg_oracle as ora
+from tests import gpu_util as U
+
+pytestmark = pytest.mark.gpu
+
+torch = pytest.importorskip("torch")
+
+ONEPAIR = 5
+
+
+@pytest.fixture(scope="module")
+def cabi():
+    assert torch.cuda.is_available(), "GPU tests need a GPU"
+    from gelib_amd import cabi as c
+    c.lib()
+    c.set_option("force_generic", 0)
+    c.set_option("onepair", 1)
+    return c
+
+
+def c128(L):
+    return [a.astype(np.complex128) for a in L]
+
+
+CASES = [
+    # (B, l1, n1, l2, n2, maxl, diag)
+    (9, 10, 8, 10, 8, -1, False),    # the benchmark pair: 64 slots, every l from 0 to 20
+    (7, 5, 3, 6, 5, -1, False),      # 3 x 5 channels padded to 4 x 8 slots, two cells per wave, odd batch
+    (5, 10, 2, 11, 4, -1, False),    # l1 + l2 = 21: 44 rows of sums, 21 values of l starting at 1
+    (6, 8, 8, 8, 8, 9, False),       # product capped below l1 + l2
+    (11, 7, 20, 7, 20, -1, True),    # Diag, 20 channels padded to 32: two cells per wave
+    (3, 9, 64, 6, 64, -1, True),     # Diag, a full wave per cell
+    (70, 6, 1, 5, 1, -1, False),     # one channel pair: 64 cells per wave
+]
+
+
+@pytest.mark.parametrize("B,l1,n1,l2,n2,maxl,diag", CASES)
+def test_onepair_bwd(cabi, B, l1, n1, l2, n2, maxl, diag):
+    seed = 1300 + B
+    xs = [U.seeded(seed, B, 2 * l1 + 1, n1)]
+    ys = [U.seeded(seed + 1, B, 2 * l2 + 1, n2)]
+    r32 = ora.vec_fwd(xs, ys, maxl, diag)
+    gs = [U.seeded(seed + 100 + i, *p.shape) for i, p in enumerate(r32)]
+    xg32, yg32 = ora.vec_bwd(gs, xs, ys, diag)
+    xg64, yg64 = ora.vec_bwd(c128(gs), c128(xs), c128(ys), diag)
+    dxs, dys, dgs = [U.dev(a) for a in xs], [U.dev(a) for a in ys], [U.dev(a) for a in gs]
+    dxg = [torch.full(a.shape, 3.0 - 2j, dtype=torch.complex64, device="cuda") for a in xs]
+    dyg = [torch.full(a.shape, 3.0 - 2j, dtype=torch.complex64, device="cuda") for a in ys]
+    cabi.so3vec_bwd(dxg, dyg, dgs, dxs, dys, accumulate=False, diag=diag)
+    assert cabi.last_path() == ONEPAIR
+    torch.cuda.synchronize()
+    tag = "B%d (%d,%d)x(%d,%d) maxl %d diag %d" % (B, l1, n1, l2, n2, maxl, diag)
+    U.assert_parity(U.host(dxg[0]), xg32[0], xg64[0], "xg " + tag, slack=4.0)
+    U.assert_parity(U.host(dyg[0]), yg32[0], yg64[0], "yg " + tag, slack=4.0)
+    dxg2, dyg2 = [a.clone() for a in dxg], [a.clone() for a in dyg]
+    cabi.so3vec_bwd(dxg2, dyg2, dgs, dxs, dys, accumulate=True, diag=diag)
+    assert cabi.last_path() == ONEPAIR
+    torch.cuda.synchronize()
+    for a, b in zip(dxg2 + dyg2, dxg + dyg):
+        assert U.gate_excess(U.host(a), 2 * U.host(b), rtol=2e-5, atol=2e-5) <= 1.0
+
+
+def test_onepair_leaves_the_rest_alone(cabi):
+    # one gradient alone, two x parts, l1 + l2 above 21: other kernels
+    x, y = [U.dev(U.seeded(1, 4, 21, 8))], [U.dev(U.seeded(2, 4, 21, 8))]
+    want = ora.vec_fwd([U.host(x[0])], [U.host(y[0])])
+    g = [U.dev(U.seeded(10 + i, *p.shape)) for i, p in enumerate(want)]
+    xg = [torch.zeros_like(x[0])]
+    cabi.so3vec_bwd(xg, None, g, x, y, accumulate=False)
+    assert cabi.last_path() != ONEPAIR
+    wxg, _ = ora.vec_bwd([U.host(t) for t in g], [U.host(x[0])], [U.host(y[0])])
+    assert U.gate_excess(U.host(xg[0]), wxg[0], rtol=1e-4, atol=1e-4) <= 1.0
+    x11, y11 = [U.dev(U.seeded(3, 2, 23, 4))], [U.dev(U.seeded(4, 2, 23, 4))]
+    w11 = ora.vec_fwd([U.host(x11[0])], [U.host(y11[0])], 3)
+    g11 = [U.dev(U.seeded(20 + i, *p.shape)) for i, p in enumerate(w11)]
+    xg11, yg11 = [torch.zeros_like(x11[0])], [torch.zeros_like(y11[0])]
+    cabi.so3vec_bwd(xg11, yg11, g11, x11, y11, accumulate=False)
+    assert cabi.last_path() != ONEPAIR

@@ -27,10 +27,12 @@ def cabi(request):
     c.lib()
     c.set_option("force_generic", 0)
     c.set_option("diag6", 0)   # the lane-per-channel Diag kernels would take some of these cases first
+    c.set_option("onepair", 0) # and the single-pair backward kernel others
     c.set_option("staged_bwd_stripes", 2 if request.param == "striped" else 0)
     c.set_option("staged_bwd_pairs", int(request.param == "pairwise"))
     yield c
     c.set_option("diag6", 1)
+    c.set_option("onepair", 1)
     c.set_option("staged_bwd_threads", 0)
     c.set_option("staged_bwd_stripes", 1)
     c.set_option("staged_bwd_pairs", 0)

@@ -26,7 +26,7 @@ MEASURED_TRAFFIC = {
     "so3vec_cg_L4_tau16_B32768_maxl4": {"so3vec_fwd": 27148781681, "so3vec_bwd": 25959930442},
     # x and y are re-read by the waves that share a cell (mostly from the memory-side cache): 1.25 / 1.23 x algorithmic
     "so3vec_diagcg_L6_n64_B131072": {"so3vec_fwd": 127684806967, "so3vec_bwd": 133009610533},
-    "so3part_cg_10x10_all_l_n8_B16384": {"so3vec_fwd": 3747009028, "so3vec_bwd": 3809547747},
+    "so3part_cg_10x10_all_l_n8_B16384": {"so3vec_fwd": 3747210969, "so3vec_bwd": 3936276724},
 }
 
 WORKLOADS = {

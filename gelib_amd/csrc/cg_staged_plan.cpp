@@ -179,6 +179,9 @@ int get_plan(bool diag, const std::vector<VecTriple> &triples, const std::vector
           n_other = no;
         }
         table[3 * k + 1] = filled - table[3 * k];
+        // a part that no triple feeds has a zero gradient; a stripe without units would leave it unwritten, so such
+        // types go to the kernels that write every part from their images
+        if (table[3 * k + 1] == 0) ok = false;
         // lane slots: channel counts rounded up to powers of two
         const int lgu = diag ? ilog2(std::max(1, n_own)) : ilog2(std::max(1, n_own)) + ilog2(std::max(1, n_other));
         if (lgu > 20) ok = false;

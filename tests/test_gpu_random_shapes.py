@@ -86,3 +86,69 @@ def test_random_product(cabi, seed):
     if dxg is not None:
         for a, b, c in zip(dxg, xg32, xg64):
             U.assert_parity(U.host(a), b, c, "xg " + tag + " path %d" % path, slack=4.0)
+
+
+@pytest.mark.parametrize("seed", range(120))
+def test_random_part_call(cabi, seed):
+    """One part-level entry point per draw: random l, channel counts, channel offset, grid, batch broadcast, views with
+    a channel stride, accumulate or overwrite."""
+    rng = np.random.default_rng(9000 + seed)
+    diag = bool(rng.integers(0, 2))
+    l1, l2 = int(rng.integers(0, 11)), int(rng.integers(0, 11))
+    l = int(rng.integers(abs(l1 - l2), l1 + l2 + 1))
+    n1 = int(rng.choice([1, 2, 3, 4, 7, 8, 16, 33, 64]))
+    n2 = n1 if diag else int(rng.choice([1, 2, 3, 4, 8, 16]))
+    nout = n1 if diag else n1 * n2
+    offs, tail = int(rng.choice([0, 0, 3, 8])), int(rng.choice([0, 5]))
+    B = int(rng.choice([1, 2, 6, 37]))
+    grid = [(), (3,), (2, 2)][int(rng.integers(0, 3))]
+    kind = int(rng.integers(0, 3))              # 0 forward, 1 back0, 2 back1
+    accumulate = bool(rng.integers(0, 2))
+    bcast = int(rng.integers(0, 4)) == 0        # an operand (not the destination) shared by the whole batch
+    stride2 = int(rng.integers(0, 5)) == 0      # the destination is every second channel of a wider tensor
+
+    def lead(b):
+        return (b,) + grid
+
+    xb = 1 if (bcast and kind != 1) else B
+    yb = 1 if (bcast and kind == 1) else B
+    x = U.seeded(seed * 7 + 1, *lead(xb), 2 * l1 + 1, n1)
+    y = U.seeded(seed * 7 + 2, *lead(yb), 2 * l2 + 1, n2)
+    r = U.seeded(seed * 7 + 3, *lead(B), 2 * l + 1, offs + nout + tail)   # product, or the incoming gradient
+    full = lambda a: np.ascontiguousarray(np.broadcast_to(a, lead(B) + a.shape[-2:]))
+    flat = lambda a: a.reshape((-1,) + a.shape[-2:])
+    ops = (ora.DIAG_FWD, ora.DIAG_BACK0, ora.DIAG_BACK1) if diag else (ora.CG_FWD, ora.CG_BACK0, ora.CG_BACK1)
+    fns = ((cabi.so3part_diagcg_fwd, cabi.so3part_diagcg_back0, cabi.so3part_diagcg_back1) if diag else
+           (cabi.so3part_cg_fwd, cabi.so3part_cg_back0, cabi.so3part_cg_back1))
+    dest0 = [r, U.seeded(seed * 7 + 4, *lead(B), 2 * l1 + 1, n1), U.seeded(seed * 7 + 5, *lead(B), 2 * l2 + 1, n2)][kind]
+
+    def reference(prec):
+        c = (lambda a: flat(full(a)).astype(np.complex128)) if prec == 64 else (lambda a: flat(full(a)).copy())
+        d = c(dest0)
+        if not accumulate:
+            if kind == 0:
+                d[..., offs:offs + nout] = 0      # overwrite touches the block of this triple only
+            else:
+                d[...] = 0
+        if kind == 0:
+            ora.part_op(ops[0], d, c(x), c(y), offs)
+        elif kind == 1:
+            ora.part_op(ops[1], c(r), d, c(y), offs)
+        else:
+            ora.part_op(ops[2], c(r), c(x), d, offs)
+        return d
+
+    want32, want64 = reference(32), reference(64)
+    if stride2:
+        wide = torch.zeros(dest0.shape[:-1] + (2 * dest0.shape[-1],), dtype=torch.complex64, device="cuda")
+        dest = wide[..., ::2]
+        dest.copy_(U.dev(dest0))
+    else:
+        dest = U.dev(dest0)
+    dx, dy, dr = U.dev(x), U.dev(y), U.dev(r)
+    args = [(dest, dx, dy), (dest, dr, dy), (dest, dr, dx)][kind]
+    fns[kind](*args, offs=offs, accumulate=accumulate)
+    torch.cuda.synchronize()
+    tag = "seed %d kind %d diag %d (%d,%d)x(%d,%d)->%d offs %d B %d grid %s bcast %d acc %d stride2 %d path %d" % (
+        seed, kind, diag, l1, n1, l2, n2, l, offs, B, grid, bcast, accumulate, stride2, cabi.last_path())
+    U.assert_parity(flat(U.host(dest.contiguous())), want32, want64, tag, slack=4.0)

@@ -47,15 +47,8 @@ struct OnePairArgs {
 typedef float v2f __attribute__((ext_vector_type(2)));
 typedef const __attribute__((address_space(1))) v2f *GlobalIn;
 typedef __attribute__((address_space(1))) v2f *GlobalOut;
-typedef __attribute__((address_space(1))) char *RowPtr;
 typedef const __attribute__((address_space(4))) float *CoeffPtr;
 typedef const __attribute__((address_space(4))) int *IntPtr;
-
-__device__ __forceinline__ float2 row_load(RowPtr row, unsigned lane_off) {
-  asm volatile("" : "+v"(lane_off));  // keeps base + 32-bit offset visible to the instruction selector
-  const v2f t = *(GlobalIn)(row + lane_off);
-  return make_float2(t.x, t.y);
-}
 
 template <bool DIAG>
 __global__ void __launch_bounds__(64) onepair_bwd_kernel(const OnePairArgs a) {
@@ -94,24 +87,27 @@ __global__ void __launch_bounds__(64) onepair_bwd_kernel(const OnePairArgs a) {
   }
   __syncthreads();
 
-  // per part: the lane's byte offset from row 0 of the wave's first cell
-  unsigned lane_off[kNL];
+  // per part: the address of the lane's element in the row that is read next (rows are read in ascending order, one
+  // per m while |m| <= l), and the distance between rows
+  typedef __attribute__((address_space(1))) char *LanePtr;
+  LanePtr next_row[kNL];
   static_for<kNL>([&](auto dc) __attribute__((always_inline)) {
     constexpr int dl = decltype(dc)::value;
-    lane_off[dl] = ((unsigned)cell_local * (unsigned)a.g[dl].sb + (unsigned)(a.offs[dl] + a.offs_add + chan)) * 8u;
+    const FastPart P = a.g[dl];
+    const int L = lmin + dl;
+    const int first = L > lt ? L - lt : 0;  // row m + L of the first m = -min(L, lt)
+    next_row[dl] = (LanePtr)P.ptr + (((cell0 + cell_local) * P.sb + (long long)first * P.sm) + (a.offs[dl] + a.offs_add + chan)) * 8;
   });
 
   auto load_m = [&](int m, float2(&G)[kNL]) __attribute__((always_inline)) {
     const int mabs = m < 0 ? -m : m;
     static_for<kNL>([&](auto dc) __attribute__((always_inline)) {
       constexpr int dl = decltype(dc)::value;
-      const FastPart P = a.g[dl];
-      const int L = lmin + dl;
       G[dl] = make_float2(0.f, 0.f);
-      if (P.ptr != nullptr && L >= mabs) {  // uniform
-        RowPtr row = (RowPtr)P.ptr + (cell0 * P.sb + (long long)(m + L) * P.sm) * 8;
-        const float2 t = row_load(row, lane_off[dl]);
-        if (valid) G[dl] = t;
+      if (a.g[dl].ptr != nullptr && lmin + dl >= mabs) {  // uniform
+        const v2f t = *(GlobalIn)next_row[dl];
+        next_row[dl] += (long long)a.g[dl].sm * 8;
+        if (valid) G[dl] = make_float2(t.x, t.y);
       }
     });
   };

@@ -4,7 +4,8 @@
 //
 // The map arrives target-major (row_ptr / sources), so every output element is written by exactly one thread, which
 // adds its sources in the order of the map: no atomics, and the float sum is reproducible.  Threads run along
-// (other leading cells, m, channel) with the channel fastest, so the loads of one source slice and the store coalesce.
+// (target, other leading cells, m, channel) with the channel fastest, so the loads of one source slice and the store
+// coalesce, and short slices do not leave lanes idle.
 // HBM-bound: 8 B per (pair, element) read, 8 B per output element written (and read when accumulating).
 #include <algorithm>
 
@@ -25,14 +26,15 @@ struct GatherArgs {
 };
 
 __global__ void __launch_bounds__(256) gather_kernel(const GatherArgs a) {
-  // extents with the gathered dimension taken out: one thread per element of a target slice
+  // extents with the gathered dimension taken out: one thread per element of a target slice, the element index
+  // running fastest, so a wave covers 64 consecutive elements of one target (or the end of one and the start of the next)
   long long E[5];
   for (int k = 0; k < 5; k++) E[k] = k == a.dim ? 1 : a.D[k];
   const long long per_target = E[0] * E[1] * E[2] * E[3] * E[4];
-  const int t = blockIdx.y;
-  const int k0 = a.row_ptr[t], k1 = a.row_ptr[t + 1];
-  for (long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x; e < per_target; e += (long long)gridDim.x * blockDim.x) {
-    long long rem = e, ro = (long long)t * a.rs[a.dim], xo = 0;
+  const long long total = per_target * a.D[a.dim];
+  for (long long w = (long long)blockIdx.x * blockDim.x + threadIdx.x; w < total; w += (long long)gridDim.x * blockDim.x) {
+    const long long t = w / per_target;
+    long long rem = w - t * per_target, ro = t * a.rs[a.dim], xo = 0;
     for (int k = 4; k >= 0; k--) {
       const long long i = rem % E[k];
       rem /= E[k];
@@ -40,6 +42,7 @@ __global__ void __launch_bounds__(256) gather_kernel(const GatherArgs a) {
       xo += i * a.xs[k];   // i = 0 along the gathered dimension
     }
     float2 acc = a.accumulate ? a.r[ro] : make_float2(0.f, 0.f);
+    const int k0 = a.row_ptr[t], k1 = a.row_ptr[t + 1];
     for (int k = k0; k < k1; k++) {
       const float2 v = a.x[xo + (long long)a.sources[k] * a.xs[a.dim]];
       acc.x += v.x;
@@ -68,18 +71,9 @@ int launch_gather(float2 *r, const float2 *x, const long long rs[5], const long 
   a.sources = sources;
   a.accumulate = accumulate ? 1 : 0;
   if (per_target == 0 || D[dim] == 0) return 0;
-  const long long want = (per_target + 255) / 256;
-  const long long cap = std::max<long long>(1, (256LL * 64) / std::max<long long>(1, D[dim]));  // about 64 blocks per CU in all
-  dim3 grid((unsigned)std::min<long long>(want, std::max<long long>(cap, 1)), 1, 1);
-  // gridDim.y is limited to 65535: walk the targets in chunks
-  for (long long t0 = 0; t0 < D[dim]; t0 += 65535) {
-    GatherArgs b = a;
-    const long long nt = std::min<long long>(65535, D[dim] - t0);
-    b.r = a.r + t0 * rs[dim];
-    b.row_ptr = a.row_ptr + t0;
-    grid.y = (unsigned)nt;
-    hipLaunchKernelGGL(gather_kernel, grid, dim3(256), 0, s, b);
-  }
+  const long long total = per_target * D[dim];
+  const long long want = (total + 255) / 256;
+  hipLaunchKernelGGL(gather_kernel, dim3((unsigned)std::min<long long>(want, 256LL * 64)), dim3(256), 0, s, a);
   return hipGetLastError() == hipSuccess ? 0 : 10;
 }
 

@@ -49,6 +49,7 @@ struct Diag6Args {
   int n;              // channels of every part
   int offs_add;
   int accumulate;
+  int want_x, want_y;  // backward: which gradients are stored (the operand of an unwanted one is never read)
 };
 
 int launch_diag6_fwd_l6(const Diag6Args &a, hipStream_t s);  // product l up to 6

@@ -306,23 +306,37 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(PACKED
   const WavePos q = wave_pos(a, w);
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const bool accumulate = a.accumulate != 0;
+  const bool wx = a.want_x != 0, wy = a.want_y != 0;
   for (int e = threadIdx.x; e < kImgRows * 64; e += 256) yimg[e] = make_float2(0.f, 0.f);
   __syncthreads();
   static_for<kNP>([&](auto l1c) __attribute__((always_inline)) {
     constexpr int L1 = decltype(l1c)::value;
     if (a.x[L1].ptr != nullptr) {  // the same for the whole block
+      // x is needed for the y-gradient only and y for the x-gradient only; an operand whose gradient is not wanted is
+      // never read (a part-level call for one gradient does not even have it) and enters as zeros
       float2 xv[2 * L1 + 1], ax[2 * L1 + 1];
-      load_rows<L1, PACKED>(xv, a.x[L1], q);
+      if (wy) {
+        load_rows<L1, PACKED>(xv, a.x[L1], q);
+      } else {
+#pragma unroll
+        for (int m1 = 0; m1 <= 2 * L1; m1++) xv[m1] = make_float2(0.f, 0.f);
+      }
 #pragma unroll
       for (int m1 = 0; m1 <= 2 * L1; m1++) ax[m1] = make_float2(0.f, 0.f);
       static_for<kNP>([&](auto l2c) __attribute__((always_inline)) {
         constexpr int L2 = kL6 - decltype(l2c)::value;  // descending, so that neighbours in l2 run at the same time
         if (owner_of(L2) == wave && a.y[L2].ptr != nullptr) {
           float2 yv[2 * L2 + 1];
-          load_rows<L2, PACKED>(yv, a.y[L2], q);
+          if (wx) {
+            load_rows<L2, PACKED>(yv, a.y[L2], q);
+          } else {
+#pragma unroll
+            for (int m2 = 0; m2 <= 2 * L2; m2++) yv[m2] = make_float2(0.f, 0.f);
+          }
           bwd_pair<L1, L2, LCAP, PACKED>(a, xv, yv, ax, yimg, q);
         }
       });
+      if (!wx) return;  // continues with the next l1 (this is the body of a per-l1 lambda); uniform for the block
       float2 *mine = xpart + wave * kXRows * 64 + lane;
 #pragma unroll
       for (int m1 = 0; m1 <= 2 * L1; m1++) mine[m1 * 64] = ax[m1];
@@ -350,7 +364,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(PACKED
   static_for<kNP>([&](auto l2c) __attribute__((always_inline)) {
     constexpr int L2 = decltype(l2c)::value;
     const FastPart YG = a.yg[L2];
-    if (owner_of(L2) == wave && YG.ptr != nullptr)
+    if (wy && owner_of(L2) == wave && YG.ptr != nullptr)
       store_rows<L2, PACKED>(yimg + (L2 * L2) * 64 + lane, 64, YG, q, accumulate);
   });
 }

@@ -139,17 +139,42 @@ int diag6_vec_bwd(const VecPlan &plan, const std::vector<const gelib_part_desc *
                   const std::vector<const gelib_part_desc *> &xg, const std::vector<const gelib_part_desc *> &yg,
                   bool accumulate, hipStream_t s, int *used) {
   *used = 0;
-  if (xg.empty() || yg.empty()) return GELIB_HIP_OK;  // one gradient alone goes to the other kernel families
+  if (xg.empty() && yg.empty()) return GELIB_HIP_OK;
   Diag6Args a;
   int lcap = 0;
   bool ok = false;
-  int rc = make_args(plan, g, x, y, &xg, &yg, false, &a, &lcap, &ok);
+  int rc = make_args(plan, g, x, y, xg.empty() ? nullptr : &xg, yg.empty() ? nullptr : &yg, false, &a, &lcap, &ok);
   if (rc || !ok) return rc;
   if (lcap > kL6) return GELIB_HIP_OK;
   a.accumulate = accumulate ? 1 : 0;
+  a.want_x = xg.empty() ? 0 : 1;
+  a.want_y = yg.empty() ? 0 : 1;
   if ((rc = a.lg_npad < 6 ? launch_diag6_bwd_l6_packed(a, s) : launch_diag6_bwd_l6(a, s))) return rc;
   *used = 1;
   return GELIB_HIP_OK;
+}
+
+// One triple (the part-level entry points).  kind 0: r += x * y; 1: the x-shaped tensor is the gradient wanted, r is the
+// incoming gradient and the x operand does not exist; 2: likewise for y.  The missing operand is stood in for by the
+// gradient's own descriptor: it only marks the part as present, the kernel never reads an operand whose gradient is
+// not wanted.
+int diag6_part(int kind, const long long E[3], const gelib_part_desc *r, const gelib_part_desc *x,
+               const gelib_part_desc *y, int l1, int l2, int l, int offs, bool accumulate, hipStream_t s, int *used) {
+  *used = 0;
+  VecPlan plan;
+  plan.diag = true;
+  for (int k = 0; k < 3; k++) plan.E[k] = E[k];
+  VecTriple t;
+  t.xi = t.yi = t.ri = 0;
+  t.l1 = l1;
+  t.l2 = l2;
+  t.l = l;
+  t.offs = offs;
+  t.nout = (int)x->dims[4];
+  plan.triples.push_back(t);
+  const std::vector<const gelib_part_desc *> R = {r}, X = {x}, Y = {y}, none;
+  if (kind == 0) return diag6_vec_fwd(plan, R, X, Y, accumulate, s, used);
+  return diag6_vec_bwd(plan, R, X, Y, kind == 1 ? X : none, kind == 2 ? Y : none, accumulate, s, used);
 }
 
 int diag6_set_option(const char *name, int value) {

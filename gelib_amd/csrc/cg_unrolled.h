@@ -84,6 +84,9 @@ int diag6_vec_bwd(const VecPlan &plan, const std::vector<const gelib_part_desc *
                   const std::vector<const gelib_part_desc *> &x, const std::vector<const gelib_part_desc *> &y,
                   const std::vector<const gelib_part_desc *> &xg, const std::vector<const gelib_part_desc *> &yg,
                   bool accumulate, hipStream_t s, int *used);
+// one triple; kind 0 forward, 1 gradient of x (x is the destination), 2 gradient of y; E = common leading extents
+int diag6_part(int kind, const long long E[3], const gelib_part_desc *r, const gelib_part_desc *x,
+               const gelib_part_desc *y, int l1, int l2, int l, int offs, bool accumulate, hipStream_t s, int *used);
 int diag6_set_option(const char *name, int value);
 
 }  // namespace gelib_hip

@@ -80,6 +80,15 @@ def test_diag6_vec(cabi, B, tx, ty, maxl):
         assert U.gate_excess(U.host(a), 2 * U.host(b)) <= 1.0
     for a, b in zip(dxg2 + dyg2, dxg + dyg):
         assert U.gate_excess(U.host(a), 2 * U.host(b), rtol=2e-5, atol=2e-5) <= 1.0
+    # one gradient per call: the same kernel with the other one switched off, bit for bit the same sums
+    dxg3 = [torch.full_like(a, 9.0) for a in dxg]
+    dyg3 = [torch.full_like(a, 9.0) for a in dyg]
+    cabi.so3vec_bwd(dxg3, None, dgs, dxs, dys, accumulate=False, diag=True)
+    assert cabi.last_path() == DIAG6
+    cabi.so3vec_bwd(None, dyg3, dgs, dxs, dys, accumulate=False, diag=True)
+    assert cabi.last_path() == DIAG6
+    for a, b in zip(dxg3 + dyg3, dxg + dyg):
+        assert torch.equal(torch.view_as_real(a), torch.view_as_real(b))
 
 
 def test_diag6_declines_what_it_cannot_do(cabi):

@@ -261,32 +261,43 @@ PartOp triple_op(const VecPlan &plan, const VecTriple &t, const std::vector<View
   return op;
 }
 
-int vec_fwd_entry(bool diag, int nr, const gelib_part_desc *r, int nx, const gelib_part_desc *x, int ny,
-                  const gelib_part_desc *y, int accumulate, void *stream) {
-  t_last_path = kPathNone;
-  std::vector<View> R, X, Y;
+// A Diag product that reaches above l = 6: the lane-per-channel kernels (built for products up to l = 6) take the
+// triples up to there, the other families the rest.  R is sorted by l, so A keeps a prefix of it and B the remainder.
+bool split_diag(const VecPlan &plan, const std::vector<View> &R, VecPlan &A, VecPlan &B, std::vector<View> &RA,
+                std::vector<View> &RB) {
+  constexpr int kSplit = 6;
+  if (!plan.diag) return false;
+  bool lo = false, hi = false;
+  for (auto &t : plan.triples) (t.l <= kSplit ? lo : hi) = true;
+  if (!lo || !hi) return false;
+  size_t k0 = 0;
+  while (k0 < R.size() && R[k0].l <= kSplit) k0++;
+  A.diag = B.diag = true;
+  for (int k = 0; k < 3; k++) A.E[k] = B.E[k] = plan.E[k];
+  for (auto t : plan.triples) {
+    if (t.l <= kSplit) {
+      A.triples.push_back(t);
+    } else {
+      t.ri -= (int)k0;
+      B.triples.push_back(t);
+    }
+  }
+  RA.assign(R.begin(), R.begin() + k0);
+  RB.assign(R.begin() + k0, R.end());
+  return true;
+}
+
+// The kernel families in the order they are tried, then the shape-agnostic kernels.
+int fwd_dispatch(const VecPlan &plan, const std::vector<View> &R, const std::vector<View> &X, const std::vector<View> &Y,
+                 int accumulate, hipStream_t s) {
   int rc;
-  if ((rc = sort_parts(nr, r, kMaxOutParts, R)) || (rc = sort_parts(nx, x, kMaxParts, X)) ||
-      (rc = sort_parts(ny, y, kMaxParts, Y)))
-    return rc;
-  if (R.empty() || X.empty() || Y.empty()) return GELIB_HIP_OK;
-  VecPlan plan;
-  if ((rc = build_vec_plan(diag, R, X, Y, plan))) return rc;
-  for (auto &v : R)
-    if ((rc = check_pointer(v.d))) return rc;
-  for (auto &v : X)
-    if ((rc = check_pointer(v.d))) return rc;
-  for (auto &v : Y)
-    if ((rc = check_pointer(v.d))) return rc;
-  if (plan.E[0] * plan.E[1] * plan.E[2] == 0 || plan.triples.empty()) return GELIB_HIP_OK;
-  hipStream_t s = (hipStream_t)stream;
   if (!g_force_generic) {
     std::vector<const gelib_part_desc *> rd, xd, yd;
     for (auto &v : R) rd.push_back(v.d);
     for (auto &v : X) xd.push_back(v.d);
     for (auto &v : Y) yd.push_back(v.d);
     int used = 0;
-    // Diag products with more than 32 channels: one lane per channel beats the lane-per-channel-pair kernels
+    // Diag products: one lane per channel beats the lane-per-channel-pair kernels
     rc = diag6_vec_fwd(plan, rd, xd, yd, accumulate != 0, s, &used);
     if (rc) return rc;
     if (used) {
@@ -311,6 +322,108 @@ int vec_fwd_entry(bool diag, int nr, const gelib_part_desc *r, int nx, const gel
     PartOp op = triple_op(plan, t, R, X, Y);
     if ((rc = launch_generic_fwd(op, accumulate != 0, s))) return rc;
   }
+  return GELIB_HIP_OK;
+}
+
+int vec_fwd_entry(bool diag, int nr, const gelib_part_desc *r, int nx, const gelib_part_desc *x, int ny,
+                  const gelib_part_desc *y, int accumulate, void *stream) {
+  t_last_path = kPathNone;
+  std::vector<View> R, X, Y;
+  int rc;
+  if ((rc = sort_parts(nr, r, kMaxOutParts, R)) || (rc = sort_parts(nx, x, kMaxParts, X)) ||
+      (rc = sort_parts(ny, y, kMaxParts, Y)))
+    return rc;
+  if (R.empty() || X.empty() || Y.empty()) return GELIB_HIP_OK;
+  VecPlan plan;
+  if ((rc = build_vec_plan(diag, R, X, Y, plan))) return rc;
+  for (auto &v : R)
+    if ((rc = check_pointer(v.d))) return rc;
+  for (auto &v : X)
+    if ((rc = check_pointer(v.d))) return rc;
+  for (auto &v : Y)
+    if ((rc = check_pointer(v.d))) return rc;
+  if (plan.E[0] * plan.E[1] * plan.E[2] == 0 || plan.triples.empty()) return GELIB_HIP_OK;
+  hipStream_t s = (hipStream_t)stream;
+  if (!g_force_generic) {
+    VecPlan A, B;
+    std::vector<View> RA, RB;
+    if (split_diag(plan, R, A, B, RA, RB)) {
+      std::vector<const gelib_part_desc *> rd, xd, yd;
+      for (auto &v : RA) rd.push_back(v.d);
+      for (auto &v : X) xd.push_back(v.d);
+      for (auto &v : Y) yd.push_back(v.d);
+      int used = 0;
+      if ((rc = diag6_vec_fwd(A, rd, xd, yd, accumulate != 0, s, &used))) return rc;
+      if (used) {
+        rc = fwd_dispatch(B, RB, X, Y, accumulate, s);
+        t_last_path = kPathDiag6;
+        return rc;
+      }
+    }
+  }
+  return fwd_dispatch(plan, R, X, Y, accumulate, s);
+}
+
+int bwd_dispatch(const VecPlan &plan, const std::vector<View> &G, const std::vector<View> &X, const std::vector<View> &Y,
+                 const std::vector<View> &XG, const std::vector<View> &YG, bool want_x, bool want_y, int accumulate,
+                 hipStream_t s, bool skip_unrolled = false) {
+  int rc;
+  if (!g_force_generic && !plan.triples.empty()) {
+    std::vector<const gelib_part_desc *> gd, xd, yd, xgd, ygd;
+    for (auto &v : G) gd.push_back(v.d);
+    for (auto &v : X) xd.push_back(v.d);
+    for (auto &v : Y) yd.push_back(v.d);
+    for (auto &v : XG) xgd.push_back(v.d);
+    for (auto &v : YG) ygd.push_back(v.d);
+    int used = 0;
+    rc = diag6_vec_bwd(plan, gd, xd, yd, xgd, ygd, accumulate != 0, s, &used);
+    if (rc) return rc;
+    if (used) {
+      t_last_path = kPathDiag6;
+      return GELIB_HIP_OK;
+    }
+    if (!skip_unrolled) {
+      rc = unrolled_vec_bwd(plan, gd, xd, yd, xgd, ygd, accumulate != 0, s, &used);
+      if (rc) return rc;
+      if (used) {
+        t_last_path = kPathUnrolled;
+        return GELIB_HIP_OK;
+      }
+    }
+    rc = onepair_vec_bwd(plan, gd, xd, yd, xgd, ygd, accumulate != 0, s, &used);
+    if (rc) return rc;
+    if (used) {
+      t_last_path = kPathOnePair;
+      return GELIB_HIP_OK;
+    }
+    rc = staged_vec_bwd(plan, gd, xd, yd, xgd, ygd, accumulate != 0, s, &used);
+    if (rc) return rc;
+    if (used) {
+      t_last_path = kPathStaged;
+      return GELIB_HIP_OK;
+    }
+  }
+  t_last_path = kPathGeneric;
+  // shape-agnostic route: zero the destinations when overwriting, then one accumulation per triple,
+  // all back0 first and then all back1 like the reference (python/src/gelib/SO3vec.py:267-268)
+  if (!accumulate) {
+    for (auto *L : {&XG, &YG})
+      for (auto &v : *L) {
+        long long own[3];
+        PartDev pd = to_dev(v.d, plan.E, own);
+        if ((rc = launch_zero_fill(pd, own, 2 * v.l + 1, v.n, s))) return rc;
+      }
+  }
+  if (want_x)
+    for (auto &t : plan.triples) {
+      PartOp op = triple_op(plan, t, G, XG, Y);
+      if ((rc = launch_generic_back0(op, true, s))) return rc;
+    }
+  if (want_y)
+    for (auto &t : plan.triples) {
+      PartOp op = triple_op(plan, t, G, X, YG);
+      if ((rc = launch_generic_back1(op, true, s))) return rc;
+    }
   return GELIB_HIP_OK;
 }
 
@@ -347,61 +460,29 @@ int vec_bwd_entry(bool diag, const gelib_part_desc *xg, const gelib_part_desc *y
       if ((rc = check_pointer(v.d))) return rc;
   if (plan.E[0] * plan.E[1] * plan.E[2] == 0) return GELIB_HIP_OK;
   hipStream_t s = (hipStream_t)stream;
-  if (!g_force_generic && !plan.triples.empty()) {
-    std::vector<const gelib_part_desc *> gd, xd, yd, xgd, ygd;
-    for (auto &v : G) gd.push_back(v.d);
-    for (auto &v : X) xd.push_back(v.d);
-    for (auto &v : Y) yd.push_back(v.d);
-    for (auto &v : XG) xgd.push_back(v.d);
-    for (auto &v : YG) ygd.push_back(v.d);
-    int used = 0;
-    rc = diag6_vec_bwd(plan, gd, xd, yd, xgd, ygd, accumulate != 0, s, &used);
-    if (rc) return rc;
-    if (used) {
-      t_last_path = kPathDiag6;
-      return GELIB_HIP_OK;
-    }
-    rc = unrolled_vec_bwd(plan, gd, xd, yd, xgd, ygd, accumulate != 0, s, &used);
-    if (rc) return rc;
-    if (used) {
-      t_last_path = kPathUnrolled;
-      return GELIB_HIP_OK;
-    }
-    rc = onepair_vec_bwd(plan, gd, xd, yd, xgd, ygd, accumulate != 0, s, &used);
-    if (rc) return rc;
-    if (used) {
-      t_last_path = kPathOnePair;
-      return GELIB_HIP_OK;
-    }
-    rc = staged_vec_bwd(plan, gd, xd, yd, xgd, ygd, accumulate != 0, s, &used);
-    if (rc) return rc;
-    if (used) {
-      t_last_path = kPathStaged;
-      return GELIB_HIP_OK;
-    }
-  }
-  t_last_path = kPathGeneric;
-  // shape-agnostic route: zero the destinations when overwriting, then one accumulation per triple,
-  // all back0 first and then all back1 like the reference (python/src/gelib/SO3vec.py:267-268)
-  if (!accumulate) {
-    for (auto *L : {&XG, &YG})
-      for (auto &v : *L) {
-        long long own[3];
-        PartDev pd = to_dev(v.d, plan.E, own);
-        if ((rc = launch_zero_fill(pd, own, 2 * v.l + 1, v.n, s))) return rc;
+  if (!g_force_generic) {
+    VecPlan A, B;
+    std::vector<View> GA, GB;
+    if (split_diag(plan, G, A, B, GA, GB)) {
+      std::vector<const gelib_part_desc *> gd, xd, yd, xgd, ygd;
+      for (auto &v : GA) gd.push_back(v.d);
+      for (auto &v : X) xd.push_back(v.d);
+      for (auto &v : Y) yd.push_back(v.d);
+      for (auto &v : XG) xgd.push_back(v.d);
+      for (auto &v : YG) ygd.push_back(v.d);
+      int used = 0;
+      if ((rc = diag6_vec_bwd(A, gd, xd, yd, xgd, ygd, accumulate != 0, s, &used))) return rc;
+      if (used) {
+        // The rest adds on top of what the first part wrote.  It is a few triples of a vector with many parts: the
+        // unrolled backward kernels stage and flush the images of all parts per cell whatever the number of triples
+        // (39 ms against 18 ms on Diag L=4, 64 channels, 131072 cells, uncapped), so they are passed over here.
+        rc = bwd_dispatch(B, GB, X, Y, XG, YG, xg != nullptr, yg != nullptr, 1, s, true);
+        t_last_path = kPathDiag6;
+        return rc;
       }
+    }
   }
-  if (xg)
-    for (auto &t : plan.triples) {
-      PartOp op = triple_op(plan, t, G, XG, Y);
-      if ((rc = launch_generic_back0(op, true, s))) return rc;
-    }
-  if (yg)
-    for (auto &t : plan.triples) {
-      PartOp op = triple_op(plan, t, G, X, YG);
-      if ((rc = launch_generic_back1(op, true, s))) return rc;
-    }
-  return GELIB_HIP_OK;
+  return bwd_dispatch(plan, G, X, Y, XG, YG, xg != nullptr, yg != nullptr, accumulate, s);
 }
 
 }  // namespace

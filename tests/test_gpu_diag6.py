@@ -92,12 +92,12 @@ def test_diag6_vec(cabi, B, tx, ty, maxl):
 
 
 def test_diag6_declines_what_it_cannot_do(cabi):
-    # a broadcast operand whose gradient is wanted, a product above l = 6: other families run
+    # a product above l = 6 is shared with the other families; a broadcast operand whose gradient is wanted is theirs
     x = [U.dev(U.seeded(1, 1, 13, 64))]
     y = [U.dev(U.seeded(2, 4, 13, 64))]
     r = [torch.zeros(4, 2 * l + 1, 64, dtype=torch.complex64, device="cuda") for l in range(13)]
     cabi.so3vec_fwd(r, x, y, accumulate=False, diag=True)
-    assert cabi.last_path() != DIAG6          # product l up to 12
+    assert cabi.last_path() == DIAG6          # product l up to 12: split at l = 6
     want = ora.vec_fwd([U.host(x[0])], [U.host(y[0])], -1, True)
     for a, b in zip(r, want):
         assert U.gate_excess(U.host(a), b) <= 1.0
@@ -118,3 +118,34 @@ def test_diag6_declines_what_it_cannot_do(cabi):
     want8 = ora.vec_fwd([U.host(x8[0])], [U.host(y8[0])], 6, True)
     for a, b in zip(r8, want8):
         assert U.gate_excess(U.host(a), b) <= 1.0
+
+
+@pytest.mark.parametrize("B,tau,maxl", [(5, {l: 64 for l in range(5)}, -1), (3, {l: 16 for l in range(7)}, -1),
+                                        (4, {2: 40, 6: 40}, 9)])
+def test_diag_product_above_l6_is_split(cabi, B, tau, maxl):
+    """A Diag product whose l reaches above 6: the triples up to l = 6 run on the lane-per-channel kernels, the rest on
+    the other families, the gradients of the second part added on top of the first."""
+    xs = [U.seeded(40 + l, B, 2 * l + 1, n) for l, n in sorted(tau.items())]
+    ys = [U.seeded(60 + l, B, 2 * l + 1, n) for l, n in sorted(tau.items())]
+    r32 = ora.vec_fwd(xs, ys, maxl, True)
+    r64 = ora.vec_fwd(c128(xs), c128(ys), maxl, True)
+    assert max((p.shape[1] - 1) // 2 for p in r32) > 6
+    gs = [U.seeded(80 + i, *p.shape) for i, p in enumerate(r32)]
+    xg32, yg32 = ora.vec_bwd(gs, xs, ys, True)
+    xg64, yg64 = ora.vec_bwd(c128(gs), c128(xs), c128(ys), True)
+    dxs, dys, dgs = [U.dev(a) for a in xs], [U.dev(a) for a in ys], [U.dev(a) for a in gs]
+    for accumulate in (False, True):
+        start = 5.0 - 1j if accumulate else 7.0 + 1j
+        drs = [torch.full(p.shape, start, dtype=torch.complex64, device="cuda") for p in r32]
+        cabi.so3vec_fwd(drs, dxs, dys, accumulate=accumulate, diag=True)
+        assert cabi.last_path() == DIAG6
+        dxg = [torch.full(a.shape, start, dtype=torch.complex64, device="cuda") for a in xs]
+        dyg = [torch.full(a.shape, start, dtype=torch.complex64, device="cuda") for a in ys]
+        cabi.so3vec_bwd(dxg, dyg, dgs, dxs, dys, accumulate=accumulate, diag=True)
+        assert cabi.last_path() == DIAG6
+        torch.cuda.synchronize()
+        off = start if accumulate else 0
+        for a, b, c in zip(drs, r32, r64):
+            U.assert_parity(U.host(a) - np.complex64(off), b, c, "fwd", slack=4.0)
+        for a, b, c in zip(dxg + dyg, xg32 + yg32, xg64 + yg64):
+            U.assert_parity(U.host(a) - np.complex64(off), b, c, "grad", slack=8.0)

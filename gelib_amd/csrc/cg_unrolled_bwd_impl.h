@@ -2,7 +2,7 @@
 //
 // Work split.  A block owns a few whole cells (one cell when a cell has >= 256 channel slots).  The operands x, y
 // of those cells are staged once in LDS next to the coefficient bank.  For every (l1,l2) pair the flattened
-// (cell, slot) space is cut into runs of 64 slots; a wave takes every fourth run.  In a run a lane owns one
+// (cell, slot) space is cut into runs of 64 slots; the runs of all pairs are dealt to the four waves in turn.  In a run a lane owns one
 // channel pair (i, j) of the gradient block: it reads g[m, i*n2+j] for every m (contiguous across the wave), forms
 // C*g once per (m1,m2) and feeds two complex FMAs,
 //     ax[m1] += (C g) conj(y[m2, j])        ay[m2] += (C g) conj(x[m1, i]),
@@ -318,11 +318,15 @@ __global__ void __launch_bounds__(kBlock) unrolled_bwd_kernel(const BwdArgs a) {
   static_for<LCAP + 1>([&](auto l) __attribute__((always_inline)) { gp.G[l.value] = a.g[l.value]; });
   const CoeffPtr Zc = (CoeffPtr)(a.bank + a.zero_off);    // a table of zeros and ...
   const GlobalRows zrows = (GlobalRows)(a.bank + a.zero_off);  // ... a row of zeros, for parts that are absent
+  int dealt = 0;  // runs handed out so far: the runs of all pairs go round the waves, so that pairs with fewer runs
+                  // than waves (few channels, few cells per block) do not leave the same waves idle every time
   for (int pidx = 0; pidx < npairs; pidx++) {
     const PairPtr p = pairs + pidx;
     const int nruns = runs_of(pidx);
     CoeffPtr C = (CoeffPtr)(a.bank + p->cg_base);
-    for (int run = wave; run < nruns; run += kWaves) {
+    const int first = (wave - dealt) & (kWaves - 1);
+    dealt += nruns;
+    for (int run = first; run < nruns; run += kWaves) {
       const LanePos q = lane_pos(run, lane, p->log2_u, ncell);
       switch (p->l1 * (kLT + 1) + p->l2) {
 #define GELIB_CASE(A, B)                                                                                      \

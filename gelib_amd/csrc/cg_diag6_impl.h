@@ -21,7 +21,8 @@ namespace gelib_hip {
 
 namespace {
 
-constexpr int kRowBudget = 28;  // rows of g a lane keeps in flight
+constexpr int kRowBudget = 28;        // rows of g a lane keeps in flight
+constexpr int kRowBudgetPacked = 20;  // several cells per wave: a lane offset per part costs registers, and 168 is the limit
 
 typedef float v2f __attribute__((ext_vector_type(2)));
 typedef const __attribute__((address_space(1))) v2f *GlobalIn;
@@ -192,7 +193,8 @@ __device__ __forceinline__ void bwd_pair(const Diag6Args &a, const float2 (&xv)[
   if constexpr (LMIN <= LCAP) {
     constexpr int NL = LTOP - LMIN + 1;
     constexpr int ROWS = (LTOP + 1) * (LTOP + 1) - LMIN * LMIN;
-    constexpr int PF = ROWS <= kRowBudget ? 2 * LTOP + 1 : (kRowBudget / NL > 1 ? kRowBudget / NL : 1);
+    constexpr int kBudget = PACKED ? kRowBudgetPacked : kRowBudget;
+    constexpr int PF = ROWS <= kBudget ? 2 * LTOP + 1 : (kBudget / NL > 1 ? kBudget / NL : 1);
     const OffsPtr offs = (OffsPtr)a.offs + (L1 * kNP + L2) * kNR;
     const CoeffPtr C = (CoeffPtr)a.bank;
     // a triple that is not there reads a row of zeros (its coefficients then do not matter), so the arithmetic has
@@ -295,10 +297,11 @@ constexpr int owner_of(int l2) { return l2 == 6 ? 0 : (l2 == 5 || l2 == 0) ? 1 :
 // wave; the partials meet in LDS after the last pair of l1, are added in the order of the waves and written out, the
 // rows dealt round-robin to the waves.  Pairs (l1, l2) and (l1, l2 +- 1) read neighbouring 512-byte blocks of the same
 // rows of g, and they are in flight at about the same time.
-// Three waves per SIMD (168 registers) is what the LDS of a block lets a compute unit hold.  The one-cell form fits by
-// itself; the packed form is one register over and is capped (capping the other one too changes its schedule for the worse).
+// Three waves per SIMD (168 registers) is what the LDS of a block lets a compute unit hold; both forms fit by
+// themselves (the packed one with a smaller row budget).  Forcing the limit with amdgpu_waves_per_eu instead changed the
+// schedule for the worse (twice as many waits).
 template <int LCAP, bool PACKED>
-__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(PACKED ? 3 : 1))) diag6_bwd_kernel(const Diag6Args a) {
+__global__ void __launch_bounds__(256) diag6_bwd_kernel(const Diag6Args a) {
   constexpr int kXRows = 2 * kL6 + 1;
   __shared__ float2 yimg[kImgRows * 64];
   __shared__ float2 xpart[4 * kXRows * 64];  // [wave][row][lane]

@@ -17,7 +17,7 @@ SYMBOLS = [
     "gelib_hip_so3part_diagcg_fwd", "gelib_hip_so3part_diagcg_back0", "gelib_hip_so3part_diagcg_back1",
     "gelib_hip_so3vec_cg_fwd", "gelib_hip_so3vec_cg_bwd", "gelib_hip_so3vec_diagcg_fwd",
     "gelib_hip_so3vec_diagcg_bwd", "gelib_hip_so3part_spharm", "gelib_hip_gather_map_create",
-    "gelib_hip_gather_map_destroy", "gelib_hip_part_gather", "gelib_hip_set_option", "gelib_hip_last_path",
+    "gelib_hip_gather_map_destroy", "gelib_hip_part_gather", "gelib_hip_part_mix_channels", "gelib_hip_set_option", "gelib_hip_last_path",
     "gelib_hip_malloc", "gelib_hip_free", "gelib_hip_memcpy", "gelib_hip_memset", "gelib_hip_synchronize",
 ]
 
@@ -68,6 +68,9 @@ def lib():
         L.gelib_hip_gather_map_destroy.argtypes = [ctypes.c_void_p]
         L.gelib_hip_part_gather.argtypes = [P, P, ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int,
                                             ctypes.c_void_p]
+        L.gelib_hip_part_mix_channels.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64,
+                                                  ctypes.c_int, ctypes.c_int, ctypes.c_int64, ctypes.c_int64,
+                                                  ctypes.c_int, ctypes.c_void_p]
         L.gelib_hip_set_option.argtypes = [ctypes.c_char_p, ctypes.c_int]
         _lib = L
     return _lib
@@ -213,6 +216,24 @@ def part_gather(r, x, gmap, dim, inverse=False, accumulate=True):
     5-D views; inverse swaps the roles of sources and targets."""
     check(lib().gelib_hip_part_gather(ctypes.byref(desc(r)), ctypes.byref(desc(x)), gmap.handle, int(dim), int(inverse),
                                       int(accumulate), _stream(r)))
+
+
+def mix_channels_ok(x):
+    """True if part_mix_channels takes x as it is: contiguous rows of an even number of channels, 16-byte aligned."""
+    return x.is_contiguous() and x.shape[-1] > 0 and x.shape[-1] % 2 == 0 and x.data_ptr() % 16 == 0
+
+
+def part_mix_channels(r, x, w, adjoint=False):
+    """r[..., o] = sum_c x[..., c] V[c, o] with V = w (n_in, n_out), or V = w^H for w (n_out, n_in) when adjoint.
+    r and x are contiguous complex64 tensors that differ only in their last extent."""
+    n_in, n_out = x.shape[-1], r.shape[-1]
+    if tuple(w.shape) != ((n_out, n_in) if adjoint else (n_in, n_out)) or r.shape[:-1] != x.shape[:-1]:
+        raise ValueError("shapes of r, x and w do not fit")
+    if not (r.is_contiguous() and x.is_contiguous() and w.is_contiguous()):
+        raise ValueError("contiguous tensors are needed")
+    rows = x.numel() // n_in if n_in else 0
+    check(lib().gelib_hip_part_mix_channels(r.data_ptr(), x.data_ptr(), w.data_ptr(), rows, n_in, n_out, n_out, n_in,
+                                            int(adjoint), _stream(r)))
 
 
 def set_option(name, value):

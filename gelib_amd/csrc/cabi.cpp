@@ -703,6 +703,29 @@ int gelib_hip_part_gather(const gelib_part_desc *r, const gelib_part_desc *x, co
                        accumulate != 0, (hipStream_t)stream);
 }
 
+// ---- channel mixing (the linear layer that consumes a product) ------------------------------------------------------
+int gelib_hip_part_mix_channels(void *r, const void *x, const void *w, int64_t rows, int n_in, int n_out,
+                                int64_t r_row_stride, int64_t x_row_stride, int adjoint, void *stream) {
+  t_last_path = kPathNone;
+  if (rows < 0 || n_in < 0 || n_out < 0 || r_row_stride < n_out || x_row_stride < n_in) return GELIB_HIP_ERR_ARG;
+  if (rows == 0 || n_out == 0) return GELIB_HIP_OK;
+  if (!r || (n_in > 0 && (!x || !w))) return GELIB_HIP_ERR_NULL;
+  if (n_in == 0 || (n_in & 1) || (x_row_stride & 1) || ((uintptr_t)x & 15) || rows > (1LL << 38))
+    return GELIB_HIP_ERR_ARG;
+  const int64_t rd[5] = {rows, 1, 1, 1, n_out}, rst[5] = {r_row_stride, 0, 0, 0, 1};
+  const int64_t xd[5] = {rows, 1, 1, 1, n_in}, xst[5] = {x_row_stride, 0, 0, 0, 1};
+  const int64_t wd[5] = {adjoint ? n_out : n_in, 1, 1, 1, adjoint ? n_in : n_out};
+  const int64_t wst[5] = {wd[4], 0, 0, 0, 1};
+  int rc;
+  if ((rc = check_range(r, rd, rst, 2 * sizeof(float))) || (rc = check_range(x, xd, xst, 2 * sizeof(float))) ||
+      (rc = check_range(w, wd, wst, 2 * sizeof(float))))
+    return rc;
+  t_last_path = kPathGeneric;
+  rc = launch_mix((float2 *)r, (const float2 *)x, (const float2 *)w, rows, n_in, n_out, x_row_stride, r_row_stride,
+                  adjoint != 0, (hipStream_t)stream);
+  return rc == 11 ? GELIB_HIP_ERR_ARG : rc;
+}
+
 int gelib_hip_malloc(void **ptr, uint64_t bytes) {
   if (!ptr) return GELIB_HIP_ERR_NULL;
   *ptr = nullptr;

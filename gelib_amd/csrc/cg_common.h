@@ -59,4 +59,9 @@ int launch_spharm(const PartDev &r, const float *x, const long long xs[5], const
 int launch_gather(float2 *r, const float2 *x, const long long rs[5], const long long xs[5], const long long D[5], int dim,
                   const int *row_ptr, const int *sources, bool accumulate, hipStream_t s);
 
+// ---- channel mixing on the matrix cores (mix.hip): r[row, :] = x[row, :] V, V = W (n_in, n_out) or W^H for W (n_out, n_in);
+// strides in complex elements.  Returns 0, 10 (a HIP call failed) or 11 (n_in odd or rows of x not 16-byte aligned)
+int launch_mix(float2 *r, const float2 *x, const float2 *w, long long rows, int n_in, int n_out, long long xs,
+               long long rs, bool adjoint, hipStream_t s);
+
 }  // namespace gelib_hip

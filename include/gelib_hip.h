@@ -133,6 +133,16 @@ int gelib_hip_so3vec_diagcg_bwd(const gelib_part_desc *xg, const gelib_part_desc
 int gelib_hip_so3part_spharm(const gelib_part_desc *r, const float *x, const int64_t xdims[5],
                              const int64_t xstrides[5], int accumulate, void *stream);
 
+/* ---- consumer of a product: channel mixing ----------------------------------------------------------------------------
+ * r[row, o] = sum_c x[row, c] V[c, o], row = 0..rows-1 (the flattened (batch, grid, m) index of a part), overwriting r.
+ * adjoint == 0: V = w, a row-major (n_in, n_out) complex matrix: the torch.matmul(part, W) of SO3vec.__mul__ /
+ * SO3linear (python/src/gelib/SO3vec.py:174-177, python/src/gelib/SO3weights.py:75-85).  adjoint != 0: w is
+ * (n_out, n_in) and V = w^H: the gradient of that matmul with respect to the part (torch's autograd forms it in the
+ * reference).  Row strides in complex elements.  n_in must be even and the rows of x 16-byte aligned (else
+ * GELIB_HIP_ERR_ARG).  The re-packed matrix is kept in a buffer per (device, stream) that grows on demand. */
+int gelib_hip_part_mix_channels(void *r, const void *x, const void *w, int64_t rows, int n_in, int n_out,
+                                int64_t r_row_stride, int64_t x_row_stride, int adjoint, void *stream);
+
 /* ---- gather: sums of slices along the batch or a grid dimension ---------------------------------------------------------
  * A gather map is a list of (source, target) pairs with 0 <= source < n_in, 0 <= target < n_out (the arguments of
  * cnine::GatherMapB(sources, targets), python/bindings/gather_map_py.cpp:17-18).  create() checks the indices, sorts the

@@ -1,0 +1,62 @@
+"""Channel mixing (the linear layer that consumes a product) through the C-ABI, against numpy's complex128 matmul.
+
+Tolerance: the matrix cores add the 2 n_in real terms of an output one after the other in float32, so the error of an
+output is a rounding error of its sum and is measured against the size of that sum, not of its (possibly cancelling)
+value:  |gpu - exact| <= 1e-6 + 4 eps32 * sum_c |x_c| |V_co|.  A dropped term, a wrong sign or a transposed weight
+is off by the size of a term, 10^5 times more."""
+import numpy as np
+import pytest
+
+from tests import gpu_util as U
+
+pytestmark = pytest.mark.gpu
+
+torch = pytest.importorskip("torch")
+
+
+@pytest.fixture(scope="module")
+def cabi():
+    assert torch.cuda.is_available()
+    from gelib_amd import cabi as c
+    c.lib()
+    return c
+
+
+def rand(shape, seed):
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    return torch.view_as_complex(torch.randn(*shape, 2, device="cuda", generator=g))
+
+
+# (leading extents, n_in, n_out): single and several tiles of output, reductions shorter and longer than one step of
+# 16 channels, row counts that are not multiples of the 64 rows of a wave, and the wide-output (gradient) shapes
+CASES = [
+    ((64,), 16, 16), ((1,), 2, 1), ((7, 3), 6, 5), ((100, 5), 256, 16), ((33, 9), 48, 16), ((130,), 34, 3),
+    ((40, 3), 64, 32), ((40, 3), 20, 24), ((17, 5), 40, 64), ((9, 7), 96, 40), ((65,), 16, 256), ((31, 3), 32, 300),
+    ((12, 9), 8, 70), ((257,), 1280, 16),
+]
+
+
+@pytest.mark.parametrize("lead,n_in,n_out", CASES)
+@pytest.mark.parametrize("adjoint", [False, True])
+def test_mix_channels(cabi, lead, n_in, n_out, adjoint):
+    x = rand(lead + (n_in,), 1)
+    w = rand((n_out, n_in) if adjoint else (n_in, n_out), 2)
+    r = torch.full(lead + (n_out,), float("nan"), dtype=torch.complex64, device="cuda")
+    cabi.part_mix_channels(r, x, w, adjoint=adjoint)
+    hx, hw = U.host(x).astype(np.complex128), U.host(w).astype(np.complex128)
+    v = hw.conj().T if adjoint else hw
+    want = hx @ v
+    tol = 1e-6 + 4 * np.finfo(np.float32).eps * (np.abs(hx) @ np.abs(v))
+    got = U.host(r)
+    assert np.isfinite(got.view(np.float32)).all()
+    err = np.abs(got - want)
+    assert (err <= tol).all(), "mix %s %d %d %s: worst error / tolerance %.2f" % (lead, n_in, n_out, adjoint, (err / tol).max())
+
+
+def test_mix_channels_rejects(cabi):
+    x = rand((8, 3), 1)
+    w = rand((3, 4), 2)
+    r = torch.empty(8, 4, dtype=torch.complex64, device="cuda")
+    with pytest.raises(cabi.GelibHipError):
+        cabi.part_mix_channels(r, x, w)     # an odd number of input channels
+    assert not cabi.mix_channels_ok(x)

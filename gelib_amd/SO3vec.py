@@ -3,6 +3,7 @@ of python/src/gelib/SO3vec.py:22-309 for the CG product path.  The products are 
 forward writes into uninitialised parts and the backward computes both gradients from a single pass over g."""
 import torch
 
+from gelib_amd.SO3weights import mix_channels
 from gelib_amd.gelib_common import backend, common_batch
 from gelib_amd.SO3part import SO3part
 
@@ -85,7 +86,7 @@ class SO3vec:
 
     def __mul__(self, y):
         """Multiply every part by the matching weight matrix of an SO3weights (python/src/gelib/SO3vec.py:174-177)."""
-        return SO3vec(*[torch.matmul(p, w) for p, w in zip(self.parts.values(), y.parts)])
+        return SO3vec(*[mix_channels(p, w) for p, w in zip(self.parts.values(), y.parts)])
 
     def CGproduct(self, y, maxl=-1):
         xparts = list(self.parts.values())

@@ -3,6 +3,7 @@ and autograd functions of python/src/gelib/SO3vecArr.py:23-401 for the CG produc
 fused launches as for SO3vec; the grid dimensions ride in the part descriptors."""
 import torch
 
+from gelib_amd.SO3weights import mix_channels
 from gelib_amd.gelib_common import backend
 from gelib_amd.SO3partArr import SO3partArr
 from gelib_amd.SO3vec import _product_fn
@@ -119,7 +120,7 @@ class SO3vecArr:
 
     def __mul__(self, y):
         """Multiply every part by the matching weight matrix of an SO3weights (python/src/gelib/SO3vec.py:174-177)."""
-        return SO3vecArr(*[torch.matmul(p, w) for p, w in zip(self.parts.values(), y.parts)])
+        return SO3vecArr(*[mix_channels(p, w) for p, w in zip(self.parts.values(), y.parts)])
 
     def CGproduct(self, y, maxl=-1):
         assert isinstance(y, SO3vecArr)

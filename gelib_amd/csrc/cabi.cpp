@@ -769,6 +769,7 @@ int gelib_hip_set_option(const char *name, int value) {
   if (!std::strncmp(name, "staged_", 7)) return staged_set_option(name, value);
   if (!std::strncmp(name, "diag6", 5)) return diag6_set_option(name, value);
   if (!std::strncmp(name, "onepair", 7)) return onepair_set_option(name, value);
+  if (!std::strncmp(name, "mix_", 4)) return mix_set_option(name, value);
   return unrolled_set_option(name, value);
 }
 

@@ -18,6 +18,7 @@
 #include <algorithm>
 #include <map>
 #include <mutex>
+#include <string>
 
 #include "cg_common.h"
 
@@ -38,16 +39,17 @@ struct MixArgs {
   int ct_total;      // tiles of 32 output floats, padded to a multiple of CTW
 };
 
-// V'[kf][col] for kf = 32 q + 16 h + j, col = 32 ct + i, stored at ((q * ct_total + ct) * 64 + lane) * 16 + j
+// V'[kf][col] for kf = 2 P q + P h + j (j < P), col = 32 ct + i, stored at ((q * ct_total + ct) * 64 + lane) * P + j:
+// P = 2^lg_p floats per lane and step, 16 for the short-step kernel and 64 for the long-step one
 __global__ void __launch_bounds__(256) pack_kernel(const float2 *w, float *vp, int n_in, int n_out, int nq, int ct_total,
-                                                   int adjoint) {
-  const long long total = (long long)nq * ct_total * 1024;
+                                                   int adjoint, int lg_p) {
+  const long long total = ((long long)nq * ct_total * 64) << lg_p;
   for (long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
        idx += (long long)gridDim.x * blockDim.x) {
-    const int j = (int)(idx & 15), lane = (int)((idx >> 4) & 63);
-    const long long tile = idx >> 10;
+    const int j = (int)(idx & ((1 << lg_p) - 1)), lane = (int)((idx >> lg_p) & 63);
+    const long long tile = idx >> (lg_p + 6);
     const int ct = (int)(tile % ct_total), q = (int)(tile / ct_total);
-    const int kf = 32 * q + 16 * (lane >> 5) + j, col = 32 * ct + (lane & 31);
+    const int kf = ((2 * q + (lane >> 5)) << lg_p) + j, col = 32 * ct + (lane & 31);
     const int c = kf >> 1, o = col >> 1;
     float v = 0.f;
     if (c < n_in && o < n_out) {
@@ -83,13 +85,18 @@ __global__ void __launch_bounds__(256) mix_kernel(const MixArgs p) {
   const float *vp = p.vp + ((long long)ct0 * 64 + lane) * 16;
   const long long vstep = (long long)p.ct_total * 1024;
 
-  f16v acc[RT][CTW];
+  // matrix instructions that add into the same registers run one after the other, so every wave keeps at least
+  // four sums going: with fewer than four tiles the reduction is dealt over NCH sums per tile, added up at the end
+  constexpr int NCH = RT * CTW >= 4 ? 1 : 4 / (RT * CTW);
+  f16v acc[RT][CTW][NCH];
 #pragma unroll
   for (int t = 0; t < RT; t++)
 #pragma unroll
     for (int c = 0; c < CTW; c++)
 #pragma unroll
-      for (int v = 0; v < 16; v++) acc[t][c][v] = 0.f;
+      for (int n = 0; n < NCH; n++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) acc[t][c][n][v] = 0.f;
 
   auto load = [&](int q, Operands<RT, CTW> &o) {
 #pragma unroll
@@ -115,7 +122,7 @@ __global__ void __launch_bounds__(256) mix_kernel(const MixArgs p) {
           for (int c = 0; c < CTW; c++) {
             const float av = e == 0 ? o.a[t][s].x : (e == 1 ? o.a[t][s].y : (e == 2 ? o.a[t][s].z : o.a[t][s].w));
             const float bv = e == 0 ? o.b[c][s].x : (e == 1 ? o.b[c][s].y : (e == 2 ? o.b[c][s].z : o.b[c][s].w));
-            acc[t][c] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv, acc[t][c], 0, 0, 0);
+            acc[t][c][e % NCH] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv, acc[t][c][e % NCH], 0, 0, 0);
           }
   };
 
@@ -144,12 +151,108 @@ __global__ void __launch_bounds__(256) mix_kernel(const MixArgs p) {
 #pragma unroll
     for (int c = 0; c < CTW; c++) {
       const int col = 32 * (ct0 + c) + i;
+      f16v sum = acc[t][c][0];
+#pragma unroll
+      for (int n = 1; n < NCH; n++) sum += acc[t][c][n];
 #pragma unroll
       for (int v = 0; v < 16; v++) {
         const long long row = row0 + 32 * t + 8 * (v / 4) + 4 * h + (v % 4);
-        if (row < p.rows && col < p.n2) p.r[row * p.rs + col] = acc[t][c][v];
+        if (row < p.rows && col < p.n2) p.r[row * p.rs + col] = sum[v];
       }
     }
+}
+
+// Long reductions (n_in of hundreds or thousands).  In the kernel above a lane is tied to a row, so one load instruction
+// touches 64 different cache lines and uses 16 B of each, and a row is visited 128 B at a time.  Here a wave of its own
+// (a 64-thread block) reads 32 rows 512 B at a time with loads whose lanes run along the row (two rows per instruction),
+// turns the tile through LDS into the layout of the matrix cores, and multiplies it while the loads of the next tile are
+// in flight.  V' arrives 16 floats per lane at a time, one group ahead of the 16 matrix instructions that use it.
+constexpr int kLongChunk = 128;            // floats of a row per step
+constexpr int kLongPitch = kLongChunk + 4; // LDS row pitch: consecutive rows start 4 banks apart
+
+template <int CTW>
+__global__ void __launch_bounds__(64, 8) mix_long_kernel(const MixArgs p) {
+  __shared__ float4 tile4[32 * kLongPitch / 4];
+  float *tile = (float *)tile4;
+  const int lane = threadIdx.x, i = lane & 31, h = lane >> 5;
+  const long long groups = (p.rows + 31) / 32;
+  const long long grp = blockIdx.x % groups;
+  const int ct0 = (int)(blockIdx.x / groups) * CTW;
+  const long long row0 = grp * 32;
+
+  // loads: instruction u covers rows 2u and 2u+1, lane (i, h) the 16 bytes at float 4 i of row 2u + h
+  long long lrow = row0 + h;
+  const float *src[16];
+#pragma unroll
+  for (int u = 0; u < 16; u++) {
+    long long row = lrow + 2 * u;
+    if (row > p.rows - 1) row = p.rows - 1;   // rows past the end repeat the last one; their results are not stored
+    src[u] = p.x + row * p.xs + 4 * i;
+  }
+  const float *vp = p.vp + ((long long)ct0 * 64 + lane) * 64;
+  const long long vstep = (long long)p.ct_total * 4096;
+
+  constexpr int NCH = CTW >= 4 ? 1 : 4 / CTW;   // sums per tile, as in the kernel above
+  f16v acc[CTW][NCH];
+#pragma unroll
+  for (int c = 0; c < CTW; c++)
+#pragma unroll
+    for (int n = 0; n < NCH; n++)
+#pragma unroll
+      for (int v = 0; v < 16; v++) acc[c][n][v] = 0.f;
+
+  float4 stage[16];
+  auto fetch = [&](int q) {
+    const bool inside = q * kLongChunk + 4 * i < p.k2;   // k2 is a multiple of 4
+#pragma unroll
+    for (int u = 0; u < 16; u++)
+      stage[u] = inside ? *(const float4 *)(src[u] + q * kLongChunk) : make_float4(0.f, 0.f, 0.f, 0.f);
+  };
+  fetch(0);
+  for (int q = 0; q < p.nq; q++) {
+    __syncthreads();   // the reads of the previous tile are over
+#pragma unroll
+    for (int u = 0; u < 16; u++) *(float4 *)(tile + (2 * u + h) * kLongPitch + 4 * i) = stage[u];
+    __syncthreads();
+    float4 a[16];
+#pragma unroll
+    for (int s = 0; s < 16; s++) a[s] = *(const float4 *)(tile + i * kLongPitch + 64 * h + 4 * s);
+    if (q + 1 < p.nq) fetch(q + 1);
+    const float *vq = vp + q * vstep;
+    float4 b[2][4];
+#pragma unroll
+    for (int s = 0; s < 4; s++) b[0][s] = *(const float4 *)(vq + 4 * s);
+#pragma unroll
+    for (int g = 0; g < 4 * CTW; g++) {   // group g: output tile g / 4, floats 16 (g % 4) .. of the lane's 64
+      if (g + 1 < 4 * CTW) {
+#pragma unroll
+        for (int s = 0; s < 4; s++)
+          b[(g + 1) & 1][s] = *(const float4 *)(vq + ((g + 1) / 4) * 4096 + 16 * ((g + 1) % 4) + 4 * s);
+      }
+#pragma unroll
+      for (int s = 0; s < 4; s++) {
+        const float4 av = a[4 * (g % 4) + s], bv = b[g & 1][s];
+        f16v *sum = acc[g / 4];
+        sum[0 % NCH] = __builtin_amdgcn_mfma_f32_32x32x2f32(av.x, bv.x, sum[0 % NCH], 0, 0, 0);
+        sum[1 % NCH] = __builtin_amdgcn_mfma_f32_32x32x2f32(av.y, bv.y, sum[1 % NCH], 0, 0, 0);
+        sum[2 % NCH] = __builtin_amdgcn_mfma_f32_32x32x2f32(av.z, bv.z, sum[2 % NCH], 0, 0, 0);
+        sum[3 % NCH] = __builtin_amdgcn_mfma_f32_32x32x2f32(av.w, bv.w, sum[3 % NCH], 0, 0, 0);
+      }
+    }
+  }
+
+#pragma unroll
+  for (int c = 0; c < CTW; c++) {
+    const int col = 32 * (ct0 + c) + i;
+    f16v sum = acc[c][0];
+#pragma unroll
+    for (int n = 1; n < NCH; n++) sum += acc[c][n];
+#pragma unroll
+    for (int v = 0; v < 16; v++) {
+      const long long row = row0 + 8 * (v / 4) + 4 * h + (v % 4);
+      if (row < p.rows && col < p.n2) p.r[row * p.rs + col] = sum[v];
+    }
+  }
 }
 
 // the packed matrix of a call lives in a buffer kept per (device, stream): calls on one stream are ordered, calls on
@@ -180,6 +283,8 @@ float *workspace(size_t bytes, hipStream_t s) {
   return w.ptr;
 }
 
+int g_mix_long = 1;
+
 template <int RT, int CTW, bool PIPE>
 void launch(const MixArgs &a, hipStream_t s) {
   const long long waves = (a.rows + 32 * RT - 1) / (32 * RT);
@@ -204,19 +309,26 @@ int launch_mix(float2 *r, const float2 *x, const float2 *w, long long rows, int 
   a.rs = 2 * rs;
   a.k2 = 2 * n_in;
   a.n2 = 2 * n_out;
-  a.nq = (a.k2 + 31) / 32;
   const int tiles = (a.n2 + 31) / 32;
+  const bool long_rows = a.k2 >= 4 * kLongChunk && g_mix_long;   // rows of 2 KB and more: the LDS-staged kernel
   const bool wide = tiles > 2;
   const int ctw = wide ? 4 : tiles;
   a.ct_total = (tiles + ctw - 1) / ctw * ctw;
-  const size_t bytes = (size_t)a.nq * a.ct_total * 1024 * sizeof(float);
-  float *vp = workspace(bytes, s);
+  const int lg_p = long_rows ? 6 : 4;
+  a.nq = (a.k2 + (2 << lg_p) - 1) / (2 << lg_p);
+  const long long total = ((long long)a.nq * a.ct_total * 64) << lg_p;
+  float *vp = workspace((size_t)total * sizeof(float), s);
   if (!vp) return 10;
   a.vp = vp;
-  const long long total = (long long)a.nq * a.ct_total * 1024;
   hipLaunchKernelGGL(pack_kernel, dim3((unsigned)std::min<long long>((total + 255) / 256, 4096)), dim3(256), 0, s, w, vp,
-                     n_in, n_out, a.nq, a.ct_total, adjoint ? 1 : 0);
-  if (!wide) {
+                     n_in, n_out, a.nq, a.ct_total, adjoint ? 1 : 0, lg_p);
+  if (long_rows) {
+    const long long blocks = (rows + 31) / 32 * (a.ct_total / ctw);
+    if (blocks > 0x7fffffffLL) return 11;
+    if (ctw == 1) hipLaunchKernelGGL(mix_long_kernel<1>, dim3((unsigned)blocks), dim3(64), 0, s, a);
+    else if (ctw == 2) hipLaunchKernelGGL(mix_long_kernel<2>, dim3((unsigned)blocks), dim3(64), 0, s, a);
+    else hipLaunchKernelGGL(mix_long_kernel<4>, dim3((unsigned)blocks), dim3(64), 0, s, a);
+  } else if (!wide) {
     if (ctw == 1) launch<2, 1, true>(a, s);
     else launch<2, 2, true>(a, s);
   } else if (a.nq <= 2) {
@@ -225,6 +337,14 @@ int launch_mix(float2 *r, const float2 *x, const float2 *w, long long rows, int 
     launch<1, 4, true>(a, s);
   }
   return hipGetLastError() == hipSuccess ? 0 : 10;
+}
+
+int mix_set_option(const char *name, int value) {   // 0, or 12 for a name that is not an option of this file
+  if (std::string(name) == "mix_long") {
+    g_mix_long = value;
+    return 0;
+  }
+  return 12;
 }
 
 }  // namespace gelib_hip

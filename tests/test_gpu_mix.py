@@ -33,6 +33,9 @@ CASES = [
     ((64,), 16, 16), ((1,), 2, 1), ((7, 3), 6, 5), ((100, 5), 256, 16), ((33, 9), 48, 16), ((130,), 34, 3),
     ((40, 3), 64, 32), ((40, 3), 20, 24), ((17, 5), 40, 64), ((9, 7), 96, 40), ((65,), 16, 256), ((31, 3), 32, 300),
     ((12, 9), 8, 70), ((257,), 1280, 16),
+    # rows of 2 KB and more run on the LDS-staged kernel: a last step that is partly outside the row, two and eight
+    # tiles of output, fewer rows than the 32 of a wave
+    ((70,), 258, 5), ((33, 3), 300, 24), ((20, 3), 260, 70), ((5,), 1024, 16), ((3, 7), 514, 128),
 ]
 
 
@@ -51,6 +54,23 @@ def test_mix_channels(cabi, lead, n_in, n_out, adjoint):
     assert np.isfinite(got.view(np.float32)).all()
     err = np.abs(got - want)
     assert (err <= tol).all(), "mix %s %d %d %s: worst error / tolerance %.2f" % (lead, n_in, n_out, adjoint, (err / tol).max())
+
+
+def test_mix_channels_long_rows_on_the_short_step_kernel(cabi):
+    x = rand((67, 3, 384), 3)
+    w = rand((384, 16), 4)
+    r0 = torch.empty(67, 3, 16, dtype=torch.complex64, device="cuda")
+    r1 = torch.empty_like(r0)
+    cabi.part_mix_channels(r0, x, w)
+    cabi.set_option("mix_long", 0)
+    try:
+        cabi.part_mix_channels(r1, x, w)
+    finally:
+        cabi.set_option("mix_long", 1)
+    want = U.host(x).astype(np.complex128) @ U.host(w).astype(np.complex128)
+    tol = 1e-6 + 4 * np.finfo(np.float32).eps * (np.abs(U.host(x)).astype(np.float64) @ np.abs(U.host(w)).astype(np.float64))
+    for r in (r0, r1):
+        assert (np.abs(U.host(r) - want) <= tol).all()
 
 
 def test_mix_channels_rejects(cabi):

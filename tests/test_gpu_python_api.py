@@ -181,3 +181,28 @@ def test_product_then_linear_layer(G):
     assert torch.allclose(net(x, y, W2).odot(test_vec) - loss, dW, rtol=1e-3, atol=1e-2)
     xeps = G.SO3vec.randn_like(x)
     assert torch.allclose(net(x + xeps, y, W).odot(test_vec) - loss, xeps.odot(x.get_grad()), rtol=1e-3, atol=1e-2)
+
+
+def test_linear_layer_runs_on_the_library_kernel_and_matches_matmul(G):
+    """SO3vec * SO3weights on the GPU: values and both gradients against torch.matmul in complex128."""
+    from gelib_amd import cabi
+    tau_in = G.SO3type({0: 24, 1: 40, 2: 256})
+    tau_out = G.SO3type({0: 16, 1: 5, 2: 48})
+    x = G.SO3vec.randn(37, tau_in, device="cuda")
+    W = G.SO3weights.randn(tau_in, tau_out, device="cuda").requires_grad_()
+    x.requires_grad_()
+    out = x * W
+    assert cabi.last_path() == 1        # the library ran, not torch.matmul
+    g = G.SO3vec.randn_like(out)
+    out.odot(g).backward()
+    for l, w in zip(tau_in, W.parts):
+        xp = x.parts[l].detach().as_subclass(torch.Tensor)
+        x64 = xp.to(torch.complex128).requires_grad_()
+        w64 = w.detach().to(torch.complex128).requires_grad_()
+        ref = torch.matmul(x64, w64)
+        assert torch.allclose(out.parts[l].detach().as_subclass(torch.Tensor).to(torch.complex128), ref.detach(), rtol=1e-4, atol=1e-3)
+        gl = g.parts[l].detach().as_subclass(torch.Tensor).to(torch.complex128)
+        # the same scalar as odot: sum of re*re + im*im
+        (torch.view_as_real(ref) * torch.view_as_real(gl)).sum().backward()
+        assert torch.allclose(x.parts[l].grad.as_subclass(torch.Tensor).to(torch.complex128), x64.grad, rtol=1e-4, atol=1e-3)
+        assert torch.allclose(w.grad.to(torch.complex128), w64.grad, rtol=1e-4, atol=2e-3)

@@ -39,17 +39,19 @@ struct MixArgs {
   int ct_total;      // tiles of 32 output floats, padded to a multiple of CTW
 };
 
-// V'[kf][col] for kf = 2 P q + P h + j (j < P), col = 32 ct + i, stored at ((q * ct_total + ct) * 64 + lane) * P + j:
+// V'[kf][col] for kf = 2 P q + P h + 4 s + e (4 s + e < P), col = 32 ct + i, stored at
+// (((q * ct_total + ct) * P / 4 + s) * 64 + lane) * 4 + e: a wave reads 1 KB in one piece per load instruction.
 // P = 2^lg_p floats per lane and step, 16 for the short-step kernel and 64 for the long-step one
 __global__ void __launch_bounds__(256) pack_kernel(const float2 *w, float *vp, int n_in, int n_out, int nq, int ct_total,
                                                    int adjoint, int lg_p) {
   const long long total = ((long long)nq * ct_total * 64) << lg_p;
   for (long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
        idx += (long long)gridDim.x * blockDim.x) {
-    const int j = (int)(idx & ((1 << lg_p) - 1)), lane = (int)((idx >> lg_p) & 63);
+    const int e = (int)(idx & 3), lane = (int)((idx >> 2) & 63);
+    const int sg = (int)((idx >> 8) & ((1 << (lg_p - 2)) - 1));
     const long long tile = idx >> (lg_p + 6);
     const int ct = (int)(tile % ct_total), q = (int)(tile / ct_total);
-    const int kf = ((2 * q + (lane >> 5)) << lg_p) + j, col = 32 * ct + (lane & 31);
+    const int kf = ((2 * q + (lane >> 5)) << lg_p) + 4 * sg + e, col = 32 * ct + (lane & 31);
     const int c = kf >> 1, o = col >> 1;
     float v = 0.f;
     if (c < n_in && o < n_out) {
@@ -82,7 +84,7 @@ __global__ void __launch_bounds__(256) mix_kernel(const MixArgs p) {
     if (row > p.rows - 1) row = p.rows - 1;   // rows past the end repeat the last one; their results are not stored
     xrow[t] = p.x + row * p.xs + 16 * h;
   }
-  const float *vp = p.vp + ((long long)ct0 * 64 + lane) * 16;
+  const float *vp = p.vp + (long long)ct0 * 1024 + lane * 4;
   const long long vstep = (long long)p.ct_total * 1024;
 
   // matrix instructions that add into the same registers run one after the other, so every wave keeps at least
@@ -109,7 +111,7 @@ __global__ void __launch_bounds__(256) mix_kernel(const MixArgs p) {
 #pragma unroll
     for (int c = 0; c < CTW; c++)
 #pragma unroll
-      for (int s = 0; s < 4; s++) o.b[c][s] = *(const float4 *)(vp + q * vstep + c * 1024 + 4 * s);
+      for (int s = 0; s < 4; s++) o.b[c][s] = *(const float4 *)(vp + q * vstep + c * 1024 + 256 * s);
   };
   auto compute = [&](const Operands<RT, CTW> &o) {
 #pragma unroll
@@ -162,96 +164,90 @@ __global__ void __launch_bounds__(256) mix_kernel(const MixArgs p) {
     }
 }
 
-// Long reductions (n_in of hundreds or thousands).  In the kernel above a lane is tied to a row, so one load instruction
-// touches 64 different cache lines and uses 16 B of each, and a row is visited 128 B at a time.  Here a wave of its own
-// (a 64-thread block) reads 32 rows 512 B at a time with loads whose lanes run along the row (two rows per instruction),
-// turns the tile through LDS into the layout of the matrix cores, and multiplies it while the loads of the next tile are
-// in flight.  V' arrives 16 floats per lane at a time, one group ahead of the 16 matrix instructions that use it.
+// Long reductions (n_in of hundreds or thousands) into one tile of output (n_out <= 16).  In the kernel above a lane
+// is tied to a row, so one load instruction touches 64 different cache lines and uses 16 B of each, and a row is visited
+// 128 B at a time.  Here a wave of its own (a 64-thread block) reads 32 rows 512 B at a time with loads whose lanes run
+// along the row (two rows per instruction) and turns the tile through LDS into the layout of the matrix cores.  The loads
+// of the next tile and of the next 64 floats per lane of V' are issued before the 64 matrix instructions of a step and
+// waited for after them; the operands of x come out of LDS four matrix instructions at a time.
 constexpr int kLongChunk = 128;            // floats of a row per step
 constexpr int kLongPitch = kLongChunk + 4; // LDS row pitch: consecutive rows start 4 banks apart
 
-template <int CTW>
 __global__ void __launch_bounds__(64, 8) mix_long_kernel(const MixArgs p) {
   __shared__ float4 tile4[32 * kLongPitch / 4];
   float *tile = (float *)tile4;
   const int lane = threadIdx.x, i = lane & 31, h = lane >> 5;
-  const long long groups = (p.rows + 31) / 32;
-  const long long grp = blockIdx.x % groups;
-  const int ct0 = (int)(blockIdx.x / groups) * CTW;
-  const long long row0 = grp * 32;
+  const long long row0 = (long long)blockIdx.x * 32;
+  const float *xbase = p.x + row0 * p.xs;
+  const long long left = p.rows - 1 - row0;
+  const int lim = left < 31 ? (int)left : 31;   // rows past the end repeat the last one; their results are not stored
+  const unsigned pitch = (unsigned)p.xs;
+  const float *vp = p.vp + lane * 4;
 
-  // loads: instruction u covers rows 2u and 2u+1, lane (i, h) the 16 bytes at float 4 i of row 2u + h
-  long long lrow = row0 + h;
-  const float *src[16];
+  f16v acc;
 #pragma unroll
-  for (int u = 0; u < 16; u++) {
-    long long row = lrow + 2 * u;
-    if (row > p.rows - 1) row = p.rows - 1;   // rows past the end repeat the last one; their results are not stored
-    src[u] = p.x + row * p.xs + 4 * i;
-  }
-  const float *vp = p.vp + ((long long)ct0 * 64 + lane) * 64;
-  const long long vstep = (long long)p.ct_total * 4096;
+  for (int v = 0; v < 16; v++) acc[v] = 0.f;
 
-  constexpr int NCH = CTW >= 4 ? 1 : 4 / CTW;   // sums per tile, as in the kernel above
-  f16v acc[CTW][NCH];
+  float4 stage[16], b0[16], b1[16];
+  // instruction u covers rows 2u and 2u+1, lane (i, h) the 16 bytes at float 4 i of row 2u + h; a chunk that starts
+  // outside the row (k2 is a multiple of 4, so it is inside or outside as a whole) is read from the row's end instead
+  // and replaced by zeros on its way into LDS
+  auto fetch_x = [&](int q) {
+    const int kf = q * kLongChunk + 4 * i;
+    const unsigned col = kf < p.k2 ? kf : p.k2 - 4;
 #pragma unroll
-  for (int c = 0; c < CTW; c++)
+    for (int u = 0; u < 16; u++) {
+      const int r = 2 * u + h < lim ? 2 * u + h : lim;
+      unsigned off = (unsigned)r * pitch + col;
+      asm volatile("" : "+v"(off));
+      stage[u] = *(const float4 *)(xbase + off);
+    }
+  };
+  auto fetch_v = [&](int q, float4 (&b)[16]) {
 #pragma unroll
-    for (int n = 0; n < NCH; n++)
-#pragma unroll
-      for (int v = 0; v < 16; v++) acc[c][n][v] = 0.f;
-
-  float4 stage[16];
-  auto fetch = [&](int q) {
-    const bool inside = q * kLongChunk + 4 * i < p.k2;   // k2 is a multiple of 4
+    for (int s = 0; s < 16; s++) b[s] = *(const float4 *)(vp + (long long)q * 4096 + 256 * s);
+  };
+  auto step = [&](int q, const float4 (&bcur)[16], float4 (&bnext)[16]) {
+    __syncthreads();   // the reads of the previous tile are over
+    const bool inside = q * kLongChunk + 4 * i < p.k2;
 #pragma unroll
     for (int u = 0; u < 16; u++)
-      stage[u] = inside ? *(const float4 *)(src[u] + q * kLongChunk) : make_float4(0.f, 0.f, 0.f, 0.f);
-  };
-  fetch(0);
-  for (int q = 0; q < p.nq; q++) {
-    __syncthreads();   // the reads of the previous tile are over
-#pragma unroll
-    for (int u = 0; u < 16; u++) *(float4 *)(tile + (2 * u + h) * kLongPitch + 4 * i) = stage[u];
+      *(float4 *)(tile + (2 * u + h) * kLongPitch + 4 * i) = inside ? stage[u] : make_float4(0.f, 0.f, 0.f, 0.f);
     __syncthreads();
-    float4 a[16];
-#pragma unroll
-    for (int s = 0; s < 16; s++) a[s] = *(const float4 *)(tile + i * kLongPitch + 64 * h + 4 * s);
-    if (q + 1 < p.nq) fetch(q + 1);
-    const float *vq = vp + q * vstep;
-    float4 b[2][4];
-#pragma unroll
-    for (int s = 0; s < 4; s++) b[0][s] = *(const float4 *)(vq + 4 * s);
-#pragma unroll
-    for (int g = 0; g < 4 * CTW; g++) {   // group g: output tile g / 4, floats 16 (g % 4) .. of the lane's 64
-      if (g + 1 < 4 * CTW) {
-#pragma unroll
-        for (int s = 0; s < 4; s++)
-          b[(g + 1) & 1][s] = *(const float4 *)(vq + ((g + 1) / 4) * 4096 + 16 * ((g + 1) % 4) + 4 * s);
-      }
-#pragma unroll
-      for (int s = 0; s < 4; s++) {
-        const float4 av = a[4 * (g % 4) + s], bv = b[g & 1][s];
-        f16v *sum = acc[g / 4];
-        sum[0 % NCH] = __builtin_amdgcn_mfma_f32_32x32x2f32(av.x, bv.x, sum[0 % NCH], 0, 0, 0);
-        sum[1 % NCH] = __builtin_amdgcn_mfma_f32_32x32x2f32(av.y, bv.y, sum[1 % NCH], 0, 0, 0);
-        sum[2 % NCH] = __builtin_amdgcn_mfma_f32_32x32x2f32(av.z, bv.z, sum[2 % NCH], 0, 0, 0);
-        sum[3 % NCH] = __builtin_amdgcn_mfma_f32_32x32x2f32(av.w, bv.w, sum[3 % NCH], 0, 0, 0);
-      }
+    if (q + 1 < p.nq) {
+      fetch_v(q + 1, bnext);
+      fetch_x(q + 1);
     }
+    const float *arow = tile + i * kLongPitch + 64 * h;
+    float4 a0 = *(const float4 *)arow, a1 = *(const float4 *)(arow + 4);
+#pragma unroll
+    for (int s = 0; s < 16; s += 2) {
+      const float4 c0 = a0, c1 = a1;
+      if (s + 2 < 16) {   // the next two operands leave LDS while these eight instructions run
+        a0 = *(const float4 *)(arow + 4 * (s + 2));
+        a1 = *(const float4 *)(arow + 4 * (s + 3));
+      }
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(c0.x, bcur[s].x, acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(c0.y, bcur[s].y, acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(c0.z, bcur[s].z, acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(c0.w, bcur[s].w, acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(c1.x, bcur[s + 1].x, acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(c1.y, bcur[s + 1].y, acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(c1.z, bcur[s + 1].z, acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(c1.w, bcur[s + 1].w, acc, 0, 0, 0);
+    }
+  };
+  fetch_v(0, b0);
+  fetch_x(0);
+  for (int q = 0; q < p.nq; q += 2) {
+    step(q, b0, b1);
+    if (q + 1 < p.nq) step(q + 1, b1, b0);
   }
 
 #pragma unroll
-  for (int c = 0; c < CTW; c++) {
-    const int col = 32 * (ct0 + c) + i;
-    f16v sum = acc[c][0];
-#pragma unroll
-    for (int n = 1; n < NCH; n++) sum += acc[c][n];
-#pragma unroll
-    for (int v = 0; v < 16; v++) {
-      const long long row = row0 + 8 * (v / 4) + 4 * h + (v % 4);
-      if (row < p.rows && col < p.n2) p.r[row * p.rs + col] = sum[v];
-    }
+  for (int v = 0; v < 16; v++) {
+    const long long row = row0 + 8 * (v / 4) + 4 * h + (v % 4);
+    if (row < p.rows && i < p.n2) p.r[row * p.rs + i] = acc[v];
   }
 }
 
@@ -310,7 +306,8 @@ int launch_mix(float2 *r, const float2 *x, const float2 *w, long long rows, int 
   a.k2 = 2 * n_in;
   a.n2 = 2 * n_out;
   const int tiles = (a.n2 + 31) / 32;
-  const bool long_rows = a.k2 >= 4 * kLongChunk && g_mix_long;   // rows of 2 KB and more: the LDS-staged kernel
+  // rows of 2 KB and more into a single tile of output: the LDS-staged kernel (32 rows must lie within 2^32 floats)
+  const bool long_rows = tiles == 1 && a.k2 >= 4 * kLongChunk && a.xs < (1LL << 26) && g_mix_long;
   const bool wide = tiles > 2;
   const int ctw = wide ? 4 : tiles;
   a.ct_total = (tiles + ctw - 1) / ctw * ctw;
@@ -323,11 +320,9 @@ int launch_mix(float2 *r, const float2 *x, const float2 *w, long long rows, int 
   hipLaunchKernelGGL(pack_kernel, dim3((unsigned)std::min<long long>((total + 255) / 256, 4096)), dim3(256), 0, s, w, vp,
                      n_in, n_out, a.nq, a.ct_total, adjoint ? 1 : 0, lg_p);
   if (long_rows) {
-    const long long blocks = (rows + 31) / 32 * (a.ct_total / ctw);
+    const long long blocks = (rows + 31) / 32;
     if (blocks > 0x7fffffffLL) return 11;
-    if (ctw == 1) hipLaunchKernelGGL(mix_long_kernel<1>, dim3((unsigned)blocks), dim3(64), 0, s, a);
-    else if (ctw == 2) hipLaunchKernelGGL(mix_long_kernel<2>, dim3((unsigned)blocks), dim3(64), 0, s, a);
-    else hipLaunchKernelGGL(mix_long_kernel<4>, dim3((unsigned)blocks), dim3(64), 0, s, a);
+    hipLaunchKernelGGL(mix_long_kernel, dim3((unsigned)blocks), dim3(64), 0, s, a);
   } else if (!wide) {
     if (ctw == 1) launch<2, 1, true>(a, s);
     else launch<2, 2, true>(a, s);

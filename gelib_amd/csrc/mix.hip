@@ -100,50 +100,67 @@ __global__ void __launch_bounds__(256) mix_kernel(const MixArgs p) {
 #pragma unroll
         for (int v = 0; v < 16; v++) acc[t][c][n][v] = 0.f;
 
+  // k2 is a multiple of 4, so a float4 of a row is inside it or outside it as a whole; one that would start outside
+  // is read from the row's end instead (no branch around a load, so loads stay in flight across the matrix
+  // instructions) and replaced by zeros when it is used
   auto load = [&](int q, Operands<RT, CTW> &o) {
 #pragma unroll
     for (int t = 0; t < RT; t++)
 #pragma unroll
       for (int s = 0; s < 4; s++) {
-        const int kf = 32 * q + 16 * h + 4 * s;   // k2 is a multiple of 4: a float4 is inside the row or outside it
-        o.a[t][s] = kf < p.k2 ? *(const float4 *)(xrow[t] + 32 * q + 4 * s) : make_float4(0.f, 0.f, 0.f, 0.f);
+        const int kf = 32 * q + 16 * h + 4 * s;
+        const int at = kf < p.k2 ? 32 * q + 4 * s : p.k2 - 4 - 16 * h;
+        o.a[t][s] = *(const float4 *)(xrow[t] + at);
       }
 #pragma unroll
     for (int c = 0; c < CTW; c++)
 #pragma unroll
       for (int s = 0; s < 4; s++) o.b[c][s] = *(const float4 *)(vp + q * vstep + c * 1024 + 256 * s);
   };
-  auto compute = [&](const Operands<RT, CTW> &o) {
+  auto compute = [&](int q, const Operands<RT, CTW> &o) {
 #pragma unroll
-    for (int s = 0; s < 4; s++)
+    for (int s = 0; s < 4; s++) {
+      const bool inside = 32 * q + 16 * h + 4 * s < p.k2;
 #pragma unroll
       for (int e = 0; e < 4; e++)
 #pragma unroll
         for (int t = 0; t < RT; t++)
 #pragma unroll
           for (int c = 0; c < CTW; c++) {
-            const float av = e == 0 ? o.a[t][s].x : (e == 1 ? o.a[t][s].y : (e == 2 ? o.a[t][s].z : o.a[t][s].w));
+            const float ar = e == 0 ? o.a[t][s].x : (e == 1 ? o.a[t][s].y : (e == 2 ? o.a[t][s].z : o.a[t][s].w));
+            const float av = inside ? ar : 0.f;
             const float bv = e == 0 ? o.b[c][s].x : (e == 1 ? o.b[c][s].y : (e == 2 ? o.b[c][s].z : o.b[c][s].w));
             acc[t][c][e % NCH] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv, acc[t][c][e % NCH], 0, 0, 0);
           }
+    }
   };
 
   if (PIPE) {
     Operands<RT, CTW> o0, o1;
     load(0, o0);
-    for (int q = 0; q < p.nq; q += 2) {
-      if (q + 1 < p.nq) load(q + 1, o1);
-      compute(o0);
-      if (q + 1 < p.nq) {
-        if (q + 2 < p.nq) load(q + 2, o0);
-        compute(o1);
-      }
+    int q = 0;
+    for (; q + 2 < p.nq; q += 2) {   // no branch inside: the waits count exactly the loads issued after the ones needed
+      load(q + 1, o1);
+      __builtin_amdgcn_sched_barrier(0);   // keep the loads ahead of the matrix instructions of the other buffer
+      compute(q, o0);
+      __builtin_amdgcn_sched_barrier(0);
+      load(q + 2, o0);
+      __builtin_amdgcn_sched_barrier(0);
+      compute(q + 1, o1);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    if (q + 1 < p.nq) {
+      load(q + 1, o1);
+      compute(q, o0);
+      compute(q + 1, o1);
+    } else {
+      compute(q, o0);
     }
   } else {
     Operands<RT, CTW> o0;
     for (int q = 0; q < p.nq; q++) {
       load(q, o0);
-      compute(o0);
+      compute(q, o0);
     }
   }
 

@@ -1,9 +1,9 @@
 """SO3weights / SO3linear: the channel-mixing linear layer that consumes a product
 (python/src/gelib/SO3weights.py:22-85; SO3vec.__mul__, python/src/gelib/SO3vec.py:174-177).  One complex
 (n_in, n_out) matrix per l, applied to the channel index of every part.  The reference does this with torch.matmul; on
-the GPU the product of a part with its matrix, and the gradient with respect to the part, run on the library's
-matrix-core kernel for tall, skinny complex matrices (mix_channels below); the gradient with respect to the matrix and
-tensors on the host stay with torch."""
+the GPU the product of a part with its matrix and the gradient with respect to the part run on the library's
+matrix-core kernels for tall, skinny complex matrices (mix_channels below), as does the gradient with respect to the
+matrix; tensors on the host stay with torch."""
 import torch
 
 from gelib_amd.SO3type import SO3type
@@ -33,7 +33,8 @@ class MixChannelsFn(torch.autograd.Function):
             else:
                 gx = torch.matmul(g, w.conj().transpose(0, 1))
         if ctx.needs_input_grad[1]:
-            gw = torch.matmul(x.reshape(-1, x.shape[-1]).conj().transpose(0, 1), g.reshape(-1, g.shape[-1]))
+            gw = torch.empty_like(w)
+            cabi.part_mix_channels_wgrad(gw, x, g)
         return gx, gw
 
 

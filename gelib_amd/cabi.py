@@ -17,7 +17,7 @@ SYMBOLS = [
     "gelib_hip_so3part_diagcg_fwd", "gelib_hip_so3part_diagcg_back0", "gelib_hip_so3part_diagcg_back1",
     "gelib_hip_so3vec_cg_fwd", "gelib_hip_so3vec_cg_bwd", "gelib_hip_so3vec_diagcg_fwd",
     "gelib_hip_so3vec_diagcg_bwd", "gelib_hip_so3part_spharm", "gelib_hip_gather_map_create",
-    "gelib_hip_gather_map_destroy", "gelib_hip_part_gather", "gelib_hip_part_mix_channels", "gelib_hip_set_option", "gelib_hip_last_path",
+    "gelib_hip_gather_map_destroy", "gelib_hip_part_gather", "gelib_hip_part_mix_channels", "gelib_hip_part_mix_channels_wgrad", "gelib_hip_set_option", "gelib_hip_last_path",
     "gelib_hip_malloc", "gelib_hip_free", "gelib_hip_memcpy", "gelib_hip_memset", "gelib_hip_synchronize",
 ]
 
@@ -71,6 +71,9 @@ def lib():
         L.gelib_hip_part_mix_channels.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64,
                                                   ctypes.c_int, ctypes.c_int, ctypes.c_int64, ctypes.c_int64,
                                                   ctypes.c_int, ctypes.c_void_p]
+        L.gelib_hip_part_mix_channels_wgrad.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+                                                        ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.c_int64,
+                                                        ctypes.c_int64, ctypes.c_void_p]
         L.gelib_hip_set_option.argtypes = [ctypes.c_char_p, ctypes.c_int]
         _lib = L
     return _lib
@@ -234,6 +237,18 @@ def part_mix_channels(r, x, w, adjoint=False):
     rows = x.numel() // n_in if n_in else 0
     check(lib().gelib_hip_part_mix_channels(r.data_ptr(), x.data_ptr(), w.data_ptr(), rows, n_in, n_out, n_out, n_in,
                                             int(adjoint), _stream(r)))
+
+
+def part_mix_channels_wgrad(wg, x, g):
+    """wg (n_in, n_out) = sum over the leading indices of conj(x[..., c]) g[..., o] for contiguous complex64 tensors."""
+    n_in, n_out = x.shape[-1], g.shape[-1]
+    if tuple(wg.shape) != (n_in, n_out) or g.shape[:-1] != x.shape[:-1]:
+        raise ValueError("shapes of wg, x and g do not fit")
+    if not (wg.is_contiguous() and x.is_contiguous() and g.is_contiguous()):
+        raise ValueError("contiguous tensors are needed")
+    rows = x.numel() // n_in if n_in else 0
+    check(lib().gelib_hip_part_mix_channels_wgrad(wg.data_ptr(), x.data_ptr(), g.data_ptr(), rows, n_in, n_out, n_in,
+                                                  n_out, _stream(wg)))
 
 
 def set_option(name, value):

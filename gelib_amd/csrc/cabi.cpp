@@ -726,6 +726,26 @@ int gelib_hip_part_mix_channels(void *r, const void *x, const void *w, int64_t r
   return rc == 11 ? GELIB_HIP_ERR_ARG : rc;
 }
 
+int gelib_hip_part_mix_channels_wgrad(void *wg, const void *x, const void *g, int64_t rows, int n_in, int n_out,
+                                      int64_t x_row_stride, int64_t g_row_stride, void *stream) {
+  t_last_path = kPathNone;
+  if (rows < 0 || n_in < 0 || n_out < 0 || x_row_stride < n_in || g_row_stride < n_out) return GELIB_HIP_ERR_ARG;
+  if (n_in == 0 || n_out == 0) return GELIB_HIP_OK;
+  if (!wg || (rows > 0 && (!x || !g))) return GELIB_HIP_ERR_NULL;
+  if ((n_in & 1) || (x_row_stride & 1) || ((uintptr_t)x & 15) || rows > (1LL << 38)) return GELIB_HIP_ERR_ARG;
+  const int64_t xd[5] = {rows, 1, 1, 1, n_in}, xst[5] = {x_row_stride, 0, 0, 0, 1};
+  const int64_t gd[5] = {rows, 1, 1, 1, n_out}, gst[5] = {g_row_stride, 0, 0, 0, 1};
+  const int64_t wd[5] = {n_in, 1, 1, 1, n_out}, wst[5] = {n_out, 0, 0, 0, 1};
+  int rc;
+  if ((rc = check_range(wg, wd, wst, 2 * sizeof(float))) || (rc = check_range(x, xd, xst, 2 * sizeof(float))) ||
+      (rc = check_range(g, gd, gst, 2 * sizeof(float))))
+    return rc;
+  t_last_path = kPathGeneric;
+  rc = launch_mix_wgrad((float2 *)wg, (const float2 *)x, (const float2 *)g, rows, n_in, n_out, x_row_stride,
+                        g_row_stride, (hipStream_t)stream);
+  return rc == 11 ? GELIB_HIP_ERR_ARG : rc;
+}
+
 int gelib_hip_malloc(void **ptr, uint64_t bytes) {
   if (!ptr) return GELIB_HIP_ERR_NULL;
   *ptr = nullptr;

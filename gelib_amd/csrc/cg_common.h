@@ -63,6 +63,9 @@ int launch_gather(float2 *r, const float2 *x, const long long rs[5], const long 
 // strides in complex elements.  Returns 0, 10 (a HIP call failed) or 11 (n_in odd or rows of x not 16-byte aligned)
 int launch_mix(float2 *r, const float2 *x, const float2 *w, long long rows, int n_in, int n_out, long long xs,
                long long rs, bool adjoint, hipStream_t s);
+// wg (n_in, n_out) = sum over the rows of conj(x[row, :])^T g[row, :]
+int launch_mix_wgrad(float2 *wg, const float2 *x, const float2 *g, long long rows, int n_in, int n_out, long long xs,
+                     long long gs, hipStream_t s);
 int mix_set_option(const char *name, int value);   // "mix_long": 0 keeps long rows off the LDS-staged kernel
 
 }  // namespace gelib_hip

@@ -351,6 +351,186 @@ int launch_mix(float2 *r, const float2 *x, const float2 *w, long long rows, int 
   return hipGetLastError() == hipSuccess ? 0 : 10;
 }
 
+// ---- gradient with respect to the matrix:  wg[c, o] = sum_rows conj(x[row, c]) g[row, o] ----------------------------------
+// The reduction runs over the rows, hundreds of thousands of them, and the result is small.  In real terms
+// D[kf][jf] = sum_rows xf[row][kf] gf[row][jf] over the floats of x and g as they lie in memory, and
+// wg[c, o] = (D[2c][2o] + D[2c+1][2o+1]) + i (D[2c][2o+1] - D[2c+1][2o]).  One matrix instruction takes two rows:
+// lane (i, h) supplies xf[row + h][.] and gf[row + h][.].  A lane loads EW consecutive floats of its row of x in one
+// piece (the 64 lanes read 128 EW bytes of each of the two rows) and feeds them to EW instructions that add into EW
+// separate 32 x 32 sums, so sum e of lane row i stands for kf = kf0 + EW i + e.  A wave owns 32 EW floats of x, JT
+// tiles of 32 floats of g and a range of rows; the sums of the ranges go to a scratch array and a second kernel adds
+// them in a fixed order and forms the complex result (no atomics: the result does not depend on timing).
+struct WgradArgs {
+  const float *x, *g;
+  float *part;   // [nranges][k2][32 jt_total]
+  long long rows, xs, gs, rows_per_range;
+  int k2, n2, kgroups, jt_total;
+};
+
+template <int EW>
+struct FloatVec;
+template <>
+struct FloatVec<4> { typedef float4 type; };
+template <>
+struct FloatVec<2> { typedef float2 type; };
+
+template <int EW, int JT, int U>
+struct WgradStage {
+  typename FloatVec<EW>::type xv[U];
+  float gv[U][JT];
+};
+
+template <int EW, int JT, int U>
+__global__ void __launch_bounds__(64) wgrad_kernel(const WgradArgs p) {
+  typedef typename FloatVec<EW>::type vec;
+  const int lane = threadIdx.x, i = lane & 31, h = lane >> 5;
+  const int kg = blockIdx.x % p.kgroups;
+  const long long rr = blockIdx.x / p.kgroups;
+  const int jt0 = blockIdx.y * JT;
+  const int kf0 = kg * 32 * EW;
+  int col = kf0 + EW * i;
+  if (col > p.k2 - EW) col = p.k2 - EW;   // k2 is a multiple of 4: sums of columns past the end are not stored
+  int jcol[JT];
+#pragma unroll
+  for (int c = 0; c < JT; c++) {
+    jcol[c] = 32 * (jt0 + c) + i;
+    if (jcol[c] > p.n2 - 1) jcol[c] = p.n2 - 1;
+  }
+  const long long r_begin = rr * p.rows_per_range;
+  long long r_end = r_begin + p.rows_per_range;
+  if (r_end > p.rows) r_end = p.rows;
+  const float *xp = p.x + col;
+
+  f16v acc[JT][EW];
+#pragma unroll
+  for (int c = 0; c < JT; c++)
+#pragma unroll
+    for (int e = 0; e < EW; e++)
+#pragma unroll
+      for (int v = 0; v < 16; v++) acc[c][e][v] = 0.f;
+
+  // a row past the end of the range is read as the last row of the part and its g is replaced by zero when it is used
+  auto load = [&](long long step, WgradStage<EW, JT, U> &st) {
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+      long long row = r_begin + step * (2 * U) + 2 * u + h;
+      if (row > p.rows - 1) row = p.rows - 1;
+      st.xv[u] = *(const vec *)(xp + row * p.xs);
+#pragma unroll
+      for (int c = 0; c < JT; c++) st.gv[u][c] = p.g[row * p.gs + jcol[c]];
+    }
+  };
+  auto compute = [&](long long step, const WgradStage<EW, JT, U> &st) {
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+      const bool valid = r_begin + step * (2 * U) + 2 * u + h < r_end;
+#pragma unroll
+      for (int c = 0; c < JT; c++) {
+        const float gv = valid ? st.gv[u][c] : 0.f;
+        if constexpr (EW == 4) {
+          acc[c][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(st.xv[u].x, gv, acc[c][0], 0, 0, 0);
+          acc[c][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(st.xv[u].y, gv, acc[c][1], 0, 0, 0);
+          acc[c][2] = __builtin_amdgcn_mfma_f32_32x32x2f32(st.xv[u].z, gv, acc[c][2], 0, 0, 0);
+          acc[c][3] = __builtin_amdgcn_mfma_f32_32x32x2f32(st.xv[u].w, gv, acc[c][3], 0, 0, 0);
+        } else {
+          acc[c][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(st.xv[u].x, gv, acc[c][0], 0, 0, 0);
+          acc[c][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(st.xv[u].y, gv, acc[c][1], 0, 0, 0);
+        }
+      }
+    }
+  };
+
+  const long long nsteps = (r_end - r_begin + 2 * U - 1) / (2 * U);
+  WgradStage<EW, JT, U> s0, s1;
+  load(0, s0);
+  long long q = 0;
+  for (; q + 2 < nsteps; q += 2) {   // no branch inside, and fences: the next step's loads stay ahead of these sums
+    load(q + 1, s1);
+    __builtin_amdgcn_sched_barrier(0);
+    compute(q, s0);
+    __builtin_amdgcn_sched_barrier(0);
+    load(q + 2, s0);
+    __builtin_amdgcn_sched_barrier(0);
+    compute(q + 1, s1);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  if (q + 1 < nsteps) {
+    load(q + 1, s1);
+    compute(q, s0);
+    compute(q + 1, s1);
+  } else {
+    compute(q, s0);
+  }
+
+  // register v of a sum holds row 8 (v / 4) + 4 h + (v % 4) of the 32 x 32 tile, column i
+  const long long pitch = 32LL * p.jt_total;
+  float *out = p.part + rr * p.k2 * pitch;
+#pragma unroll
+  for (int c = 0; c < JT; c++)
+#pragma unroll
+    for (int e = 0; e < EW; e++)
+#pragma unroll
+      for (int v = 0; v < 16; v++) {
+        const int kf = kf0 + EW * (8 * (v / 4) + 4 * h + (v % 4)) + e;
+        if (kf < p.k2) out[kf * pitch + 32 * (jt0 + c) + i] = acc[c][e][v];
+      }
+}
+
+__global__ void __launch_bounds__(256) wgrad_sum_kernel(const float *part, float2 *wg, int n_in, int n_out, int nranges,
+                                                        long long pitch) {
+  const long long total = (long long)n_in * n_out;
+  for (long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+       idx += (long long)gridDim.x * blockDim.x) {
+    const int o = (int)(idx % n_out);
+    const long long c = idx / n_out;
+    float re = 0.f, im = 0.f;
+    for (int r = 0; r < nranges; r++) {
+      const float *d = part + ((long long)r * 2 * n_in + 2 * c) * pitch + 2 * o;
+      re += d[0] + d[pitch + 1];
+      im += d[1] - d[pitch];
+    }
+    wg[idx] = make_float2(re, im);
+  }
+}
+
+// 0, 10 or 11 as launch_mix
+int launch_mix_wgrad(float2 *wg, const float2 *x, const float2 *g, long long rows, int n_in, int n_out, long long xs,
+                     long long gs, hipStream_t s) {
+  if (n_in == 0 || n_out == 0) return 0;
+  if ((n_in & 1) || (xs & 1) || ((uintptr_t)x & 15) || rows > (1LL << 38)) return 11;
+  if (rows == 0) return hipMemsetAsync(wg, 0, sizeof(float2) * (size_t)n_in * n_out, s) == hipSuccess ? 0 : 10;
+  WgradArgs a;
+  a.x = (const float *)x;
+  a.g = (const float *)g;
+  a.rows = rows;
+  a.xs = 2 * xs;
+  a.gs = 2 * gs;
+  a.k2 = 2 * n_in;
+  a.n2 = 2 * n_out;
+  const int tiles = (a.n2 + 31) / 32;
+  const int ew = tiles <= 2 ? 4 : 2, jt = tiles == 1 ? 1 : (tiles == 2 ? 2 : 4), u = tiles == 1 ? 16 : 8;
+  a.jt_total = (tiles + jt - 1) / jt * jt;
+  a.kgroups = (a.k2 + 32 * ew - 1) / (32 * ew);
+  // enough waves to fill the chip a few times over, every range a whole number of steps and not empty
+  const long long waves_per_range = (long long)a.kgroups * (a.jt_total / jt);
+  long long nranges = std::max<long long>(1, std::min<long long>(4096 / waves_per_range, rows / (8LL * u)));
+  nranges = std::min<long long>(nranges, 256);
+  a.rows_per_range = ((rows + nranges - 1) / nranges + 2 * u - 1) / (2 * u) * (2 * u);
+  nranges = (rows + a.rows_per_range - 1) / a.rows_per_range;
+  const long long pitch = 32LL * a.jt_total;
+  float *part = workspace((size_t)nranges * a.k2 * pitch * sizeof(float), s);
+  if (!part) return 10;
+  a.part = part;
+  const dim3 grid((unsigned)(nranges * a.kgroups), (unsigned)(a.jt_total / jt));
+  if (tiles == 1) hipLaunchKernelGGL((wgrad_kernel<4, 1, 16>), grid, dim3(64), 0, s, a);
+  else if (tiles == 2) hipLaunchKernelGGL((wgrad_kernel<4, 2, 8>), grid, dim3(64), 0, s, a);
+  else hipLaunchKernelGGL((wgrad_kernel<2, 4, 8>), grid, dim3(64), 0, s, a);
+  const long long total = (long long)n_in * n_out;
+  hipLaunchKernelGGL(wgrad_sum_kernel, dim3((unsigned)std::min<long long>((total + 255) / 256, 4096)), dim3(256), 0, s,
+                     part, wg, n_in, n_out, (int)nranges, pitch);
+  return hipGetLastError() == hipSuccess ? 0 : 10;
+}
+
 int mix_set_option(const char *name, int value) {   // 0, or 12 for a name that is not an option of this file
   if (std::string(name) == "mix_long") {
     g_mix_long = value;

@@ -142,6 +142,12 @@ int gelib_hip_so3part_spharm(const gelib_part_desc *r, const float *x, const int
  * GELIB_HIP_ERR_ARG).  The re-packed matrix is kept in a buffer per (device, stream) that grows on demand. */
 int gelib_hip_part_mix_channels(void *r, const void *x, const void *w, int64_t rows, int n_in, int n_out,
                                 int64_t r_row_stride, int64_t x_row_stride, int adjoint, void *stream);
+/* wg[c, o] = sum over the rows of conj(x[row, c]) g[row, o], overwriting the row-major (n_in, n_out) matrix wg: the
+ * gradient of the same matmul with respect to W (torch's autograd forms it in the reference).  Same conditions on
+ * n_in and x.  The rows are summed in ranges whose partial sums are added in a fixed order: the result does not depend
+ * on timing.  The partial sums live in the same per-(device, stream) buffer. */
+int gelib_hip_part_mix_channels_wgrad(void *wg, const void *x, const void *g, int64_t rows, int n_in, int n_out,
+                                      int64_t x_row_stride, int64_t g_row_stride, void *stream);
 
 /* ---- gather: sums of slices along the batch or a grid dimension ---------------------------------------------------------
  * A gather map is a list of (source, target) pairs with 0 <= source < n_in, 0 <= target < n_out (the arguments of

@@ -56,6 +56,34 @@ def test_mix_channels(cabi, lead, n_in, n_out, adjoint):
     assert (err <= tol).all(), "mix %s %d %d %s: worst error / tolerance %.2f" % (lead, n_in, n_out, adjoint, (err / tol).max())
 
 
+WGRAD_CASES = [
+    ((64,), 16, 16), ((1,), 2, 1), ((7, 3), 6, 5), ((1000, 5), 256, 16), ((33, 9), 48, 16), ((130,), 34, 3),
+    ((400, 3), 64, 32), ((40, 3), 20, 24), ((170, 5), 40, 64), ((9, 7), 96, 40), ((650,), 16, 256), ((31, 3), 32, 70),
+    ((5000,), 130, 16), ((2, 2049), 8, 8),
+]
+
+
+@pytest.mark.parametrize("lead,n_in,n_out", WGRAD_CASES)
+def test_mix_channels_wgrad(cabi, lead, n_in, n_out):
+    """wg = sum over the rows of conj(x)^T g.  Tolerance as above, against the size of the sum: the partial sums of the
+    row ranges are float32 and are added in float32."""
+    x = rand(lead + (n_in,), 5)
+    g = rand(lead + (n_out,), 6)
+    wg = torch.full((n_in, n_out), float("nan"), dtype=torch.complex64, device="cuda")
+    cabi.part_mix_channels_wgrad(wg, x, g)
+    hx = U.host(x).astype(np.complex128).reshape(-1, n_in)
+    hg = U.host(g).astype(np.complex128).reshape(-1, n_out)
+    want = hx.conj().T @ hg
+    tol = 1e-6 + 4 * np.finfo(np.float32).eps * (np.abs(hx).T @ np.abs(hg))
+    got = U.host(wg)
+    assert np.isfinite(got.view(np.float32)).all()
+    err = np.abs(got - want)
+    assert (err <= tol).all(), "wgrad %s %d %d: worst error / tolerance %.2f" % (lead, n_in, n_out, (err / tol).max())
+    wg2 = torch.empty_like(wg)
+    cabi.part_mix_channels_wgrad(wg2, x, g)
+    assert torch.equal(torch.view_as_real(wg), torch.view_as_real(wg2))     # fixed summation order
+
+
 def test_mix_channels_long_rows_on_the_short_step_kernel(cabi):
     x = rand((67, 3, 384), 3)
     w = rand((384, 16), 4)

@@ -124,12 +124,14 @@ def cpu_baseline(torch, xs, ys, gs, rs, xgs, ygs, maxl, diag, nsample):
     return nsample / dt, dt, parity, {"value": nsample / dt_all, "unit": "samples/s", "cores": nth}
 
 
-AUX_WORKLOADS = ("spharm_l4_n16_B1048576", "gather_l2_n16_cells262144_deg8")
+AUX_WORKLOADS = ("spharm_l4_n16_B1048576", "gather_l2_n16_cells262144_deg8", "linear_l4_3840to16_B32768")
 
 
 def aux_bench(torch, args, name):
-    """The two kernels either side of the product: the producer of y (spherical harmonics) and the sum of cells
-    that precedes it in message passing (gather).  Same JSON shape; a step is one launch."""
+    """The kernels either side of the product: the producer of y (spherical harmonics), the sum of cells that precedes
+    it in message passing (gather), and the linear layer that consumes it (the l = 4 part of the L = 4 product, 3840
+    channels, mixed down to 16: forward, gradient of the part, gradient of the matrix).  Same JSON shape; a step is one
+    launch (three for the linear layer)."""
     import numpy as np
     from gelib_amd import cabi
     from oracle import cg_oracle as ora
@@ -149,6 +151,37 @@ def aux_bench(torch, args, name):
             return ns * n / (time.perf_counter() - t0), want, r[:ns].cpu().numpy()
         sample = "first %d of the batch" % ns
         tol = dict(rtol=1e-5, atol=1e-6)
+    elif name.startswith("linear"):
+        l, n_in, n_out, B = 4, 3840, 16, args.batch or 32768
+        gd = torch.Generator(device=dev).manual_seed(78)
+        X = torch.view_as_complex(torch.randn(B, 2 * l + 1, n_in, 2, device=dev, generator=gd))
+        G = torch.view_as_complex(torch.randn(B, 2 * l + 1, n_out, 2, device=dev, generator=gd))
+        W = torch.view_as_complex(torch.randn(n_in, n_out, 2, device=dev, generator=gd))
+        r = torch.empty(B, 2 * l + 1, n_out, dtype=torch.complex64, device=dev)
+        xg = torch.empty_like(X)
+        wg = torch.empty_like(W)
+
+        def step():
+            cabi.part_mix_channels(r, X, W)
+            cabi.part_mix_channels(xg, G, W, adjoint=True)
+            cabi.part_mix_channels_wgrad(wg, X, G)
+        rows = B * (2 * l + 1)
+        # x is read twice and its gradient written once; the narrow tensors and the matrix are read or written once
+        # per kernel that touches them
+        nbytes = 8 * (3 * rows * n_in + 3 * rows * n_out + 3 * n_in * n_out)
+        units, unit = B, "samples/s"
+        ns = min(B, 256)
+
+        def cpu():
+            hx, hw = X[:ns].cpu().numpy(), W.cpu().numpy()
+            hg = G[:ns].cpu().numpy()
+            t0 = time.perf_counter()
+            want = hx @ hw
+            _ = hg @ hw.conj().T
+            _ = hx.reshape(-1, n_in).conj().T @ hg.reshape(-1, n_out)
+            return ns / (time.perf_counter() - t0), want, r[:ns].cpu().numpy()
+        sample = "first %d samples, numpy complex64 matmuls (what the reference's torch.matmul does on the host)" % ns
+        tol = dict(rtol=1e-4, atol=2e-3)   # sums of 7680 float32 terms of size 1
     else:
         l, n, N, deg = 2, 16, args.batch or 262144, 8
         rng = np.random.default_rng(5)

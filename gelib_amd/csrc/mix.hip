@@ -37,6 +37,7 @@ struct MixArgs {
   int n2;            // 2 n_out
   int nq;            // ceil(k2 / 32)
   int ct_total;      // tiles of 32 output floats, padded to a multiple of CTW
+  int wide_store;    // rows of r are 16-byte aligned and n2 is a multiple of 4: results leave through LDS, 512 B a row
 };
 
 // V'[kf][col] for kf = 2 P q + P h + 4 s + e (4 s + e < P), col = 32 ct + i, stored at
@@ -75,7 +76,8 @@ __global__ void __launch_bounds__(256) mix_kernel(const MixArgs p) {
   const int lane = threadIdx.x & 63, i = lane & 31, h = lane >> 5;
   const long long wave = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
   const long long row0 = wave * (32 * RT);
-  if (row0 >= p.rows) return;
+  constexpr bool kWide = !PIPE && CTW == 4;   // the variant for short reductions into many tiles (gradient of a part)
+  if (row0 >= p.rows && !(kWide && p.wide_store)) return;   // with wide stores every wave reaches the barriers below
   const int ct0 = blockIdx.y * CTW;
   const float *xrow[RT];
 #pragma unroll
@@ -165,6 +167,32 @@ __global__ void __launch_bounds__(256) mix_kernel(const MixArgs p) {
   }
 
   // register v of the 32 x 32 result holds row 8 (v / 4) + 4 h + (v % 4), column i
+  if constexpr (kWide) {
+    // Straight from the registers a store instruction covers two rows of 128 B.  Through LDS the 32 x 128 floats of a
+    // row tile leave as two rows of 512 B per instruction.
+    constexpr int kPitch = 128;   // four waves: 64 KB in all
+    __shared__ float4 out4[4][32 * kPitch / 4];
+    if (p.wide_store) {
+      float *tile = (float *)out4[threadIdx.x >> 6];
+#pragma unroll
+      for (int t = 0; t < RT; t++) {
+        if (t > 0) __syncthreads();
+#pragma unroll
+        for (int c = 0; c < CTW; c++)
+#pragma unroll
+          for (int v = 0; v < 16; v++) tile[(8 * (v / 4) + 4 * h + (v % 4)) * kPitch + 32 * c + i] = acc[t][c][0][v];
+        __syncthreads();
+        const int col = 32 * ct0 + 4 * i;
+#pragma unroll
+        for (int u = 0; u < 16; u++) {
+          const long long row = row0 + 32 * t + 2 * u + h;
+          const float4 v = *(const float4 *)(tile + (2 * u + h) * kPitch + 4 * i);
+          if (row < p.rows && col < p.n2) *(float4 *)(p.r + row * p.rs + col) = v;
+        }
+      }
+      return;
+    }
+  }
 #pragma unroll
   for (int t = 0; t < RT; t++)
 #pragma unroll
@@ -297,6 +325,7 @@ float *workspace(size_t bytes, hipStream_t s) {
 }
 
 int g_mix_long = 1;
+int g_mix_wide_store = 1;
 
 template <int RT, int CTW, bool PIPE>
 void launch(const MixArgs &a, hipStream_t s) {
@@ -322,6 +351,7 @@ int launch_mix(float2 *r, const float2 *x, const float2 *w, long long rows, int 
   a.rs = 2 * rs;
   a.k2 = 2 * n_in;
   a.n2 = 2 * n_out;
+  a.wide_store = (n_out % 2 == 0 && rs % 2 == 0 && ((uintptr_t)r & 15) == 0) ? g_mix_wide_store : 0;
   const int tiles = (a.n2 + 31) / 32;
   // rows of 2 KB and more into a single tile of output: the LDS-staged kernel (32 rows must lie within 2^32 floats)
   const bool long_rows = tiles == 1 && a.k2 >= 4 * kLongChunk && a.xs < (1LL << 26) && g_mix_long;
@@ -534,6 +564,10 @@ int launch_mix_wgrad(float2 *wg, const float2 *x, const float2 *g, long long row
 int mix_set_option(const char *name, int value) {   // 0, or 12 for a name that is not an option of this file
   if (std::string(name) == "mix_long") {
     g_mix_long = value;
+    return 0;
+  }
+  if (std::string(name) == "mix_wide_store") {
+    g_mix_wide_store = value;
     return 0;
   }
   return 12;

@@ -36,6 +36,8 @@ CASES = [
     # rows of 2 KB and more run on the LDS-staged kernel: a last step that is partly outside the row, two and eight
     # tiles of output, fewer rows than the 32 of a wave
     ((70,), 258, 5), ((33, 3), 300, 24), ((20, 3), 260, 70), ((5,), 1024, 16), ((3, 7), 514, 128),
+    # many tiles of output: an odd number of output channels keeps the stores narrow, an even one sends them through LDS
+    ((50,), 8, 35), ((333,), 16, 130), ((260,), 16, 64),
 ]
 
 
@@ -99,6 +101,20 @@ def test_mix_channels_long_rows_on_the_short_step_kernel(cabi):
     tol = 1e-6 + 4 * np.finfo(np.float32).eps * (np.abs(U.host(x)).astype(np.float64) @ np.abs(U.host(w)).astype(np.float64))
     for r in (r0, r1):
         assert (np.abs(U.host(r) - want) <= tol).all()
+
+
+def test_mix_channels_wide_and_narrow_stores_agree(cabi):
+    x = rand((77, 5, 16), 7)
+    w = rand((200, 16), 8)
+    r0 = torch.empty(77, 5, 200, dtype=torch.complex64, device="cuda")
+    r1 = torch.empty_like(r0)
+    cabi.part_mix_channels(r0, x, w, adjoint=True)
+    cabi.set_option("mix_wide_store", 0)
+    try:
+        cabi.part_mix_channels(r1, x, w, adjoint=True)
+    finally:
+        cabi.set_option("mix_wide_store", 1)
+    assert torch.equal(torch.view_as_real(r0), torch.view_as_real(r1))
 
 
 def test_mix_channels_rejects(cabi):

@@ -296,6 +296,120 @@ __global__ void __launch_bounds__(64, 8) mix_long_kernel(const MixArgs p) {
   }
 }
 
+// Short reductions (n_in <= 16, one step) into many tiles of output: the gradient of a part after a layer that mixed it
+// down to 16 channels.  The work is all in the stores.  A wave of its own keeps its 64 rows of x in registers and walks
+// along the output 64 floats (two tiles) at a time: the next two tiles of V' are fetched while the 64 matrix
+// instructions of this pair run, and the 64 x 64 results leave through LDS as four rows of 256 B per store instruction.
+constexpr int kWidePitch = 64 + 4;
+
+struct WideArgs {
+  MixArgs m;
+  int pairs;            // pairs of output tiles (ct_total / 2)
+  int parts;            // waves per 64 rows
+};
+
+// The block is one wave and LDS serves the instructions of a wave in the order they were issued, so a write of one lane
+// followed by a read of another needs no barrier instruction -- only that the compiler keeps the order.  A real barrier
+// would also wait for every store in flight (the compiler drains all memory counters in front of one), and the
+// stores are what this kernel is made of.
+__device__ __forceinline__ void wave_sync() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+__global__ void __launch_bounds__(64, 8) mix_wide_kernel(const WideArgs w) {
+  const MixArgs &p = w.m;
+  __shared__ float4 tile4[64 * kWidePitch / 4];
+  float *tile = (float *)tile4;
+  const int lane = threadIdx.x, i = lane & 31, h = lane >> 5;
+  const int part = blockIdx.x % w.parts;
+  const long long row0 = (long long)(blockIdx.x / w.parts) * 64;
+  // the waves of one group of rows take the pairs of tiles in turn (wave `part` takes pairs part, part + parts, ...):
+  // they start together, so at any time they write neighbouring pieces of the same rows
+  const int npairs = (w.pairs - part + w.parts - 1) / w.parts;
+  if (npairs <= 0) return;   // the whole block leaves
+  // the 32 floats (or fewer) of the lane's two rows of x; a float4 that would start outside the row is read from the
+  // row's end instead and zeroed
+  float4 a[2][4];
+#pragma unroll
+  for (int t = 0; t < 2; t++) {
+    long long row = row0 + 32 * t + i;
+    if (row > p.rows - 1) row = p.rows - 1;
+    const float *xr = p.x + row * p.xs;
+#pragma unroll
+    for (int s = 0; s < 4; s++) {
+      const int kf = 16 * h + 4 * s;
+      const float4 v = *(const float4 *)(xr + (kf < p.k2 ? kf : p.k2 - 4));
+      a[t][s] = kf < p.k2 ? v : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+  }
+  const float *vp = p.vp + lane * 4;
+  float4 b0[2][4], b1[2][4];
+  auto load = [&](int cp, float4 (&b)[2][4]) {
+#pragma unroll
+    for (int c = 0; c < 2; c++)
+#pragma unroll
+      for (int s = 0; s < 4; s++) b[c][s] = *(const float4 *)(vp + (long long)(2 * cp + c) * 1024 + 256 * s);
+  };
+  auto pair = [&](int cp, const float4 (&b)[2][4]) {
+    f16v acc[2][2];
+#pragma unroll
+    for (int t = 0; t < 2; t++)
+#pragma unroll
+      for (int c = 0; c < 2; c++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) acc[t][c][v] = 0.f;
+#pragma unroll
+    for (int s = 0; s < 4; s++)
+#pragma unroll
+      for (int t = 0; t < 2; t++)
+#pragma unroll
+        for (int c = 0; c < 2; c++) {
+          acc[t][c] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[t][s].x, b[c][s].x, acc[t][c], 0, 0, 0);
+          acc[t][c] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[t][s].y, b[c][s].y, acc[t][c], 0, 0, 0);
+          acc[t][c] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[t][s].z, b[c][s].z, acc[t][c], 0, 0, 0);
+          acc[t][c] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[t][s].w, b[c][s].w, acc[t][c], 0, 0, 0);
+        }
+    wave_sync();   // the reads of the previous pair come first
+#pragma unroll
+    for (int t = 0; t < 2; t++)
+#pragma unroll
+      for (int c = 0; c < 2; c++)
+#pragma unroll
+        for (int v = 0; v < 16; v++)
+          tile[(32 * t + 8 * (v / 4) + 4 * h + (v % 4)) * kWidePitch + 32 * c + i] = acc[t][c][v];
+    wave_sync();
+    const int col = 64 * cp + 4 * (lane & 15);
+#pragma unroll
+    for (int u = 0; u < 16; u++) {
+      const int lr = 4 * u + (lane >> 4);
+      const float4 v = *(const float4 *)(tile + lr * kWidePitch + 4 * (lane & 15));
+      if (row0 + lr < p.rows && col < p.n2) *(float4 *)(p.r + (row0 + lr) * p.rs + col) = v;
+    }
+  };
+  auto at = [&](int k) { return part + k * w.parts; };
+  load(at(0), b0);
+  int k = 0;
+  for (; k + 2 < npairs; k += 2) {   // no branch inside, and fences: the next tiles stay ahead of these sums
+    load(at(k + 1), b1);
+    __builtin_amdgcn_sched_barrier(0);
+    pair(at(k), b0);
+    __builtin_amdgcn_sched_barrier(0);
+    load(at(k + 2), b0);
+    __builtin_amdgcn_sched_barrier(0);
+    pair(at(k + 1), b1);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  if (k + 1 < npairs) {
+    load(at(k + 1), b1);
+    pair(at(k), b0);
+    pair(at(k + 1), b1);
+  } else {
+    pair(at(k), b0);
+  }
+}
+
 // the packed matrix of a call lives in a buffer kept per (device, stream): calls on one stream are ordered, calls on
 // different streams do not share a buffer
 struct Workspace {
@@ -326,6 +440,8 @@ float *workspace(size_t bytes, hipStream_t s) {
 
 int g_mix_long = 1;
 int g_mix_wide_store = 1;
+int g_mix_wide = 1;
+int g_mix_wide_waves = 40960;
 
 template <int RT, int CTW, bool PIPE>
 void launch(const MixArgs &a, hipStream_t s) {
@@ -373,6 +489,16 @@ int launch_mix(float2 *r, const float2 *x, const float2 *w, long long rows, int 
   } else if (!wide) {
     if (ctw == 1) launch<2, 1, true>(a, s);
     else launch<2, 2, true>(a, s);
+  } else if (a.nq == 1 && a.wide_store && g_mix_wide) {
+    WideArgs wa;
+    wa.m = a;
+    wa.pairs = a.ct_total / 2;
+    const long long groups = (rows + 63) / 64;
+    // enough waves for some ten rounds over the chip, but no wave with fewer than four pairs of tiles
+    long long parts = std::max<long long>(1, std::min<long long>(g_mix_wide_waves / groups, wa.pairs / 4));
+    wa.parts = (int)parts;
+    if (groups * wa.parts > 0x7fffffffLL) return 11;
+    hipLaunchKernelGGL(mix_wide_kernel, dim3((unsigned)(groups * wa.parts)), dim3(64), 0, s, wa);
   } else if (a.nq <= 2) {
     launch<2, 4, false>(a, s);
   } else {
@@ -564,6 +690,14 @@ int launch_mix_wgrad(float2 *wg, const float2 *x, const float2 *g, long long row
 int mix_set_option(const char *name, int value) {   // 0, or 12 for a name that is not an option of this file
   if (std::string(name) == "mix_long") {
     g_mix_long = value;
+    return 0;
+  }
+  if (std::string(name) == "mix_wide") {
+    g_mix_wide = value;
+    return 0;
+  }
+  if (std::string(name) == "mix_wide_waves") {
+    g_mix_wide_waves = value;
     return 0;
   }
   if (std::string(name) == "mix_wide_store") {

@@ -37,7 +37,7 @@ CASES = [
     # tiles of output, fewer rows than the 32 of a wave
     ((70,), 258, 5), ((33, 3), 300, 24), ((20, 3), 260, 70), ((5,), 1024, 16), ((3, 7), 514, 128),
     # many tiles of output: an odd number of output channels keeps the stores narrow, an even one sends them through LDS
-    ((50,), 8, 35), ((333,), 16, 130), ((260,), 16, 64),
+    ((50,), 8, 35), ((333,), 16, 130), ((260,), 16, 64), ((129, 3), 14, 1000), ((64,), 16, 34),
 ]
 
 
@@ -108,13 +108,18 @@ def test_mix_channels_wide_and_narrow_stores_agree(cabi):
     w = rand((200, 16), 8)
     r0 = torch.empty(77, 5, 200, dtype=torch.complex64, device="cuda")
     r1 = torch.empty_like(r0)
-    cabi.part_mix_channels(r0, x, w, adjoint=True)
-    cabi.set_option("mix_wide_store", 0)
+    r2 = torch.empty_like(r0)
+    cabi.part_mix_channels(r0, x, w, adjoint=True)      # the kernel that walks along the output
+    cabi.set_option("mix_wide", 0)
     try:
-        cabi.part_mix_channels(r1, x, w, adjoint=True)
+        cabi.part_mix_channels(r2, x, w, adjoint=True)  # one wave per four tiles, stores through LDS
+        cabi.set_option("mix_wide_store", 0)
+        cabi.part_mix_channels(r1, x, w, adjoint=True)  # stores straight from the registers
     finally:
         cabi.set_option("mix_wide_store", 1)
+        cabi.set_option("mix_wide", 1)
     assert torch.equal(torch.view_as_real(r0), torch.view_as_real(r1))
+    assert torch.equal(torch.view_as_real(r2), torch.view_as_real(r1))
 
 
 def test_mix_channels_rejects(cabi):

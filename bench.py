@@ -27,6 +27,8 @@ MEASURED_TRAFFIC = {
     # x and y are re-read by the waves that share a cell (mostly from the memory-side cache): 1.25 / 1.23 x algorithmic
     "so3vec_diagcg_L6_n64_B131072": {"so3vec_fwd": 127684806967, "so3vec_bwd": 133009610533},
     "so3part_cg_10x10_all_l_n8_B16384": {"so3vec_fwd": 3747210969, "so3vec_bwd": 3936276724},
+    # forward, gradient of the part, gradient of the matrix (with its sum kernel) and two packings of the matrix
+    "linear_l4_3840to16_B32768": {"step": 28063758950},
 }
 
 WORKLOADS = {
@@ -217,7 +219,8 @@ def aux_bench(torch, args, name):
            "steps": args.steps, "warmup": args.warmup, "ms_per_step": wall * 1e3 / args.steps, "higher_is_better": True,
            "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic", "config": {"workload": name},
            "roofline": {"bound": "hbm", "kernel": name.split("_")[0], "achieved": nbytes / (ms * 1e-3) / 1e9,
-                        "peak": HBM_PEAK / 1e9, "unit": "GB/s", "frac": nbytes / (ms * 1e-3) / HBM_PEAK, "traffic": None,
+                        "peak": HBM_PEAK / 1e9, "unit": "GB/s", "frac": nbytes / (ms * 1e-3) / HBM_PEAK,
+                        "traffic": None if args.batch else MEASURED_TRAFFIC.get(name, {}).get("step"),
                         "algorithmic_bytes_per_launch": nbytes}}
     if not args.no_cpu:
         rate, want, got = cpu()

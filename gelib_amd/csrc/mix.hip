@@ -309,9 +309,7 @@ struct WideArgs {
 };
 
 // The block is one wave and LDS serves the instructions of a wave in the order they were issued, so a write of one lane
-// followed by a read of another needs no barrier instruction -- only that the compiler keeps the order.  A real barrier
-// would also wait for every store in flight (the compiler drains all memory counters in front of one), and the
-// stores are what this kernel is made of.
+// followed by a read of another needs no barrier instruction -- only that the compiler keeps the order.
 __device__ __forceinline__ void wave_sync() {
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
   __builtin_amdgcn_wave_barrier();

@@ -10,11 +10,18 @@
 //     [-Im V   Re V ]
 // and the real product row is the complex result as it lies in memory.  v_mfma_f32_32x32x2_f32 multiplies a 32 x 2 block
 // of x by a 2 x 32 block of that matrix; lane (i, h) = (lane % 32, lane / 32) supplies x[row i][k + h] and V'[k + h][col i].
-// A wave owns 32 RT rows and CTW tiles of 32 output floats, and walks the reduction 32 floats (128 B of every row) at a
-// time: lane (i, h) reads the 16 floats of its row that start at 16 h, so each row is read in whole 128-B lines.  V' is
-// re-packed once per call into exactly the order the lanes read it (pack_kernel), 64 B per lane and step, and stays in L2.
+// V' is re-packed once per call into exactly the order the lanes read it (pack_kernel) and stays in L2.
 // Bound: HBM for n_out <= 16 (8 B of x per 8 n_out flops is 16 flop/B at n_out = 16, below the fp32 matrix-core ridge of
 // 157.3 TF / 8 TB/s = 19.7 flop/B), the matrix cores above that.
+//
+// Kernels: mix_kernel (a lane is tied to a row; any shape), mix_long_kernel (long rows into 16 channels or fewer),
+// mix_wide_kernel (16 channels or fewer into many: the gradient of a part), wgrad_kernel + wgrad_sum_kernel (the
+// gradient of the matrix).  In all of them a load never sits behind a branch (an address is clamped and the value
+// zeroed where it is used instead): behind a branch the compiler waits for every load in flight, not only the one
+// needed, which stops the loads of the next step from overlapping the matrix instructions of this one.
+//
+// mix_kernel: a wave owns 32 RT rows and CTW tiles of 32 output floats, and walks the reduction 32 floats (128 B of
+// every row) at a time: lane (i, h) reads the 16 floats of its row that start at 16 h.
 #include <algorithm>
 #include <map>
 #include <mutex>
@@ -30,12 +37,12 @@ typedef float f16v __attribute__((ext_vector_type(16)));
 
 struct MixArgs {
   const float *x;    // rows x (2 n_in) floats, row stride xs floats
-  const float *vp;   // packed V': [nq][ct_total][64 lanes][16] floats
+  const float *vp;   // packed V', in the order of pack_kernel
   float *r;          // rows x (2 n_out) floats, row stride rs floats
   long long rows, xs, rs;
   int k2;            // 2 n_in
   int n2;            // 2 n_out
-  int nq;            // ceil(k2 / 32)
+  int nq;            // steps of the reduction: ceil(k2 / 32), or ceil(k2 / 128) for the long-step kernel
   int ct_total;      // tiles of 32 output floats, padded to a multiple of CTW
   int wide_store;    // rows of r are 16-byte aligned and n2 is a multiple of 4: results leave through LDS, 512 B a row
 };
@@ -89,18 +96,13 @@ __global__ void __launch_bounds__(256) mix_kernel(const MixArgs p) {
   const float *vp = p.vp + (long long)ct0 * 1024 + lane * 4;
   const long long vstep = (long long)p.ct_total * 1024;
 
-  // matrix instructions that add into the same registers run one after the other, so every wave keeps at least
-  // four sums going: with fewer than four tiles the reduction is dealt over NCH sums per tile, added up at the end
-  constexpr int NCH = RT * CTW >= 4 ? 1 : 4 / (RT * CTW);
-  f16v acc[RT][CTW][NCH];
+  f16v acc[RT][CTW];
 #pragma unroll
   for (int t = 0; t < RT; t++)
 #pragma unroll
     for (int c = 0; c < CTW; c++)
 #pragma unroll
-      for (int n = 0; n < NCH; n++)
-#pragma unroll
-        for (int v = 0; v < 16; v++) acc[t][c][n][v] = 0.f;
+      for (int v = 0; v < 16; v++) acc[t][c][v] = 0.f;
 
   // k2 is a multiple of 4, so a float4 of a row is inside it or outside it as a whole; one that would start outside
   // is read from the row's end instead (no branch around a load, so loads stay in flight across the matrix
@@ -132,7 +134,7 @@ __global__ void __launch_bounds__(256) mix_kernel(const MixArgs p) {
             const float ar = e == 0 ? o.a[t][s].x : (e == 1 ? o.a[t][s].y : (e == 2 ? o.a[t][s].z : o.a[t][s].w));
             const float av = inside ? ar : 0.f;
             const float bv = e == 0 ? o.b[c][s].x : (e == 1 ? o.b[c][s].y : (e == 2 ? o.b[c][s].z : o.b[c][s].w));
-            acc[t][c][e % NCH] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv, acc[t][c][e % NCH], 0, 0, 0);
+            acc[t][c] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv, acc[t][c], 0, 0, 0);
           }
     }
   };
@@ -180,7 +182,7 @@ __global__ void __launch_bounds__(256) mix_kernel(const MixArgs p) {
 #pragma unroll
         for (int c = 0; c < CTW; c++)
 #pragma unroll
-          for (int v = 0; v < 16; v++) tile[(8 * (v / 4) + 4 * h + (v % 4)) * kPitch + 32 * c + i] = acc[t][c][0][v];
+          for (int v = 0; v < 16; v++) tile[(8 * (v / 4) + 4 * h + (v % 4)) * kPitch + 32 * c + i] = acc[t][c][v];
         __syncthreads();
         const int col = 32 * ct0 + 4 * i;
 #pragma unroll
@@ -198,13 +200,10 @@ __global__ void __launch_bounds__(256) mix_kernel(const MixArgs p) {
 #pragma unroll
     for (int c = 0; c < CTW; c++) {
       const int col = 32 * (ct0 + c) + i;
-      f16v sum = acc[t][c][0];
-#pragma unroll
-      for (int n = 1; n < NCH; n++) sum += acc[t][c][n];
 #pragma unroll
       for (int v = 0; v < 16; v++) {
         const long long row = row0 + 32 * t + 8 * (v / 4) + 4 * h + (v % 4);
-        if (row < p.rows && col < p.n2) p.r[row * p.rs + col] = sum[v];
+        if (row < p.rows && col < p.n2) p.r[row * p.rs + col] = acc[t][c][v];
       }
     }
 }

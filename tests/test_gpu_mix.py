@@ -129,3 +129,34 @@ def test_mix_channels_rejects(cabi):
     with pytest.raises(cabi.GelibHipError):
         cabi.part_mix_channels(r, x, w)     # an odd number of input channels
     assert not cabi.mix_channels_ok(x)
+
+
+def test_mix_channels_random_shapes(cabi):
+    """Random draws over all three operations and all kernels: row counts around the 32 and 64 rows of a wave, channel
+    counts around the tile sizes (16, 32, 64, 128 floats), long and short rows."""
+    rng = np.random.default_rng(2024)
+    eps = np.finfo(np.float32).eps
+    pick = lambda: int(rng.choice([2, 4, 6, 8, 14, 16, 18, 30, 32, 34, 62, 64, 66, 126, 128, 130, 254, 256, 258, 300, 514]))
+    for draw in range(150):
+        rows = int(rng.choice([1, 2, 31, 32, 33, 63, 64, 65, 100, 257, 1000]))
+        n_in = pick()
+        n_out = int(rng.choice([1, 3, 5, 8, 15, 16, 17, 24, 31, 32, 33, 48, 64, 65, 100, 130, 256, 400]))
+        what = draw % 3
+        x = rand((rows, n_in), 100 + draw)
+        hx = U.host(x).astype(np.complex128)
+        tag = "draw %d: rows %d n_in %d n_out %d op %d" % (draw, rows, n_in, n_out, what)
+        if what == 2:
+            g = rand((rows, n_out), 500 + draw)
+            wg = torch.full((n_in, n_out), float("nan"), dtype=torch.complex64, device="cuda")
+            cabi.part_mix_channels_wgrad(wg, x, g)
+            hg = U.host(g).astype(np.complex128)
+            want, scale, got = hx.conj().T @ hg, np.abs(hx).T @ np.abs(hg), U.host(wg)
+        else:
+            w = rand((n_out, n_in) if what else (n_in, n_out), 500 + draw)
+            r = torch.full((rows, n_out), float("nan"), dtype=torch.complex64, device="cuda")
+            cabi.part_mix_channels(r, x, w, adjoint=bool(what))
+            v = U.host(w).astype(np.complex128)
+            v = v.conj().T if what else v
+            want, scale, got = hx @ v, np.abs(hx) @ np.abs(v), U.host(r)
+        assert np.isfinite(got.view(np.float32)).all(), tag
+        assert (np.abs(got - want) <= 1e-6 + 4 * eps * scale).all(), tag

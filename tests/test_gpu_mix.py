@@ -160,3 +160,25 @@ def test_mix_channels_random_shapes(cabi):
             want, scale, got = hx @ v, np.abs(hx) @ np.abs(v), U.host(r)
         assert np.isfinite(got.view(np.float32)).all(), tag
         assert (np.abs(got - want) <= 1e-6 + 4 * eps * scale).all(), tag
+
+
+def test_mix_channels_row_strides(cabi):
+    """The C entry points take row strides: a block of channels of a wider tensor in, a block of a wider tensor out."""
+    rows, n_in, n_out = 300, 40, 16
+    xw = rand((rows, 64), 11)                 # x = channels 8..47 of a 64-channel tensor
+    rw = torch.zeros(rows, 24, dtype=torch.complex64, device="cuda")   # r = channels 4..19 of a 24-channel tensor
+    w = rand((n_in, n_out), 12)
+    x, r = xw[:, 8:8 + n_in], rw[:, 4:4 + n_out]
+    L = cabi.lib()
+    cabi.check(L.gelib_hip_part_mix_channels(r.data_ptr(), x.data_ptr(), w.data_ptr(), rows, n_in, n_out, 24, 64, 0, None))
+    want = U.host(x.contiguous()).astype(np.complex128) @ U.host(w).astype(np.complex128)
+    tol = 1e-6 + 4 * np.finfo(np.float32).eps * (np.abs(U.host(x.contiguous())).astype(np.float64) @ np.abs(U.host(w)).astype(np.float64))
+    assert (np.abs(U.host(r.contiguous()) - want) <= tol).all()
+    keep = torch.ones(24, dtype=torch.bool)
+    keep[4:4 + n_out] = False
+    assert float(rw[:, keep.cuda()].abs().max()) == 0.0      # nothing outside the block was written
+    g = rand((rows, n_out), 13)
+    wg = torch.empty(n_in, n_out, dtype=torch.complex64, device="cuda")
+    cabi.check(L.gelib_hip_part_mix_channels_wgrad(wg.data_ptr(), x.data_ptr(), g.data_ptr(), rows, n_in, n_out, 64, n_out, None))
+    hx, hg = U.host(x.contiguous()).astype(np.complex128), U.host(g).astype(np.complex128)
+    assert (np.abs(U.host(wg) - hx.conj().T @ hg) <= 1e-6 + 4 * np.finfo(np.float32).eps * (np.abs(hx).T @ np.abs(hg))).all()

@@ -7,7 +7,9 @@ headline configuration: L=4, 16 channels per part, batch 32768, product capped a
 
 Prints ONE JSON line: samples/s (whole job), the roofline of the dominant kernel from HIP-event timings taken
 inside this run, and a CPU baseline (the oracle's loop-order-faithful float32 restatement of the reference's CPU
-path, timed here on one host core over a batch slice; the GPU result for that slice is checked against it).
+path, timed here on one host core over a batch slice; the GPU result for that slice is checked against it, every
+component, and the run exits with status 3 if one fails).  After the headline, the default run times the other
+configurations of the baseline list the same way and reports one record each under config.all_configs.
 """
 import argparse
 import json
@@ -20,16 +22,36 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK = 8.0e12  # B/s, MI355X HBM3E
 
-# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs, each scaled by what the
-# counter reads for a plain 1 GiB copy: x2.000 and x1.000); summary in profiles/.
-MEASURED_TRAFFIC = {
-    "so3vec_cg_L4_tau16_B32768_maxl4": {"so3vec_fwd": 27148781681, "so3vec_bwd": 25959930442},
-    # x and y are re-read by the waves that share a cell (mostly from the memory-side cache): 1.25 / 1.23 x algorithmic
-    "so3vec_diagcg_L6_n64_B131072": {"so3vec_fwd": 127684806967, "so3vec_bwd": 133009610533},
-    "so3part_cg_10x10_all_l_n8_B16384": {"so3vec_fwd": 3747210969, "so3vec_bwd": 3936276724},
-    # forward, gradient of the part, gradient of the matrix (with its sum kernel) and two packings of the matrix
-    "linear_l4_3840to16_B32768": {"step": 28063758950},
-}
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+
+
+def kernel_sources_digest():
+    """sha256 over the kernel sources (file names and contents, sorted): what a traffic measurement belongs to."""
+    import hashlib
+    d = os.path.join(ROOT, "gelib_amd", "csrc")
+    h = hashlib.sha256()
+    for fn in sorted(os.listdir(d)):
+        if fn.endswith((".hip", ".h", ".cpp")) or fn == "Makefile":
+            h.update(fn.encode())
+            with open(os.path.join(d, fn), "rb") as f:
+                h.update(f.read())
+    return h.hexdigest()
+
+
+def measured_traffic(name, key):
+    """HBM bytes per launch from profiles/hbm_traffic.json (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, two runs, each
+    scaled by what the counter reads for a plain 1 GiB copy), or None when the kernel sources have changed since the
+    counters were read: a stale figure is not printed."""
+    try:
+        with open(TRAFFIC_FILE) as f:
+            t = json.load(f)
+    except (OSError, ValueError):
+        return None
+    rec = t.get("workloads", {}).get(name)
+    if not rec or rec.get("sources_sha256") != kernel_sources_digest():
+        return None
+    return rec.get(key)
+
 
 WORKLOADS = {
     # name: (kind, B, tau_x, tau_y, maxl, diag)
@@ -44,8 +66,14 @@ WORKLOADS = {
     "so3vec_cg_L4_tau4_B524288_maxl4": ("vec", 524288, {l: 4 for l in range(5)}, {l: 4 for l in range(5)}, 4, False),
     "so3vec_cg_L2_tau64_B8192_maxl2": ("vec", 8192, {l: 64 for l in range(3)}, {l: 64 for l in range(3)}, 2, False),
     "so3vec_diagcg_L4_n64_B131072_uncapped": ("vec", 131072, {l: 64 for l in range(5)}, {l: 64 for l in range(5)}, -1, True),
+    "so3part_cg_1x1to1_n16_B1024": ("vec", 1024, {1: 16}, {1: 16}, 1, False),
 }
-ALIASES = {"cfg4": "so3vec_cg_L4_tau16_B32768_maxl4", "cfg4u": "so3vec_cg_L4_tau16_B32768_uncapped",
+HEADLINE = "so3vec_cg_L4_tau16_B32768_maxl4"
+# the configurations of the baseline list other than the headline, with the size of the CPU slice each is checked on
+OTHER_CONFIGS = [("so3part_cg_1x1to1_n16_B1024", 1024), ("so3part_cg_2x3to4_n32_B65536", 512),
+                 ("so3vec_diagcg_L6_n64_B131072", 64), ("so3vec_cg_L4_tau16_B32768_uncapped", 256),
+                 ("so3part_cg_10x10_all_l_n8_B16384", 64)]
+ALIASES = {"cfg1": "so3part_cg_1x1to1_n16_B1024", "cfg4": "so3vec_cg_L4_tau16_B32768_maxl4", "cfg4u": "so3vec_cg_L4_tau16_B32768_uncapped",
            "cfg2": "so3part_cg_2x3to4_n32_B65536", "cfg3": "so3vec_diagcg_L6_n64_B131072",
            "cfg5": "so3part_cg_10x10_all_l_n8_B16384", "diag4": "so3vec_diagcg_L4_n64_B131072",
            "diag4n16": "so3vec_diagcg_L4_n16_B524288", "cg6": "so3vec_cg_L6_tau8_B16384_maxl6",
@@ -80,50 +108,61 @@ def seeded_parts(torch, seed, B, tau, device, scale=1.0):
     return parts
 
 
-def cpu_baseline(torch, xs, ys, gs, rs, xgs, ygs, maxl, diag, nsample):
-    """Time the oracle on the first `nsample` samples with one thread and check the GPU slice against it."""
+def cpu_slice(torch, xs, ys, gs, rs, xgs, ygs, maxl, diag, nsample, single_core):
+    """The oracle on the first `nsample` samples: timed (one thread, if single_core, and with the batch loop split over
+    the host's cores, which is what the reference's MultiLoop would do) and used as the checker of the GPU results for
+    that slice.  Every real component is held to the parity rules of tests/gpu_util.py (gate, or one of the two stated
+    rules for sums that nearly cancel); the fractions that needed each rule are reported."""
     import numpy as np
     from oracle import cg_oracle as ora
+    from tests import gpu_util as U
     hx = [t[:nsample].cpu().numpy() for t in xs]
     hy = [t[:nsample].cpu().numpy() for t in ys]
     hg = [t[:nsample].cpu().numpy() for t in gs]
     ora.lib()
-    t0 = time.perf_counter()
-    r = ora.vec_fwd(hx, hy, maxl, diag, nthreads=1)
-    xg, yg = ora.vec_bwd(hg, hx, hy, diag, nthreads=1)
-    dt = time.perf_counter() - t0
-    # the same slice with the batch loop split over the host's cores (what the reference's MultiLoop would do)
     nth = max(1, min(16, ora.max_threads(), os.cpu_count() or 1))
+    dt1 = None
+    if single_core:
+        t0 = time.perf_counter()
+        ora.vec_fwd(hx, hy, maxl, diag, nthreads=1)
+        ora.vec_bwd(hg, hx, hy, diag, nthreads=1)
+        dt1 = time.perf_counter() - t0
     t0 = time.perf_counter()
-    ora.vec_fwd(hx, hy, maxl, diag, nthreads=nth)
-    ora.vec_bwd(hg, hx, hy, diag, nthreads=nth)
+    r = ora.vec_fwd(hx, hy, maxl, diag, nthreads=nth)
+    xg, yg = ora.vec_bwd(hg, hx, hy, diag, nthreads=nth)
     dt_all = time.perf_counter() - t0
+    r64 = ora.vec_fwd(U.c128(hx), U.c128(hy), maxl, diag, nthreads=nth)
+    xg64, yg64 = ora.vec_bwd(U.c128(hg), U.c128(hx), U.c128(hy), diag, nthreads=nth)
+    Sr = ora.vec_fwd_term_sums(hx, hy, maxl, diag, nthreads=nth)
+    Sx, Sy = ora.vec_bwd_term_sums(hg, hx, hy, diag, nthreads=nth)
 
-    def excess(got, ref):
-        a = got[:nsample].cpu().numpy().view(np.float32).astype(np.float64)
-        b = ref.view(np.float32).astype(np.float64)
-        return float(np.max(np.abs(a - b) / (1e-6 + 1e-5 * np.abs(b))))
+    def merge(gpu_parts, c32, c64, S):
+        tot = {"components": 0, "outside_gate": 0.0, "cpu_f32_outside_gate_of_f64": 0.0, "by_rule_B": 0.0,
+               "by_rule_C": 0.0, "rejected": 0, "max_err_over_rule_C_bound": 0.0, "max_gate_excess": 0.0,
+               "max_err_vs_f64": {"gpu": 0.0, "cpu_f32": 0.0}}
+        for t, b, c, s in zip(gpu_parts, c32, c64, S):
+            a = t[:nsample].cpu().numpy()
+            rep = U.parity_counts(a, b, c, s)
+            n = rep["components"]
+            for k in ("outside_gate", "cpu_f32_outside_gate_of_f64", "by_rule_B", "by_rule_C"):
+                tot[k] += rep[k] * n
+            tot["components"] += n
+            tot["rejected"] += rep["rejected"]
+            tot["max_err_over_rule_C_bound"] = max(tot["max_err_over_rule_C_bound"], rep["max_err_over_rule_C_bound"])
+            tot["max_gate_excess"] = max(tot["max_gate_excess"], U.gate_excess(a, b))
+            tot["max_err_vs_f64"]["gpu"] = max(tot["max_err_vs_f64"]["gpu"], U.max_abs_err(a, c))
+            tot["max_err_vs_f64"]["cpu_f32"] = max(tot["max_err_vs_f64"]["cpu_f32"], U.max_abs_err(b, c))
+        for k in ("outside_gate", "cpu_f32_outside_gate_of_f64", "by_rule_B", "by_rule_C"):
+            tot[k] /= max(1, tot["components"])
+        return tot
 
-    # float64 oracle on a smaller slice: how far each float32 path is from the exact answer
-    n64 = min(nsample, 128)
-    c128 = lambda L: [a[:n64].astype(np.complex128) for a in L]
-    r64 = ora.vec_fwd(c128(hx), c128(hy), maxl, diag)
-    xg64, yg64 = ora.vec_bwd(c128(hg), c128(hx), c128(hy), diag)
-
-    def err(got, exact, gpu):
-        a = (got[:n64].cpu().numpy() if gpu else got[:n64]).view(np.float32).astype(np.float64)
-        return float(np.max(np.abs(a - exact.view(np.float64))))
-
-    parity = {"fwd_gate_excess": max(excess(a, b) for a, b in zip(rs, r)),
-              "bwd_gate_excess": max(excess(a, b) for a, b in zip(xgs + ygs, xg + yg)),
-              "gate": "|gpu-cpu| <= 1e-6 + 1e-5*|cpu| per real component; excess <= 1 is inside",
-              "fwd_max_err_vs_f64": {"gpu": max(err(a, b, True) for a, b in zip(rs, r64)),
-                                     "cpu_f32": max(err(a, b, False) for a, b in zip(r, r64))},
-              "bwd_max_err_vs_f64": {"gpu": max(err(a, b, True) for a, b in zip(xgs + ygs, xg64 + yg64)),
-                                     "cpu_f32": max(err(a, b, False) for a, b in zip(xg + yg, xg64 + yg64))},
-              "note": "backward sums ~1000 float32 terms per element; both float32 paths sit ~1e-5 from the "
-                      "float64 answer, which is what the gate excess of the backward pass measures"}
-    return nsample / dt, dt, parity, {"value": nsample / dt_all, "unit": "samples/s", "cores": nth}
+    fwd = merge(rs, r, r64, Sr)
+    bwd = merge(xgs + ygs, xg + yg, xg64 + yg64, Sx + Sy)
+    parity = {"ok": fwd["rejected"] == 0 and bwd["rejected"] == 0, "samples": nsample, "fwd": fwd, "bwd": bwd,
+              "rules": "per real component: A |gpu-cpu| <= 1e-6 + 1e-5|cpu|; else B (cpu_f32 itself outside that gate "
+                       "of float64 and |gpu-f64| <= |cpu-f64|); else C |gpu-f64| <= 1e-6 + 2*eps32*sum|terms|; "
+                       "outside_gate = fraction not passing A, rejected = components passing none"}
+    return {"single_core_s": dt1, "all_cores_s": dt_all, "cores": nth, "parity": parity}
 
 
 AUX_WORKLOADS = ("spharm_l4_n16_B1048576", "gather_l2_n16_cells262144_deg8", "linear_l4_3840to16_B32768")
@@ -220,13 +259,109 @@ def aux_bench(torch, args, name):
            "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic", "config": {"workload": name},
            "roofline": {"bound": "hbm", "kernel": name.split("_")[0], "achieved": nbytes / (ms * 1e-3) / 1e9,
                         "peak": HBM_PEAK / 1e9, "unit": "GB/s", "frac": nbytes / (ms * 1e-3) / HBM_PEAK,
-                        "traffic": None if args.batch else MEASURED_TRAFFIC.get(name, {}).get("step"),
+                        "traffic": None if args.batch else measured_traffic(name, "step"),
                         "algorithmic_bytes_per_launch": nbytes}}
     if not args.no_cpu:
         rate, want, got = cpu()
         out["cpu_baseline"] = {"value": rate, "unit": unit, "cores": 1, "kind": "port", "sample": sample}
         out["parity"] = {"ok": bool(np.allclose(got, want, **tol))}
     print(json.dumps(out))
+
+
+PATH_NAMES = {1: "generic", 2: "unrolled", 3: "staged", 4: "diag6", 5: "onepair"}
+
+
+def run_cg_workload(torch, cabi, name, steps, warmup, batch=0, cpu_samples=0, single_core=False, copy_probe=False,
+                    fill_reference=False):
+    """Forward + backward of one product workload: `warmup` untimed steps, then `steps` steps bracketed by device
+    synchronisations (wall clock) with HIP events around each call on the stream the kernels run on; then, outside the
+    timed region, the CPU oracle on a slice of the batch as checker and baseline.  Frees its buffers on return."""
+    dev = torch.device("cuda:0")
+    kind, B, tx, ty, maxl, diag = WORKLOADS[name]
+    if batch:
+        B = batch
+    tr = out_type(tx, ty, maxl, diag)
+    fwd_bytes, bwd_bytes = algorithmic_bytes(B, tx, ty, tr)
+    scale_y = 1e-3 if "10x10" in name else 1.0
+    xs = seeded_parts(torch, 1004, B, tx, dev)
+    ys = seeded_parts(torch, 2004, B, ty, dev, scale_y)
+    gs = seeded_parts(torch, 3004, B, tr, dev)
+    rs = [torch.empty(B, 2 * l + 1, n, dtype=torch.complex64, device=dev) for l, n in tr.items()]
+    xgs = [torch.empty_like(t) for t in xs]
+    ygs = [torch.empty_like(t) for t in ys]
+
+    def fwd():
+        cabi.so3vec_fwd(rs, xs, ys, accumulate=False, diag=diag)
+
+    def bwd():
+        cabi.so3vec_bwd(xgs, ygs, gs, xs, ys, accumulate=False, diag=diag)
+
+    if copy_probe:
+        src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
+        dst = torch.empty_like(src)
+        dst.copy_(src)   # reads 1 GiB, writes 1 GiB
+        torch.cuda.synchronize()
+        del src, dst
+    for _ in range(warmup):
+        fwd()
+        bwd()
+    torch.cuda.synchronize()
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(steps)]
+    t0 = time.perf_counter()
+    for k in range(steps):
+        ev[k][0].record()
+        fwd()
+        ev[k][1].record()
+        bwd()
+        ev[k][2].record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    path_bwd = cabi.last_path()
+    fwd_ms = sum(e[0].elapsed_time(e[1]) for e in ev) / steps
+    bwd_ms = sum(e[1].elapsed_time(e[2]) for e in ev) / steps
+    fwd()
+    path_fwd = cabi.last_path()
+    torch.cuda.synchronize()
+    full = B == WORKLOADS[name][1]
+    rec = {"workload": name, "batch": B, "tau_x": {str(k): v for k, v in tx.items()},
+           "tau_y": {str(k): v for k, v in ty.items()}, "maxl": maxl, "diag": diag,
+           "triples": sum(1 for l1 in tx for l2 in ty for l in range(abs(l1 - l2), l1 + l2 + 1) if l in tr),
+           "kernel_path": {"fwd": PATH_NAMES.get(path_fwd, str(path_fwd)), "bwd": PATH_NAMES.get(path_bwd, str(path_bwd))},
+           "timed_steps": steps, "ms_per_step_wall": wall * 1e3 / steps, "samples_per_s": B / (wall / steps),
+           "fwd_ms": fwd_ms, "bwd_ms": bwd_ms,
+           "fwd_ms_min": min(e[0].elapsed_time(e[1]) for e in ev), "bwd_ms_min": min(e[1].elapsed_time(e[2]) for e in ev),
+           "fwd_algorithmic_bytes": fwd_bytes, "bwd_algorithmic_bytes": bwd_bytes,
+           "fwd_GBps": fwd_bytes / (fwd_ms * 1e-3) / 1e9, "bwd_GBps": bwd_bytes / (bwd_ms * 1e-3) / 1e9,
+           "fwd_frac_of_peak": fwd_bytes / (fwd_ms * 1e-3) / HBM_PEAK,
+           "bwd_frac_of_peak": bwd_bytes / (bwd_ms * 1e-3) / HBM_PEAK,
+           "fwd_bwd_GBps": (fwd_bytes + bwd_bytes) / ((fwd_ms + bwd_ms) * 1e-3) / 1e9,
+           "fwd_bwd_frac_of_peak": (fwd_bytes + bwd_bytes) / ((fwd_ms + bwd_ms) * 1e-3) / HBM_PEAK,
+           "fwd_traffic_bytes": measured_traffic(name, "so3vec_fwd") if full else None,
+           "bwd_traffic_bytes": measured_traffic(name, "so3vec_bwd") if full else None}
+    if cpu_samples:
+        ns = min(cpu_samples, B)
+        c = cpu_slice(torch, xs, ys, gs, rs, xgs, ygs, maxl, diag, ns, single_core)
+        rec["parity"] = c["parity"]
+        rec["cpu"] = {"samples": ns, "cores": c["cores"], "all_cores_samples_per_s": ns / c["all_cores_s"],
+                      "single_core_samples_per_s": ns / c["single_core_s"] if c["single_core_s"] else None,
+                      "single_core_s": c["single_core_s"]}
+    if fill_reference:
+        # What a plain streaming kernel reaches on these very buffers (outside the timed region): torch's fill over the
+        # product parts.  Write bandwidth on this GPU depends on where a buffer lies in memory (about 5.6 or 6.6 TB/s
+        # for one and the same kernel), so this is the yardstick beside the nominal peak.
+        def timed(fn):
+            fn()
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            fn()
+            b.record()
+            torch.cuda.synchronize()
+            return a.elapsed_time(b) * 1e-3
+        rbytes = sum(t.numel() * 8 for t in rs)
+        rec["streaming_reference"] = {"torch_fill_of_product_GBps": rbytes / timed(lambda: [t.fill_(1.0) for t in rs]) / 1e9}
+    del xs, ys, gs, rs, xgs, ygs
+    torch.cuda.empty_cache()
+    return rec
 
 
 def main():
@@ -238,6 +373,9 @@ def main():
     ap.add_argument("--batch", type=int, default=0, help="override the batch size (debugging only)")
     ap.add_argument("--cpu-samples", type=int, default=2048)
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--only", action="store_true",
+                    help="time the named workload alone (the default run also times the other configurations of the "
+                         "baseline list and reports them under config.all_configs)")
     ap.add_argument("--generic", action="store_true", help="force the shape-agnostic kernels")
     ap.add_argument("--option", action="append", default=[], metavar="NAME=VALUE",
                     help="library tuning option (gelib_hip_set_option), may be repeated")
@@ -259,104 +397,52 @@ def main():
     for kv in args.option:
         k, v = kv.split("=")
         cabi.set_option(k, int(v))
-    dev = torch.device("cuda:0")
     name = ALIASES.get(args.workload, args.workload)
     aux = [w for w in AUX_WORKLOADS if w == name or w.split("_")[0] == name]
     if aux:
         return aux_bench(torch, args, aux[0])
-    kind, B, tx, ty, maxl, diag = WORKLOADS[name]
-    if args.batch:
-        B = args.batch
-    tr = out_type(tx, ty, maxl, diag)
-    fwd_bytes, bwd_bytes = algorithmic_bytes(B, tx, ty, tr)
 
-    scale_y = 1e-3 if "10x10" in name else 1.0
-    xs = seeded_parts(torch, 1004, B, tx, dev)
-    ys = seeded_parts(torch, 2004, B, ty, dev, scale_y)
-    gs = seeded_parts(torch, 3004, B, tr, dev)
-    rs = [torch.empty(B, 2 * l + 1, n, dtype=torch.complex64, device=dev) for l, n in tr.items()]
-    xgs = [torch.empty_like(t) for t in xs]
-    ygs = [torch.empty_like(t) for t in ys]
-
-    def fwd():
-        cabi.so3vec_fwd(rs, xs, ys, accumulate=False, diag=diag)
-
-    def bwd():
-        cabi.so3vec_bwd(xgs, ygs, gs, xs, ys, accumulate=False, diag=diag)
-
-    if args.copy_probe:
-        src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
-        dst = torch.empty_like(src)
-        dst.copy_(src)   # reads 1 GiB, writes 1 GiB
-        torch.cuda.synchronize()
-        del src, dst
-    for _ in range(args.warmup):
-        fwd()
-        bwd()
-    torch.cuda.synchronize()
-    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
-    t0 = time.perf_counter()
-    for k in range(args.steps):
-        ev[k][0].record()
-        fwd()
-        ev[k][1].record()
-        bwd()
-        ev[k][2].record()
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-    fwd_ms = sum(e[0].elapsed_time(e[1]) for e in ev) / args.steps
-    bwd_ms = sum(e[1].elapsed_time(e[2]) for e in ev) / args.steps
-    ms_per_step = wall * 1e3 / args.steps
-    path = cabi.last_path()
-
-
-    if bwd_ms >= fwd_ms:
-        dom, dom_ms, dom_bytes = "so3vec_bwd", bwd_ms, bwd_bytes
+    rec = run_cg_workload(torch, cabi, name, args.steps, args.warmup, args.batch,
+                          0 if args.no_cpu else args.cpu_samples, single_core=True, copy_probe=args.copy_probe,
+                          fill_reference=True)
+    if rec["bwd_ms"] >= rec["fwd_ms"]:
+        dom, dom_ms, dom_bytes, traffic = "so3vec_bwd", rec["bwd_ms"], rec["bwd_algorithmic_bytes"], rec["bwd_traffic_bytes"]
     else:
-        dom, dom_ms, dom_bytes = "so3vec_fwd", fwd_ms, fwd_bytes
+        dom, dom_ms, dom_bytes, traffic = "so3vec_fwd", rec["fwd_ms"], rec["fwd_algorithmic_bytes"], rec["fwd_traffic_bytes"]
     achieved = dom_bytes / (dom_ms * 1e-3) / 1e9
+    parity = rec.pop("parity", None)
+    cpu = rec.pop("cpu", None)
     out = {
         "metric": "SO3vec CGproduct fwd+bwd samples/s at L=4; achieved HBM GB/s vs peak",
-        "value": B / (ms_per_step * 1e-3),
+        "value": rec["samples_per_s"],
         "unit": "samples/s",
-        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": rec["ms_per_step_wall"],
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-        "config": {"workload": name, "batch": B, "tau_x": {str(k): v for k, v in tx.items()},
-                   "tau_y": {str(k): v for k, v in ty.items()}, "maxl": maxl, "diag": diag,
-                   "triples": sum(1 for l1 in tx for l2 in ty for l in range(abs(l1 - l2), l1 + l2 + 1) if l in tr),
-                   "kernel_path": {1: "generic", 2: "unrolled", 3: "staged", 4: "diag6", 5: "onepair"}.get(path, str(path)),
-                   "fwd_ms": fwd_ms, "bwd_ms": bwd_ms,
-                   "fwd_GBps": fwd_bytes / (fwd_ms * 1e-3) / 1e9, "bwd_GBps": bwd_bytes / (bwd_ms * 1e-3) / 1e9,
-                   "fwd_bwd_GBps": (fwd_bytes + bwd_bytes) / ((fwd_ms + bwd_ms) * 1e-3) / 1e9,
-                   "fwd_bwd_frac_of_peak": (fwd_bytes + bwd_bytes) / ((fwd_ms + bwd_ms) * 1e-3) / HBM_PEAK},
+        "config": rec,
         "roofline": {"bound": "hbm", "kernel": dom, "achieved": achieved, "peak": HBM_PEAK / 1e9, "unit": "GB/s",
-                     "frac": achieved * 1e9 / HBM_PEAK,
-                     "traffic": MEASURED_TRAFFIC.get(name, {}).get(dom) if B == WORKLOADS[name][1] and path in (2, 3, 4, 5) else None,
+                     "frac": achieved * 1e9 / HBM_PEAK, "traffic": traffic,
                      "algorithmic_bytes_per_launch": dom_bytes},
     }
-    if not args.no_cpu:
-        ns = min(args.cpu_samples, B)
-        sps, dt, parity, allc = cpu_baseline(torch, xs, ys, gs, rs, xgs, ygs, maxl, diag, ns)
-        out["cpu_baseline"] = {"value": sps, "unit": "samples/s", "cores": 1, "kind": "port",
-                               "sample": "first %d samples of the same batch, fwd+bwd, %.1f s" % (ns, dt),
-                               "all_cores": allc}
+    ok = True
+    if cpu:
+        out["cpu_baseline"] = {"value": cpu["single_core_samples_per_s"], "unit": "samples/s", "cores": 1, "kind": "port",
+                               "sample": "first %d samples of the same batch, fwd+bwd, %.1f s" % (cpu["samples"], cpu["single_core_s"]),
+                               "all_cores": {"value": cpu["all_cores_samples_per_s"], "unit": "samples/s", "cores": cpu["cores"]}}
         out["parity"] = parity
-
-    # What a plain streaming kernel reaches on these very buffers (outside the timed region): torch's fill over the
-    # product parts.  Write bandwidth on this GPU depends on where a buffer lies in memory (about 5.6 or 6.6 TB/s
-    # for one and the same kernel), so this is the yardstick beside the nominal peak.
-    def timed(fn):
-        fn()
-        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        a.record()
-        fn()
-        b.record()
-        torch.cuda.synchronize()
-        return a.elapsed_time(b) * 1e-3
-    rbytes = sum(t.numel() * 8 for t in rs)
-    fill_GBps = rbytes / timed(lambda: [t.fill_(1.0) for t in rs]) / 1e9
-    out["config"]["streaming_reference"] = {"torch_fill_of_product_GBps": fill_GBps}
+        ok = ok and parity["ok"]
+    if name == HEADLINE and not args.only and not args.batch and not args.generic:
+        # the other configurations of the baseline list, each timed the same way (HIP events, >= 10 timed steps) and
+        # checked on a CPU slice; outside the headline's timed region
+        others = []
+        for wl, ns in OTHER_CONFIGS:
+            r = run_cg_workload(torch, cabi, wl, max(10, args.steps), 3, 0, 0 if args.no_cpu else ns)
+            ok = ok and r.get("parity", {}).get("ok", True)
+            others.append(r)
+        out["config"]["all_configs"] = others
     print(json.dumps(out))
+    if not ok:
+        print("bench.py: a GPU result on the CPU slice passes none of the parity rules (see \"parity\")", file=sys.stderr)
+        sys.exit(3)
 
 
 if __name__ == "__main__":

@@ -82,6 +82,15 @@ double ora_cg_coeff(int l1, int l2, int l, int m1, int m2) {
   return plusminus(l1 - l2 - m3) * plusminus(l1 - l2 + m) * sqrt((double)(2 * l + 1)) * wigner;
 }
 
+/*
+ * Error-analysis aid, not part of the reference's algorithm: while the switch is on, ora_cg_matrix returns |C|.
+ * Run on the moduli of the operands, the float64 loop nests then give, for every element of a result, the sum of
+ * the moduli of its terms, sum |C| |a| |b|: the scale that the rounding error of a float32 evaluation of that
+ * element follows, whatever the order of its additions.  Process-wide; callers switch it off again.
+ */
+static int abs_coeffs = 0;
+void ora_set_abs_coeffs(int on) { abs_coeffs = on; }
+
 /* Row-major (2l1+1) x (2l2+1) float table; entries with |m1+m2|>l are zero (never read by the kernels). */
 int ora_cg_matrix(int l1, int l2, int l, float *out) {
   if (l1 < 0 || l2 < 0 || l < abs(l1 - l2) || l > l1 + l2) return 1;
@@ -90,7 +99,10 @@ int ora_cg_matrix(int l1, int l2, int l, float *out) {
   for (int m1 = -l1; m1 <= l1; m1++) {
     int lo = (-l2 > -l - m1) ? -l2 : -l - m1;
     int hi = (l2 < l - m1) ? l2 : l - m1;
-    for (int m2 = lo; m2 <= hi; m2++) out[(m1 + l1) * L2 + (m2 + l2)] = (float)ora_cg_coeff(l1, l2, l, m1, m2);
+    for (int m2 = lo; m2 <= hi; m2++) {
+      float c = (float)ora_cg_coeff(l1, l2, l, m1, m2);
+      out[(m1 + l1) * L2 + (m2 + l2)] = abs_coeffs ? fabsf(c) : c;
+    }
   }
   return 0;
 }

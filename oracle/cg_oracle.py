@@ -168,6 +168,44 @@ def vec_bwd(gparts, xparts, yparts, diag=False, nthreads=1):
     return xg, yg
 
 
+def _moduli(parts):
+    return [np.abs(a).astype(np.complex128) for a in parts]
+
+
+def part_term_sums(op, r, x, y, offs=0):
+    """Term sums of one part-level operation, for its destination (r forward, x back0, y back1): the float64 loop
+    nest with |C| on the moduli of the other two tensors, started from zero.  Arrays as for part_op."""
+    parts = [_moduli([a])[0] for a in (r, x, y)]
+    dest = parts[0 if op in (CG_FWD, DIAG_FWD) else 1 if op in (CG_BACK0, DIAG_BACK0) else 2]
+    dest[...] = 0
+    lib().ora_set_abs_coeffs(1)
+    try:
+        part_op(op, parts[0], parts[1], parts[2], offs)
+    finally:
+        lib().ora_set_abs_coeffs(0)
+    return dest.real.copy()
+
+
+def vec_fwd_term_sums(xparts, yparts, maxl=-1, diag=False, nthreads=1):
+    """For every element of the product, the sum of the moduli of its terms, sum |C| |x| |y| (float64, real).
+    Error-analysis aid: the rounding error of a float32 evaluation of an element scales with this sum."""
+    lib().ora_set_abs_coeffs(1)
+    try:
+        return [p.real.copy() for p in vec_fwd(_moduli(xparts), _moduli(yparts), maxl, diag, nthreads)]
+    finally:
+        lib().ora_set_abs_coeffs(0)
+
+
+def vec_bwd_term_sums(gparts, xparts, yparts, diag=False, nthreads=1):
+    """The same for both gradients: sum |C| |g| |y| per element of xg and sum |C| |g| |x| per element of yg."""
+    lib().ora_set_abs_coeffs(1)
+    try:
+        xg, yg = vec_bwd(_moduli(gparts), _moduli(xparts), _moduli(yparts), diag, nthreads)
+        return [p.real.copy() for p in xg], [p.real.copy() for p in yg]
+    finally:
+        lib().ora_set_abs_coeffs(0)
+
+
 def spharm(l, x, batch=None):
     """(B or 1, 3, n) float32 vectors -> (B, 2l+1, n) complex64 spherical harmonics, the reference's add_spharm into zeros."""
     x = np.ascontiguousarray(x, dtype=np.float32)

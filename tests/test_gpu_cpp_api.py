@@ -44,8 +44,10 @@ def test_cpp_api_demo(tmp_path):
     assert r.shape == (3, 5, 32)
     assert U.gate_excess(r, ora.cg_fwd(x, y, 2)) <= 1.0
     wxg, wyg = ora.cg_bwd(g, x, y)
-    assert U.gate_excess(xg, wxg, rtol=1e-5, atol=1e-5) <= 1.0
-    assert U.gate_excess(yg, wyg, rtol=1e-5, atol=1e-5) <= 1.0
+    c = lambda a: a.astype(np.complex128)
+    exg, eyg = ora.cg_bwd(c(g), c(x), c(y))
+    U.assert_parity(xg, wxg, exg, ora.part_term_sums(ora.CG_BACK0, g, x, y), "C++ back0")
+    U.assert_parity(yg, wyg, eyg, ora.part_term_sums(ora.CG_BACK1, g, x, y), "C++ back1")
     u, v, w = t[6:9], t[9:12], t[12:]
     want = ora.vec_fwd(u, v, 2)
     assert [p.shape for p in w] == [p.shape for p in want]

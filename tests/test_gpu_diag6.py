@@ -48,11 +48,8 @@ def test_diag6_vec(cabi, B, tx, ty, maxl):
     seed = 900 + B
     xs = [U.seeded(seed + l, B, 2 * l + 1, n) for l, n in sorted(tx.items())]
     ys = [U.seeded(seed + 50 + l, B, 2 * l + 1, n) for l, n in sorted(ty.items())]
-    r32 = ora.vec_fwd(xs, ys, maxl, True)
-    r64 = ora.vec_fwd(c128(xs), c128(ys), maxl, True)
-    gs = [U.seeded(seed + 100 + i, *p.shape) for i, p in enumerate(r32)]
-    xg32, yg32 = ora.vec_bwd(gs, xs, ys, True)
-    xg64, yg64 = ora.vec_bwd(c128(gs), c128(xs), c128(ys), True)
+    O = U.VecOracle(xs, ys, maxl, True, gseed=seed + 100)
+    r32, gs = O.r32, O.gs
     dxs, dys, dgs = [U.dev(a) for a in xs], [U.dev(a) for a in ys], [U.dev(a) for a in gs]
     drs = [torch.full(p.shape, 7.0 + 1j, dtype=torch.complex64, device="cuda") for p in r32]
     cabi.so3vec_fwd(drs, dxs, dys, accumulate=False, diag=True)
@@ -63,12 +60,8 @@ def test_diag6_vec(cabi, B, tx, ty, maxl):
     assert cabi.last_path() == DIAG6
     torch.cuda.synchronize()
     tag = "B%d %s x %s maxl %d" % (B, tx, ty, maxl)
-    for a, b, c in zip(drs, r32, r64):
-        U.assert_parity(U.host(a), b, c, "fwd " + tag)
-    for a, b, c in zip(dxg, xg32, xg64):
-        U.assert_parity(U.host(a), b, c, "xg " + tag, slack=4.0)
-    for a, b, c in zip(dyg, yg32, yg64):
-        U.assert_parity(U.host(a), b, c, "yg " + tag, slack=4.0)
+    O.check_fwd([U.host(a) for a in drs], tag)
+    O.check_bwd([U.host(a) for a in dxg], [U.host(a) for a in dyg], tag)
     # accumulate mode adds on top of what is there
     drs2 = [a.clone() for a in drs]
     cabi.so3vec_fwd(drs2, dxs, dys, accumulate=True, diag=True)
@@ -78,8 +71,8 @@ def test_diag6_vec(cabi, B, tx, ty, maxl):
     torch.cuda.synchronize()
     for a, b in zip(drs2, drs):
         assert U.gate_excess(U.host(a), 2 * U.host(b)) <= 1.0
-    for a, b in zip(dxg2 + dyg2, dxg + dyg):
-        assert U.gate_excess(U.host(a), 2 * U.host(b), rtol=2e-5, atol=2e-5) <= 1.0
+    O.check_bwd_onto([U.host(a) for a in dxg2], [U.host(a) for a in dyg2], [U.host(a) for a in dxg],
+                     [U.host(a) for a in dyg], tag + " accumulated")
     # one gradient per call: the same kernel with the other one switched off, bit for bit the same sums
     dxg3 = [torch.full_like(a, 9.0) for a in dxg]
     dyg3 = [torch.full_like(a, 9.0) for a in dyg]
@@ -127,12 +120,9 @@ def test_diag_product_above_l6_is_split(cabi, B, tau, maxl):
     the other families, the gradients of the second part added on top of the first."""
     xs = [U.seeded(40 + l, B, 2 * l + 1, n) for l, n in sorted(tau.items())]
     ys = [U.seeded(60 + l, B, 2 * l + 1, n) for l, n in sorted(tau.items())]
-    r32 = ora.vec_fwd(xs, ys, maxl, True)
-    r64 = ora.vec_fwd(c128(xs), c128(ys), maxl, True)
+    O = U.VecOracle(xs, ys, maxl, True, gseed=80)
+    r32, gs = O.r32, O.gs
     assert max((p.shape[1] - 1) // 2 for p in r32) > 6
-    gs = [U.seeded(80 + i, *p.shape) for i, p in enumerate(r32)]
-    xg32, yg32 = ora.vec_bwd(gs, xs, ys, True)
-    xg64, yg64 = ora.vec_bwd(c128(gs), c128(xs), c128(ys), True)
     dxs, dys, dgs = [U.dev(a) for a in xs], [U.dev(a) for a in ys], [U.dev(a) for a in gs]
     for accumulate in (False, True):
         start = 5.0 - 1j if accumulate else 7.0 + 1j
@@ -144,8 +134,11 @@ def test_diag_product_above_l6_is_split(cabi, B, tau, maxl):
         cabi.so3vec_bwd(dxg, dyg, dgs, dxs, dys, accumulate=accumulate, diag=True)
         assert cabi.last_path() == DIAG6
         torch.cuda.synchronize()
-        off = start if accumulate else 0
-        for a, b, c in zip(drs, r32, r64):
-            U.assert_parity(U.host(a) - np.complex64(off), b, c, "fwd", slack=4.0)
-        for a, b, c in zip(dxg + dyg, xg32 + yg32, xg64 + yg64):
-            U.assert_parity(U.host(a) - np.complex64(off), b, c, "grad", slack=8.0)
+        hr, hxg, hyg = [U.host(a) for a in drs], [U.host(a) for a in dxg], [U.host(a) for a in dyg]
+        if accumulate:
+            full = lambda parts: [np.full(p.shape, start, dtype=np.complex64) for p in parts]
+            O.check_fwd_onto(hr, full(r32), "split Diag product onto a constant")
+            O.check_bwd_onto(hxg, hyg, full(xs), full(ys), "split Diag gradients onto a constant")
+        else:
+            O.check_fwd(hr, "split Diag product")
+            O.check_bwd(hxg, hyg, "split Diag gradients")

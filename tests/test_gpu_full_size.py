@@ -82,9 +82,8 @@ def test_full_size(cabi, name):
     tidx = torch.from_numpy(idx).cuda()
     hx = [U.host(t[tidx]) for t in xs]
     hy = [U.host(t[tidx]) for t in ys]
-    want = ora.vec_fwd(hx, hy, maxl, diag, nthreads=8)
-    for t, w in zip(rs, want):
-        assert U.gate_excess(U.host(t[tidx]), w) <= 1.0, name
+    O = U.VecOracle(hx, hy, maxl, diag, nthreads=8)
+    O.check_fwd([U.host(t[tidx]) for t in rs], name)
 
     # the adjoint identity on the whole batch, the product itself as the incoming gradient
     xg = [torch.empty_like(t) for t in xs]
@@ -96,15 +95,9 @@ def test_full_size(cabi, name):
     assert rr > 0
     assert abs(xx - rr) <= 2e-5 * rr, (name, rr, xx)
     assert abs(yy - rr) <= 2e-5 * rr, (name, rr, yy)
-    # and the gradients of the slices against the oracle (float64 beside float32, as for every long sum)
-    hg = [U.host(t[tidx]) for t in rs]
-    wxg, wyg = ora.vec_bwd(hg, hx, hy, diag, nthreads=8)
-    c128 = lambda L: [a.astype(np.complex128) for a in L]
-    xg64, yg64 = ora.vec_bwd(c128(hg), c128(hx), c128(hy), diag, nthreads=8)
-    for t, w, e in zip(xg, wxg, xg64):
-        U.assert_parity(U.host(t[tidx]), w, e, name + " xg", slack=4.0)
-    for t, w, e in zip(yg, wyg, yg64):
-        U.assert_parity(U.host(t[tidx]), w, e, name + " yg", slack=4.0)
+    # and the gradients of the slices against the oracle, every component under the rules of tests/gpu_util.py
+    O.set_gradient([U.host(t[tidx]) for t in rs], nthreads=8)
+    O.check_bwd([U.host(t[tidx]) for t in xg], [U.host(t[tidx]) for t in yg], name)
     del xg, yg
 
     if not bitwise:

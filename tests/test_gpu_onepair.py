@@ -44,10 +44,8 @@ def test_onepair_bwd(cabi, B, l1, n1, l2, n2, maxl, diag):
     seed = 1300 + B
     xs = [U.seeded(seed, B, 2 * l1 + 1, n1)]
     ys = [U.seeded(seed + 1, B, 2 * l2 + 1, n2)]
-    r32 = ora.vec_fwd(xs, ys, maxl, diag)
-    gs = [U.seeded(seed + 100 + i, *p.shape) for i, p in enumerate(r32)]
-    xg32, yg32 = ora.vec_bwd(gs, xs, ys, diag)
-    xg64, yg64 = ora.vec_bwd(c128(gs), c128(xs), c128(ys), diag)
+    O = U.VecOracle(xs, ys, maxl, diag, gseed=seed + 100)
+    gs = O.gs
     dxs, dys, dgs = [U.dev(a) for a in xs], [U.dev(a) for a in ys], [U.dev(a) for a in gs]
     dxg = [torch.full(a.shape, 3.0 - 2j, dtype=torch.complex64, device="cuda") for a in xs]
     dyg = [torch.full(a.shape, 3.0 - 2j, dtype=torch.complex64, device="cuda") for a in ys]
@@ -55,14 +53,13 @@ def test_onepair_bwd(cabi, B, l1, n1, l2, n2, maxl, diag):
     assert cabi.last_path() == ONEPAIR
     torch.cuda.synchronize()
     tag = "B%d (%d,%d)x(%d,%d) maxl %d diag %d" % (B, l1, n1, l2, n2, maxl, diag)
-    U.assert_parity(U.host(dxg[0]), xg32[0], xg64[0], "xg " + tag, slack=4.0)
-    U.assert_parity(U.host(dyg[0]), yg32[0], yg64[0], "yg " + tag, slack=4.0)
+    O.check_bwd([U.host(dxg[0])], [U.host(dyg[0])], tag)
     dxg2, dyg2 = [a.clone() for a in dxg], [a.clone() for a in dyg]
     cabi.so3vec_bwd(dxg2, dyg2, dgs, dxs, dys, accumulate=True, diag=diag)
     assert cabi.last_path() == ONEPAIR
     torch.cuda.synchronize()
-    for a, b in zip(dxg2 + dyg2, dxg + dyg):
-        assert U.gate_excess(U.host(a), 2 * U.host(b), rtol=2e-5, atol=2e-5) <= 1.0
+    O.check_bwd_onto([U.host(a) for a in dxg2], [U.host(a) for a in dyg2], [U.host(a) for a in dxg],
+                     [U.host(a) for a in dyg], tag + " accumulated")
 
 
 def test_onepair_leaves_the_rest_alone(cabi):
@@ -73,8 +70,8 @@ def test_onepair_leaves_the_rest_alone(cabi):
     xg = [torch.zeros_like(x[0])]
     cabi.so3vec_bwd(xg, None, g, x, y, accumulate=False)
     assert cabi.last_path() != ONEPAIR
-    wxg, _ = ora.vec_bwd([U.host(t) for t in g], [U.host(x[0])], [U.host(y[0])])
-    assert U.gate_excess(U.host(xg[0]), wxg[0], rtol=1e-4, atol=1e-4) <= 1.0
+    O = U.VecOracle([U.host(x[0])], [U.host(y[0])], -1, False, gs=[U.host(t) for t in g])
+    O.check_bwd([U.host(xg[0])], None, "one gradient alone")
     x11, y11 = [U.dev(U.seeded(3, 2, 23, 4))], [U.dev(U.seeded(4, 2, 23, 4))]
     w11 = ora.vec_fwd([U.host(x11[0])], [U.host(y11[0])], 3)
     g11 = [U.dev(U.seeded(20 + i, *p.shape)) for i, p in enumerate(w11)]

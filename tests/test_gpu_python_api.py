@@ -136,11 +136,8 @@ def test_vec_matches_oracle_and_uses_fused_kernels(G):
     torch.autograd.backward(list(z.parts.values()), g)
     assert cabi.last_path() == 2
     hg = [U.host(t) for t in g]
-    wxg, wyg = ora.vec_bwd(hg, hx, hy)
-    x64, y64, g64 = ([a.astype(np.complex128) for a in L] for L in (hx, hy, hg))
-    exg, eyg = ora.vec_bwd(g64, x64, y64)
-    for p, b, c in zip(list(x.parts.values()) + list(y.parts.values()), wxg + wyg, exg + eyg):
-        U.assert_parity(U.host(p.grad), b, c, "vec grad", slack=4.0)
+    O = U.VecOracle(hx, hy, 4, False, gs=hg)
+    O.check_bwd([U.host(p.grad) for p in x.parts.values()], [U.host(p.grad) for p in y.parts.values()], "vec grad")
 
 
 def test_errors_are_exceptions(G):

@@ -139,13 +139,8 @@ def test_vec_matches_oracle_and_uses_fused_kernels(G):
     torch.autograd.backward(list(z.parts.values()), g)
     assert cabi.last_path() == 2
     hg = [U.host(t).reshape(-1, t.shape[-2], t.shape[-1]) for t in g]
-    wxg, wyg = ora.vec_bwd(hg, hx, hy)
-    c128 = lambda L: [a.astype(np.complex128) for a in L]
-    xg64, yg64 = ora.vec_bwd(c128(hg), c128(hx), c128(hy))
-    for a, b, c in zip(flat(x.get_grad()), wxg, xg64):
-        U.assert_parity(a, b, c, "xg", slack=4.0)
-    for a, b, c in zip(flat(y.get_grad()), wyg, yg64):
-        U.assert_parity(a, b, c, "yg", slack=4.0)
+    O = U.VecOracle(hx, hy, 3, False, gs=hg)
+    O.check_bwd(flat(x.get_grad()), flat(y.get_grad()), "grid vec grad")
 
 
 def test_strided_views(G):

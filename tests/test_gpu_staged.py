@@ -2,7 +2,7 @@
 
 Each case checks the kernel family that ran (gelib_hip_last_path() == 3) and compares with the CPU oracle in
 float32 and float64, as the other GPU tests do.  One of the two backward forms adds partial sums into LDS images with
-float atomics, so its last bits can differ from run to run; the tolerance of assert_parity covers that.
+float atomics, so its last bits can differ from run to run; the parity rules of tests/gpu_util.py hold for any order.
 """
 import numpy as np
 import pytest
@@ -45,11 +45,8 @@ def c128(L):
 def run_vec(cabi, B, tx, ty, maxl, diag, seed, expect_bwd=STAGED):
     xs = [U.seeded(seed + l, B, 2 * l + 1, n) for l, n in sorted(tx.items())]
     ys = [U.seeded(seed + 50 + l, B, 2 * l + 1, n) for l, n in sorted(ty.items())]
-    r32 = ora.vec_fwd(xs, ys, maxl, diag)
-    r64 = ora.vec_fwd(c128(xs), c128(ys), maxl, diag)
-    gs = [U.seeded(seed + 100 + i, *p.shape) for i, p in enumerate(r32)]
-    xg32, yg32 = ora.vec_bwd(gs, xs, ys, diag)
-    xg64, yg64 = ora.vec_bwd(c128(gs), c128(xs), c128(ys), diag)
+    O = U.VecOracle(xs, ys, maxl, diag, gseed=seed + 100)
+    r32, gs = O.r32, O.gs
     dxs, dys, dgs = [U.dev(a) for a in xs], [U.dev(a) for a in ys], [U.dev(a) for a in gs]
     drs = [torch.full(p.shape, 7.0 + 1j, dtype=torch.complex64, device="cuda") for p in r32]
     cabi.so3vec_fwd(drs, dxs, dys, accumulate=False, diag=diag)
@@ -60,12 +57,8 @@ def run_vec(cabi, B, tx, ty, maxl, diag, seed, expect_bwd=STAGED):
     assert cabi.last_path() == expect_bwd
     torch.cuda.synchronize()
     tag = "B%d %s x %s maxl %d diag %d" % (B, tx, ty, maxl, diag)
-    for a, b, c in zip(drs, r32, r64):
-        U.assert_parity(U.host(a), b, c, "fwd " + tag)
-    for a, b, c in zip(dxg, xg32, xg64):
-        U.assert_parity(U.host(a), b, c, "xg " + tag, slack=4.0)
-    for a, b, c in zip(dyg, yg32, yg64):
-        U.assert_parity(U.host(a), b, c, "yg " + tag, slack=4.0)
+    O.check_fwd([U.host(a) for a in drs], tag)
+    O.check_bwd([U.host(a) for a in dxg], [U.host(a) for a in dyg], tag)
     # accumulate mode adds on top of what is there; one gradient at a time
     drs2 = [a.clone() for a in drs]
     cabi.so3vec_fwd(drs2, dxs, dys, accumulate=True, diag=diag)
@@ -76,8 +69,8 @@ def run_vec(cabi, B, tx, ty, maxl, diag, seed, expect_bwd=STAGED):
     torch.cuda.synchronize()
     for a, b in zip(drs2, drs):
         assert U.gate_excess(U.host(a), 2 * U.host(b)) <= 1.0
-    for a, b in zip(dxg2 + dyg2, dxg + dyg):
-        assert U.gate_excess(U.host(a), 2 * U.host(b), rtol=2e-5, atol=2e-5) <= 1.0
+    O.check_bwd_onto([U.host(a) for a in dxg2], [U.host(a) for a in dyg2], [U.host(a) for a in dxg],
+                     [U.host(a) for a in dyg], tag + " accumulated")
 
 
 VEC_CASES = [
@@ -150,13 +143,16 @@ def test_part_level_with_offset(cabi, diag, offs):
     b0 = cabi.so3part_diagcg_back0 if diag else cabi.so3part_cg_back0
     b1 = cabi.so3part_diagcg_back1 if diag else cabi.so3part_cg_back1
     r0 = U.seeded(4, B, 2 * l + 1, offs + nout + extra)
-    want = r0.copy()
-    want[:, :, offs:offs + nout] += ora.cg_fwd(x, y, l, diag)
+    op_f, op_0, op_1 = (ora.DIAG_FWD, ora.DIAG_BACK0, ora.DIAG_BACK1) if diag else (ora.CG_FWD, ora.CG_BACK0, ora.CG_BACK1)
+    want, want64 = r0.copy(), r0.astype(np.complex128)
+    ora.part_op(op_f, want, x, y, offs)            # the reference's add into what is there
+    ora.part_op(op_f, want64, x.astype(np.complex128), y.astype(np.complex128), offs)
+    Sr = ora.part_term_sums(op_f, r0, x, y, offs) + np.abs(r0)
     dr = U.dev(r0)
     fwd(dr, U.dev(x), U.dev(y), offs, accumulate=True)
     assert cabi.last_path() == STAGED
     torch.cuda.synchronize()
-    assert U.gate_excess(U.host(dr), want, rtol=2e-5, atol=2e-5) <= 1.0
+    U.assert_parity(U.host(dr), want, want64, Sr, "part fwd onto r0")
     # outside the block nothing moves
     assert np.array_equal(U.host(dr)[:, :, :offs], r0[:, :, :offs])
     assert np.array_equal(U.host(dr)[:, :, offs + nout:], r0[:, :, offs + nout:])
@@ -170,8 +166,8 @@ def test_part_level_with_offset(cabi, diag, offs):
     b1(dyg, U.dev(g), U.dev(x), offs, accumulate=False)
     assert cabi.last_path() == STAGED
     torch.cuda.synchronize()
-    U.assert_parity(U.host(dxg), xg32, xg64, "part back0", slack=4.0)
-    U.assert_parity(U.host(dyg), yg32, yg64, "part back1", slack=4.0)
+    U.assert_parity(U.host(dxg), xg32, xg64, ora.part_term_sums(op_0, g, x, y, offs), "part back0")
+    U.assert_parity(U.host(dyg), yg32, yg64, ora.part_term_sums(op_1, g, x, y, offs), "part back1")
 
 
 def test_broadcast_operand_and_grid(cabi):

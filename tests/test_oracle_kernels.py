@@ -234,3 +234,48 @@ def test_threads_match_serial():
     a = ora.cg_fwd(x, y, 4, nthreads=1)
     b = ora.cg_fwd(x, y, 4, nthreads=4)
     assert np.array_equal(a, b)
+
+
+@pytest.mark.parametrize("diag", [False, True])
+def test_term_sums_are_sums_of_term_moduli(diag):
+    """The error-analysis aid of the oracle (|C| on the moduli of the operands) against the definition, with sympy's
+    coefficients: einsum over |W|, |x|, |y| forward and |W|, |g|, |y| / |x| backward."""
+    rng = np.random.default_rng(21)
+    l1, l2, l, n1, n2 = 2, 1, 2, 3, (3 if diag else 2)
+    x, y = H.randc(rng, 2, 2 * l1 + 1, n1), H.randc(rng, 2, 2 * l2 + 1, n2)
+    C = np.abs(H.sympy_cg_matrix(l1, l2, l))
+    ax, ay = np.abs(x).astype(np.complex128), np.abs(y).astype(np.complex128)
+    want = H.einsum_cg(ax, ay, C, l, diag).real
+    got = ora.vec_fwd_term_sums([x], [y], l, diag)   # parts l = |l1-l2| .. maxl = l: the last one is l
+    np.testing.assert_allclose(got[-1], want, rtol=1e-6, atol=1e-12)
+    part = ora.part_term_sums(ora.DIAG_FWD if diag else ora.CG_FWD, np.zeros_like(got[-1], dtype=np.complex64), x, y)
+    np.testing.assert_allclose(part, want, rtol=1e-6, atol=1e-12)
+    g = H.randc(rng, *want.shape)
+    wx, wy = H.einsum_cg_bwd(np.abs(g).astype(np.complex128), ax, ay, C, diag)
+    sx = ora.part_term_sums(ora.DIAG_BACK0 if diag else ora.CG_BACK0, g, x, y)
+    sy = ora.part_term_sums(ora.DIAG_BACK1 if diag else ora.CG_BACK1, g, x, y)
+    np.testing.assert_allclose(sx, wx.real, rtol=1e-6, atol=1e-12)
+    np.testing.assert_allclose(sy, wy.real, rtol=1e-6, atol=1e-12)
+    # every term sum bounds the modulus of the element it belongs to, and the switch is off again afterwards
+    r = ora.cg_fwd(x, y, l, diag)
+    assert np.all(np.abs(r) <= want * (1 + 1e-6) + 1e-6)
+    assert np.any(ora.cg_matrix(l1, l2, l) < 0)
+
+
+def test_parity_rules_accept_and_reject():
+    """Host logic of the per-component parity check (tests/gpu_util.py): rule A, rule B, rule C and a rejection."""
+    from tests import gpu_util as U
+    e = np.array([100.0 + 0j, 0.001 + 0j, 0.001 + 0j, 0.001 + 0j], dtype=np.complex128)
+    c = np.array([100.0005 + 0j, 0.00130 + 0j, 0.001 + 0j, 0.001 + 0j], dtype=np.complex64)   # second: CPU off by 3e-4
+    S = np.array([500.0, 500.0, 500.0, 500.0])
+    g = np.array([100.0008 + 0j,      # A: within 1e-5 relative of the CPU value
+                  0.00090 + 0j,       # B: the CPU misses its own gate, the GPU is closer to the exact value
+                  0.00105 + 0j,       # C: 5e-5 from exact, under 1e-6 + 2 eps32 * 500 = 1.2e-4
+                  0.00150 + 0j],      # rejected: 5e-4 from exact and from the CPU
+                 dtype=np.complex64)
+    rep = U.parity_counts(g, c, e, S)
+    assert rep["rejected"] == 1 and rep["first_rejected"] == 6
+    assert rep["by_rule_B"] == 1 / 8 and rep["by_rule_C"] == 1 / 8
+    with pytest.raises(AssertionError):
+        U.assert_parity(g, c, e, S, "demo")
+    U.assert_parity(g[:3], c[:3], e[:3], S[:3], "demo")

@@ -17,7 +17,9 @@ SYMBOLS = [
     "gelib_hip_so3part_diagcg_fwd", "gelib_hip_so3part_diagcg_back0", "gelib_hip_so3part_diagcg_back1",
     "gelib_hip_so3vec_cg_fwd", "gelib_hip_so3vec_cg_bwd", "gelib_hip_so3vec_diagcg_fwd",
     "gelib_hip_so3vec_diagcg_bwd", "gelib_hip_so3part_spharm", "gelib_hip_gather_map_create",
-    "gelib_hip_gather_map_destroy", "gelib_hip_part_gather", "gelib_hip_part_mix_channels", "gelib_hip_part_mix_channels_wgrad", "gelib_hip_set_option", "gelib_hip_last_path",
+    "gelib_hip_gather_map_destroy", "gelib_hip_part_gather", "gelib_hip_part_mix_channels",
+    "gelib_hip_part_mix_channels_wgrad", "gelib_hip_part_mix_workspace_bytes", "gelib_hip_set_option",
+    "gelib_hip_last_path",
     "gelib_hip_malloc", "gelib_hip_free", "gelib_hip_memcpy", "gelib_hip_memset", "gelib_hip_synchronize",
 ]
 
@@ -70,10 +72,13 @@ def lib():
                                             ctypes.c_void_p]
         L.gelib_hip_part_mix_channels.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64,
                                                   ctypes.c_int, ctypes.c_int, ctypes.c_int64, ctypes.c_int64,
-                                                  ctypes.c_int, ctypes.c_void_p]
+                                                  ctypes.c_int, ctypes.c_void_p, ctypes.c_uint64, ctypes.c_void_p]
         L.gelib_hip_part_mix_channels_wgrad.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
                                                         ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.c_int64,
-                                                        ctypes.c_int64, ctypes.c_void_p]
+                                                        ctypes.c_int64, ctypes.c_void_p, ctypes.c_uint64,
+                                                        ctypes.c_void_p]
+        L.gelib_hip_part_mix_workspace_bytes.restype = ctypes.c_uint64
+        L.gelib_hip_part_mix_workspace_bytes.argtypes = [ctypes.c_int, ctypes.c_int64, ctypes.c_int, ctypes.c_int]
         L.gelib_hip_set_option.argtypes = [ctypes.c_char_p, ctypes.c_int]
         _lib = L
     return _lib
@@ -226,6 +231,15 @@ def mix_channels_ok(x):
     return x.is_contiguous() and x.shape[-1] > 0 and x.shape[-1] % 2 == 0 and x.data_ptr() % 16 == 0
 
 
+def mix_workspace(kind, rows, n_in, n_out, device):
+    """The workspace a channel-mixing call needs (kind 0: part_mix_channels, 1: part_mix_channels_wgrad), taken from
+    torch's caching allocator: it is stream-ordered, so the buffer is not handed to anybody else before the kernels
+    queued on the current stream have read it, and the library itself never allocates."""
+    import torch
+    nbytes = int(lib().gelib_hip_part_mix_workspace_bytes(kind, rows, n_in, n_out))
+    return torch.empty(max(nbytes, 16), dtype=torch.uint8, device=device), nbytes
+
+
 def part_mix_channels(r, x, w, adjoint=False):
     """r[..., o] = sum_c x[..., c] V[c, o] with V = w (n_in, n_out), or V = w^H for w (n_out, n_in) when adjoint.
     r and x are contiguous complex64 tensors that differ only in their last extent."""
@@ -235,8 +249,9 @@ def part_mix_channels(r, x, w, adjoint=False):
     if not (r.is_contiguous() and x.is_contiguous() and w.is_contiguous()):
         raise ValueError("contiguous tensors are needed")
     rows = x.numel() // n_in if n_in else 0
+    ws, nbytes = mix_workspace(0, rows, n_in, n_out, r.device)
     check(lib().gelib_hip_part_mix_channels(r.data_ptr(), x.data_ptr(), w.data_ptr(), rows, n_in, n_out, n_out, n_in,
-                                            int(adjoint), _stream(r)))
+                                            int(adjoint), ws.data_ptr(), nbytes, _stream(r)))
 
 
 def part_mix_channels_wgrad(wg, x, g):
@@ -247,8 +262,9 @@ def part_mix_channels_wgrad(wg, x, g):
     if not (wg.is_contiguous() and x.is_contiguous() and g.is_contiguous()):
         raise ValueError("contiguous tensors are needed")
     rows = x.numel() // n_in if n_in else 0
+    ws, nbytes = mix_workspace(1, rows, n_in, n_out, wg.device)
     check(lib().gelib_hip_part_mix_channels_wgrad(wg.data_ptr(), x.data_ptr(), g.data_ptr(), rows, n_in, n_out, n_in,
-                                                  n_out, _stream(wg)))
+                                                  n_out, ws.data_ptr(), nbytes, _stream(wg)))
 
 
 def set_option(name, value):

@@ -6,6 +6,7 @@
 #include <algorithm>
 #include <cstdio>
 #include <cstring>
+#include <mutex>
 #include <string>
 #include <vector>
 
@@ -41,7 +42,7 @@ struct View {  // one validated descriptor
 int check_desc(const gelib_part_desc *d, View &v) {
   if (!d) return GELIB_HIP_ERR_NULL;
   for (int k = 0; k < 5; k++)
-    if (d->dims[k] < 0) return GELIB_HIP_ERR_ARG;
+    if (d->dims[k] < 0 || d->strides[k] < 0) return GELIB_HIP_ERR_ARG;   // whatever "check_pointers" says
   if (d->dims[3] % 2 != 1) return GELIB_HIP_ERR_ODD_DIM;
   if (d->dims[3] > 2 * (4 * kMaxL) + 1 || d->dims[4] > 0x7fffffffLL) return GELIB_HIP_ERR_PARTS;
   v.d = d;
@@ -50,6 +51,35 @@ int check_desc(const gelib_part_desc *d, View &v) {
   const bool empty = d->dims[0] == 0 || d->dims[1] == 0 || d->dims[2] == 0 || d->dims[4] == 0;
   if (!d->ptr && !empty) return GELIB_HIP_ERR_NULL;
   return GELIB_HIP_OK;
+}
+
+// Allocations that have passed the driver's checks: [base, base + size) on a device.  A view that lies inside one of
+// them passes without any driver call (a product call checks 15 to 30 pointers, most of them in the same few
+// allocations of a caching allocator, call after call).  An entry lives until it is pushed out by newer ones; memory
+// that is freed and handed out again by the driver at the same address as a different kind is not noticed, which is
+// the price of not asking every time ("check_pointers" 2 asks every time).
+struct KnownRange {
+  const char *base;
+  size_t size;
+  int device;
+};
+constexpr int kKnownRanges = 64;
+std::mutex g_known_mutex;
+KnownRange g_known[kKnownRanges];
+int g_known_count = 0, g_known_next = 0;
+
+bool known_range(const char *p, const char *end, int dev) {
+  std::lock_guard<std::mutex> lock(g_known_mutex);
+  for (int i = 0; i < g_known_count; i++)
+    if (g_known[i].device == dev && p >= g_known[i].base && end <= g_known[i].base + g_known[i].size) return true;
+  return false;
+}
+
+void remember_range(const char *base, size_t size, int dev) {
+  std::lock_guard<std::mutex> lock(g_known_mutex);
+  g_known[g_known_next] = {base, size, dev};
+  g_known_next = (g_known_next + 1) % kKnownRanges;
+  if (g_known_count < kKnownRanges) g_known_count++;
 }
 
 // The farthest element of the view must lie inside the allocation that holds ptr, and that allocation must be
@@ -62,6 +92,10 @@ int check_range(const void *ptr, const int64_t dims[5], const int64_t strides[5]
     if (strides[k] < 0) return GELIB_HIP_ERR_ARG;
     span += (dims[k] - 1) * strides[k];
   }
+  const char *end = (const char *)ptr + (span + 1) * (long long)elem_bytes;
+  int dev = 0;
+  const bool have_dev = hipGetDevice(&dev) == hipSuccess;   // no driver call: the runtime keeps it per thread
+  if (g_check_pointers == 1 && have_dev && known_range((const char *)ptr, end, dev)) return GELIB_HIP_OK;
   hipPointerAttribute_t attr;
   hipError_t e = hipPointerGetAttributes(&attr, ptr);
   if (e != hipSuccess) {
@@ -69,8 +103,7 @@ int check_range(const void *ptr, const int64_t dims[5], const int64_t strides[5]
     return GELIB_HIP_ERR_DEVICE;
   }
   if (attr.type != hipMemoryTypeDevice && attr.type != hipMemoryTypeManaged) return GELIB_HIP_ERR_DEVICE;
-  int dev = 0;
-  if (hipGetDevice(&dev) == hipSuccess && attr.type == hipMemoryTypeDevice && attr.device != dev) return GELIB_HIP_ERR_DEVICE;
+  if (have_dev && attr.type == hipMemoryTypeDevice && attr.device != dev) return GELIB_HIP_ERR_DEVICE;
   hipDeviceptr_t base = nullptr;
   size_t size = 0;
   e = hipMemGetAddressRange(&base, &size, (hipDeviceptr_t)ptr);
@@ -78,8 +111,8 @@ int check_range(const void *ptr, const int64_t dims[5], const int64_t strides[5]
     (void)hipGetLastError();
     return GELIB_HIP_OK;  // range unknown (e.g. a suballocator the runtime cannot see): type check above stands
   }
-  const char *end = (const char *)ptr + (span + 1) * (long long)elem_bytes;
   if (end > (const char *)base + size) return GELIB_HIP_ERR_DEVICE;
+  if (have_dev) remember_range((const char *)base, size, dev);
   return GELIB_HIP_OK;
 }
 
@@ -99,6 +132,14 @@ PartDev to_dev(const gelib_part_desc *d, const long long E[3], long long own[3])
   p.sm = d->strides[3];
   p.sc = d->strides[4];
   return p;
+}
+
+// A destination whose view repeats memory (extent > 1 with stride 0, e.g. an expanded torch view) would be written by
+// many threads at once; a destination that is to be summed over a dimension has extent 1 there instead.
+int check_dest(const gelib_part_desc *d) {
+  for (int k = 0; k < 5; k++)
+    if (d->dims[k] > 1 && d->strides[k] == 0) return GELIB_HIP_ERR_BROADCAST_DEST;
+  return GELIB_HIP_OK;
 }
 
 // dims equal or 1 along each leading dimension; dimension 0 is the batch, 1..2 the grid
@@ -156,6 +197,7 @@ int part_entry(Kind kind, bool diag, const gelib_part_desc *r, const gelib_part_
   PartOp op;
   int rc = make_part_op(r, x, y, offs, diag, op);
   if (rc) return rc;
+  if ((rc = check_dest(kind == kFwd ? r : (kind == kBack0 ? x : y)))) return rc;
   if ((rc = check_pointer(r)) || (rc = check_pointer(x)) || (rc = check_pointer(y))) return rc;
   if (op.E[0] * op.E[1] * op.E[2] == 0 || op.nout == 0) return GELIB_HIP_OK;
   hipStream_t s = (hipStream_t)stream;
@@ -337,6 +379,8 @@ int vec_fwd_entry(bool diag, int nr, const gelib_part_desc *r, int nx, const gel
   VecPlan plan;
   if ((rc = build_vec_plan(diag, R, X, Y, plan))) return rc;
   for (auto &v : R)
+    if ((rc = check_dest(v.d))) return rc;
+  for (auto &v : R)
     if ((rc = check_pointer(v.d))) return rc;
   for (auto &v : X)
     if ((rc = check_pointer(v.d))) return rc;
@@ -455,6 +499,9 @@ int vec_bwd_entry(bool diag, const gelib_part_desc *xg, const gelib_part_desc *y
     for (auto &v : YG) all.push_back(v.d);
     if ((rc = reconcile(all.data(), (int)all.size(), plan.E))) return rc;
   }
+  for (auto *L : {&XG, &YG})
+    for (auto &v : *L)
+      if ((rc = check_dest(v.d))) return rc;
   for (auto *L : {&G, &X, &Y, &XG, &YG})
     for (auto &v : *L)
       if ((rc = check_pointer(v.d))) return rc;
@@ -503,8 +550,9 @@ const char *gelib_hip_strerror(int status) {
     case GELIB_HIP_ERR_DEVICE: return "SO3part must be on GPU (pointer is not device memory of the current device, or the view overruns its allocation)";
     case GELIB_HIP_ERR_PARTS: return "too many parts, a repeated l, l above the supported maximum, or gradient parts that do not match their operand";
     case GELIB_HIP_ERR_RUNTIME: return "HIP runtime error";
-    case GELIB_HIP_ERR_BROADCAST_DEST: return "cannot overwrite a broadcast destination";
+    case GELIB_HIP_ERR_BROADCAST_DEST: return "the destination repeats memory (a dimension of extent > 1 with stride 0)";
     case GELIB_HIP_ERR_ARG: return "malformed argument";
+    case GELIB_HIP_ERR_WORKSPACE: return "workspace missing, not 16-byte aligned or too small";
   }
   return "unknown status";
 }
@@ -705,7 +753,8 @@ int gelib_hip_part_gather(const gelib_part_desc *r, const gelib_part_desc *x, co
 
 // ---- channel mixing (the linear layer that consumes a product) ------------------------------------------------------
 int gelib_hip_part_mix_channels(void *r, const void *x, const void *w, int64_t rows, int n_in, int n_out,
-                                int64_t r_row_stride, int64_t x_row_stride, int adjoint, void *stream) {
+                                int64_t r_row_stride, int64_t x_row_stride, int adjoint, void *workspace,
+                                uint64_t workspace_bytes, void *stream) {
   t_last_path = kPathNone;
   if (rows < 0 || n_in < 0 || n_out < 0 || r_row_stride < n_out || x_row_stride < n_in) return GELIB_HIP_ERR_ARG;
   if (rows == 0 || n_out == 0) return GELIB_HIP_OK;
@@ -720,14 +769,17 @@ int gelib_hip_part_mix_channels(void *r, const void *x, const void *w, int64_t r
   if ((rc = check_range(r, rd, rst, 2 * sizeof(float))) || (rc = check_range(x, xd, xst, 2 * sizeof(float))) ||
       (rc = check_range(w, wd, wst, 2 * sizeof(float))))
     return rc;
+  const int64_t sd[5] = {(int64_t)workspace_bytes, 1, 1, 1, 1}, sst[5] = {1, 0, 0, 0, 0};
+  if (workspace && workspace_bytes && (rc = check_range(workspace, sd, sst, 1))) return rc;
   t_last_path = kPathGeneric;
   rc = launch_mix((float2 *)r, (const float2 *)x, (const float2 *)w, rows, n_in, n_out, x_row_stride, r_row_stride,
-                  adjoint != 0, (hipStream_t)stream);
+                  adjoint != 0, (float *)workspace, (size_t)workspace_bytes, (hipStream_t)stream);
   return rc == 11 ? GELIB_HIP_ERR_ARG : rc;
 }
 
 int gelib_hip_part_mix_channels_wgrad(void *wg, const void *x, const void *g, int64_t rows, int n_in, int n_out,
-                                      int64_t x_row_stride, int64_t g_row_stride, void *stream) {
+                                      int64_t x_row_stride, int64_t g_row_stride, void *workspace,
+                                      uint64_t workspace_bytes, void *stream) {
   t_last_path = kPathNone;
   if (rows < 0 || n_in < 0 || n_out < 0 || x_row_stride < n_in || g_row_stride < n_out) return GELIB_HIP_ERR_ARG;
   if (n_in == 0 || n_out == 0) return GELIB_HIP_OK;
@@ -740,10 +792,19 @@ int gelib_hip_part_mix_channels_wgrad(void *wg, const void *x, const void *g, in
   if ((rc = check_range(wg, wd, wst, 2 * sizeof(float))) || (rc = check_range(x, xd, xst, 2 * sizeof(float))) ||
       (rc = check_range(g, gd, gst, 2 * sizeof(float))))
     return rc;
+  const int64_t sd[5] = {(int64_t)workspace_bytes, 1, 1, 1, 1}, sst[5] = {1, 0, 0, 0, 0};
+  if (workspace && workspace_bytes && (rc = check_range(workspace, sd, sst, 1))) return rc;
   t_last_path = kPathGeneric;
   rc = launch_mix_wgrad((float2 *)wg, (const float2 *)x, (const float2 *)g, rows, n_in, n_out, x_row_stride,
-                        g_row_stride, (hipStream_t)stream);
+                        g_row_stride, (float *)workspace, (size_t)workspace_bytes, (hipStream_t)stream);
   return rc == 11 ? GELIB_HIP_ERR_ARG : rc;
+}
+
+uint64_t gelib_hip_part_mix_workspace_bytes(int kind, int64_t rows, int n_in, int n_out) {
+  if (rows <= 0 || n_in <= 0 || n_out <= 0) return 0;
+  if (kind == 0) return mix_workspace_bytes(n_in, n_out);
+  if (kind == 1) return mix_wgrad_workspace_bytes(rows, n_in, n_out);
+  return 0;
 }
 
 int gelib_hip_malloc(void **ptr, uint64_t bytes) {

@@ -60,12 +60,16 @@ int launch_gather(float2 *r, const float2 *x, const long long rs[5], const long 
                   const int *row_ptr, const int *sources, bool accumulate, hipStream_t s);
 
 // ---- channel mixing on the matrix cores (mix.hip): r[row, :] = x[row, :] V, V = W (n_in, n_out) or W^H for W (n_out, n_in);
-// strides in complex elements.  Returns 0, 10 (a HIP call failed) or 11 (n_in odd or rows of x not 16-byte aligned)
+// strides in complex elements.  Returns 0, 10 (a HIP call failed), 11 (n_in odd or rows of x not 16-byte aligned) or 13
+// (workspace missing, misaligned or smaller than mix_workspace_bytes).  The library allocates nothing here: the re-packed
+// matrix goes into the caller's workspace.
+size_t mix_workspace_bytes(int n_in, int n_out);
 int launch_mix(float2 *r, const float2 *x, const float2 *w, long long rows, int n_in, int n_out, long long xs,
-               long long rs, bool adjoint, hipStream_t s);
-// wg (n_in, n_out) = sum over the rows of conj(x[row, :])^T g[row, :]
+               long long rs, bool adjoint, float *ws, size_t ws_bytes, hipStream_t s);
+// wg (n_in, n_out) = sum over the rows of conj(x[row, :])^T g[row, :]; the workspace holds the partial sums
+size_t mix_wgrad_workspace_bytes(long long rows, int n_in, int n_out);
 int launch_mix_wgrad(float2 *wg, const float2 *x, const float2 *g, long long rows, int n_in, int n_out, long long xs,
-                     long long gs, hipStream_t s);
+                     long long gs, float *ws, size_t ws_bytes, hipStream_t s);
 int mix_set_option(const char *name, int value);   // "mix_long": 0 keeps long rows off the LDS-staged kernel
 
 }  // namespace gelib_hip

@@ -31,9 +31,14 @@ struct StagedTriple {
   int cg_back1;     // m2 ascending, then m1 ascending           (gradient of y)
 };
 
+// Part lists the kernels of this family take in their argument block (the block has to stay under 4 KB); vectors
+// with more parts run on the shape-agnostic kernels.
+constexpr int kStagedMaxParts = 16;
+constexpr int kStagedMaxOutParts = 40;
+
 struct StagedArgs {
-  FastPart x[kMaxParts], y[kMaxParts], xg[kMaxParts], yg[kMaxParts];
-  FastPart r[kMaxOutParts];  // product (forward) or its gradient (backward)
+  FastPart x[kStagedMaxParts], y[kStagedMaxParts], xg[kStagedMaxParts], yg[kStagedMaxParts];
+  FastPart r[kStagedMaxOutParts];  // product (forward) or its gradient (backward)
   const StagedTriple *triples;
   const float *bank;
   // Striped backward kernels: (first, count, log2 of slots per cell) for every x part, then for every y part, then
@@ -50,7 +55,7 @@ struct StagedArgs {
   int xsize, ysize;  // complex elements of one cell's packed x / y image
   int cpb;           // cells per block
   int lds_coeffs;    // forward: floats of the coefficient stream staged in LDS behind the operands (0 = read from memory)
-  int xrows[kMaxParts], yrows[kMaxParts];
+  int xrows[kStagedMaxParts], yrows[kStagedMaxParts];
 };
 
 // tile: adjacent output channels per lane (1, 2 or 4); threads: a multiple of 64 up to 1024

@@ -254,7 +254,7 @@ void fill_args(StagedArgs &a, const DevicePlan &plan, const FastLists &f, const 
 
 bool sizes_ok(const std::vector<std::pair<int, int>> &xs, const std::vector<std::pair<int, int>> &ys,
               const std::vector<int> &rls) {
-  if (xs.size() > (size_t)kMaxParts || ys.size() > (size_t)kMaxParts || rls.size() > (size_t)kMaxOutParts) return false;
+  if (xs.size() > (size_t)kStagedMaxParts || ys.size() > (size_t)kStagedMaxParts || rls.size() > (size_t)kStagedMaxOutParts) return false;
   long long xsize = 0, ysize = 0;
   for (auto &v : xs) xsize += (2LL * v.first + 1) * v.second;
   for (auto &v : ys) ysize += (2LL * v.first + 1) * v.second;

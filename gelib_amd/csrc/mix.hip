@@ -24,7 +24,6 @@
 // every row) at a time: lane (i, h) reads the 16 floats of its row that start at 16 h.
 #include <algorithm>
 #include <map>
-#include <mutex>
 #include <string>
 
 #include "cg_common.h"
@@ -407,34 +406,6 @@ __global__ void __launch_bounds__(64, 8) mix_wide_kernel(const WideArgs w) {
   }
 }
 
-// the packed matrix of a call lives in a buffer kept per (device, stream): calls on one stream are ordered, calls on
-// different streams do not share a buffer
-struct Workspace {
-  float *ptr = nullptr;
-  size_t bytes = 0;
-};
-std::mutex g_ws_mutex;
-std::map<std::pair<int, hipStream_t>, Workspace> g_ws;
-
-float *workspace(size_t bytes, hipStream_t s) {
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess) return nullptr;
-  std::lock_guard<std::mutex> lock(g_ws_mutex);
-  Workspace &w = g_ws[{dev, s}];
-  if (w.bytes < bytes) {
-    if (w.ptr) {
-      if (hipStreamSynchronize(s) != hipSuccess) return nullptr;   // an earlier call on this stream may still read it
-      (void)hipFree(w.ptr);
-      w.ptr = nullptr;
-      w.bytes = 0;
-    }
-    const size_t want = std::max(bytes, (size_t)1 << 20);
-    if (hipMalloc((void **)&w.ptr, want) != hipSuccess) return nullptr;
-    w.bytes = want;
-  }
-  return w.ptr;
-}
-
 int g_mix_long = 1;
 int g_mix_wide_store = 1;
 int g_mix_wide = 1;
@@ -449,10 +420,28 @@ void launch(const MixArgs &a, hipStream_t s) {
 
 }  // namespace
 
+// Floats of the re-packed matrix: nq steps of (2 << lg_p) floats of a row, ct_total tiles of 32 output floats.
+static long long packed_floats(int n_in, int n_out, int lg_p) {
+  const int k2 = 2 * n_in, tiles = (2 * n_out + 31) / 32;
+  const int ctw = tiles > 2 ? 4 : tiles;
+  const long long ct_total = (tiles + ctw - 1) / ctw * ctw;
+  const long long nq = (k2 + (2 << lg_p) - 1) / (2 << lg_p);
+  return (nq * ct_total * 64) << lg_p;
+}
+
+// Bytes of workspace launch_mix needs at most for these sizes (the long-row kernel packs in steps of 128 floats, the
+// others in steps of 32; which one runs also depends on the row stride, so the larger of the two is asked for).
+size_t mix_workspace_bytes(int n_in, int n_out) {
+  if (n_in <= 0 || n_out <= 0) return 0;
+  return sizeof(float) * (size_t)std::max(packed_floats(n_in, n_out, 4), packed_floats(n_in, n_out, 6));
+}
+
 // 0 on success, 10 when a HIP call fails, 11 when the shape is not one this kernel takes (n_in odd, strides that break
-// the 16-byte alignment of a row)
+// the 16-byte alignment of a row), 13 when the workspace is missing, not 16-byte aligned or too small.  The workspace
+// (device memory, mix_workspace_bytes) receives the re-packed matrix; the kernels of this call read it, so the caller
+// keeps it until they have run.
 int launch_mix(float2 *r, const float2 *x, const float2 *w, long long rows, int n_in, int n_out, long long xs,
-               long long rs, bool adjoint, hipStream_t s) {
+               long long rs, bool adjoint, float *ws, size_t ws_bytes, hipStream_t s) {
   if (rows == 0 || n_out == 0) return 0;
   if (n_in <= 0 || (n_in & 1) || (xs & 1) || ((uintptr_t)x & 15)) return 11;
   if (rows > (1LL << 38)) return 11;
@@ -474,8 +463,8 @@ int launch_mix(float2 *r, const float2 *x, const float2 *w, long long rows, int 
   const int lg_p = long_rows ? 6 : 4;
   a.nq = (a.k2 + (2 << lg_p) - 1) / (2 << lg_p);
   const long long total = ((long long)a.nq * a.ct_total * 64) << lg_p;
-  float *vp = workspace((size_t)total * sizeof(float), s);
-  if (!vp) return 10;
+  if (!ws || ((uintptr_t)ws & 15) || ws_bytes < (size_t)total * sizeof(float)) return 13;
+  float *vp = ws;
   a.vp = vp;
   hipLaunchKernelGGL(pack_kernel, dim3((unsigned)std::min<long long>((total + 255) / 256, 4096)), dim3(256), 0, s, w, vp,
                      n_in, n_out, a.nq, a.ct_total, adjoint ? 1 : 0, lg_p);
@@ -646,12 +635,52 @@ __global__ void __launch_bounds__(256) wgrad_sum_kernel(const float *part, float
   }
 }
 
-// 0, 10 or 11 as launch_mix
+namespace {
+struct WgradPlan {
+  int ew, jt, u, tiles, jt_total, kgroups;
+  long long nranges, rows_per_range, pitch;
+};
+WgradPlan plan_wgrad(long long rows, int n_in, int n_out) {
+  WgradPlan p;
+  const int k2 = 2 * n_in, n2 = 2 * n_out;
+  p.tiles = (n2 + 31) / 32;
+  p.ew = p.tiles <= 2 ? 4 : 2;
+  p.jt = p.tiles == 1 ? 1 : (p.tiles == 2 ? 2 : 4);
+  p.u = p.tiles == 1 ? 16 : 8;
+  p.jt_total = (p.tiles + p.jt - 1) / p.jt * p.jt;
+  p.kgroups = (k2 + 32 * p.ew - 1) / (32 * p.ew);
+  // enough waves to fill the chip a few times over, every range a whole number of steps and not empty
+  const long long waves_per_range = (long long)p.kgroups * (p.jt_total / p.jt);
+  long long nranges = std::max<long long>(1, std::min<long long>(4096 / waves_per_range, rows / (8LL * p.u)));
+  nranges = std::min<long long>(nranges, 256);
+  p.rows_per_range = ((rows + nranges - 1) / nranges + 2 * p.u - 1) / (2 * p.u) * (2 * p.u);
+  p.nranges = (rows + p.rows_per_range - 1) / p.rows_per_range;
+  p.pitch = 32LL * p.jt_total;
+  return p;
+}
+
+__global__ void zero_fill_kernel(float2 *p, long long n) {
+  for (long long i = blockIdx.x * 256LL + threadIdx.x; i < n; i += 256LL * gridDim.x) p[i] = make_float2(0.f, 0.f);
+}
+}  // namespace
+
+// Bytes of workspace launch_mix_wgrad needs: the partial sums of the row ranges.
+size_t mix_wgrad_workspace_bytes(long long rows, int n_in, int n_out) {
+  if (rows <= 0 || n_in <= 0 || n_out <= 0) return 0;
+  const WgradPlan p = plan_wgrad(rows, n_in, n_out);
+  return sizeof(float) * (size_t)(p.nranges * 2 * n_in * p.pitch);
+}
+
+// 0, 10, 11 or 13 as launch_mix; the workspace (mix_wgrad_workspace_bytes) holds the partial sums of the row ranges
 int launch_mix_wgrad(float2 *wg, const float2 *x, const float2 *g, long long rows, int n_in, int n_out, long long xs,
-                     long long gs, hipStream_t s) {
+                     long long gs, float *ws, size_t ws_bytes, hipStream_t s) {
   if (n_in == 0 || n_out == 0) return 0;
   if ((n_in & 1) || (xs & 1) || ((uintptr_t)x & 15) || rows > (1LL << 38)) return 11;
-  if (rows == 0) return hipMemsetAsync(wg, 0, sizeof(float2) * (size_t)n_in * n_out, s) == hipSuccess ? 0 : 10;
+  if (rows == 0) {   // a fill kernel, not a memset node: callers may capture this call into a graph
+    const long long n = (long long)n_in * n_out;
+    hipLaunchKernelGGL(zero_fill_kernel, dim3((unsigned)std::min<long long>((n + 255) / 256, 1024)), dim3(256), 0, s, wg, n);
+    return hipGetLastError() == hipSuccess ? 0 : 10;
+  }
   WgradArgs a;
   a.x = (const float *)x;
   a.g = (const float *)g;
@@ -660,19 +689,14 @@ int launch_mix_wgrad(float2 *wg, const float2 *x, const float2 *g, long long row
   a.gs = 2 * gs;
   a.k2 = 2 * n_in;
   a.n2 = 2 * n_out;
-  const int tiles = (a.n2 + 31) / 32;
-  const int ew = tiles <= 2 ? 4 : 2, jt = tiles == 1 ? 1 : (tiles == 2 ? 2 : 4), u = tiles == 1 ? 16 : 8;
-  a.jt_total = (tiles + jt - 1) / jt * jt;
-  a.kgroups = (a.k2 + 32 * ew - 1) / (32 * ew);
-  // enough waves to fill the chip a few times over, every range a whole number of steps and not empty
-  const long long waves_per_range = (long long)a.kgroups * (a.jt_total / jt);
-  long long nranges = std::max<long long>(1, std::min<long long>(4096 / waves_per_range, rows / (8LL * u)));
-  nranges = std::min<long long>(nranges, 256);
-  a.rows_per_range = ((rows + nranges - 1) / nranges + 2 * u - 1) / (2 * u) * (2 * u);
-  nranges = (rows + a.rows_per_range - 1) / a.rows_per_range;
-  const long long pitch = 32LL * a.jt_total;
-  float *part = workspace((size_t)nranges * a.k2 * pitch * sizeof(float), s);
-  if (!part) return 10;
+  const WgradPlan pl = plan_wgrad(rows, n_in, n_out);
+  const int tiles = pl.tiles, jt = pl.jt;
+  a.jt_total = pl.jt_total;
+  a.kgroups = pl.kgroups;
+  a.rows_per_range = pl.rows_per_range;
+  const long long nranges = pl.nranges, pitch = pl.pitch;
+  if (!ws || ((uintptr_t)ws & 15) || ws_bytes < (size_t)(nranges * a.k2 * pitch) * sizeof(float)) return 13;
+  float *part = ws;
   a.part = part;
   const dim3 grid((unsigned)(nranges * a.kgroups), (unsigned)(a.jt_total / jt));
   if (tiles == 1) hipLaunchKernelGGL((wgrad_kernel<4, 1, 16>), grid, dim3(64), 0, s, a);

@@ -441,6 +441,8 @@ class SO3part : public cnine::BatchedTensor<std::complex<TYPE>>, public GpartBas
     gelib_check(gelib_hip_part_gather(&R, &X, gmap.device_handle(), d + 1, gmap.inverted ? 1 : 0, 1, gelib_stream()));
   }
   void add_gather_back(const SO3part &r, const cnine::GatherMapB &gmap, const int d = 0) const {
+    gmap.device_handle();  // made on the caller's map, so the reversed copy below shares it instead of uploading,
+                           // using and freeing a device copy of its own on every call
     add_gather(r, gmap.inv(), d);
   }
 

@@ -8,9 +8,12 @@
  * reference hands to its launchers (cuda/GPUtensor.hpp:31-38), with strides counted in complex
  * elements and stride 0 meaning "broadcast along this dimension" (core/Gpart.hpp:168-185).
  *
- * Every call is asynchronous on the HIP stream passed in (NULL = the default stream), allocates
- * nothing per call (the coefficient bank and the per-type triple tables are cached on first use),
- * and returns 0 or one of the gelib_hip_status codes without printing or throwing.
+ * Every call is asynchronous on the HIP stream passed in (NULL = the default stream) and returns 0 or
+ * one of the gelib_hip_status codes without printing or throwing.  Device memory: the first call for a
+ * new coefficient table or a new SO3vec type signature on a device computes its tables and uploads them
+ * (one allocation and one synchronous copy, kept for the life of the process); gelib_hip_gather_map_create
+ * allocates the map it returns; gelib_hip_malloc allocates what it is asked for.  No other call allocates,
+ * frees or synchronises: the channel-mixing entry points take their workspace from the caller.
  */
 #ifndef GELIB_HIP_H
 #define GELIB_HIP_H
@@ -39,13 +42,14 @@ enum gelib_hip_status {
   GELIB_HIP_ERR_DEVICE = 8,        /* a pointer is not device memory of the current GPU                              */
   GELIB_HIP_ERR_PARTS = 9,         /* too many parts, a repeated l, or l above the supported maximum                 */
   GELIB_HIP_ERR_RUNTIME = 10,      /* a HIP call failed; see gelib_hip_last_runtime_error()                          */
-  GELIB_HIP_ERR_BROADCAST_DEST = 11, /* overwrite requested into a destination that is broadcast (stride 0)          */
-  GELIB_HIP_ERR_ARG = 12           /* negative offset or other malformed argument                                    */
+  GELIB_HIP_ERR_BROADCAST_DEST = 11, /* the destination has a dimension of extent > 1 with stride 0 (an expanded view) */
+  GELIB_HIP_ERR_ARG = 12,          /* negative offset, negative stride or other malformed argument                   */
+  GELIB_HIP_ERR_WORKSPACE = 13     /* workspace missing, not 16-byte aligned or smaller than the size query says     */
 };
 
 #define GELIB_HIP_MAX_L 32          /* largest l of an operand part                     */
-#define GELIB_HIP_MAX_PARTS 16      /* parts per operand SO3vec                         */
-#define GELIB_HIP_MAX_OUT_PARTS 40  /* parts of the product / gradient SO3vec           */
+#define GELIB_HIP_MAX_PARTS 33      /* parts per operand SO3vec: every l from 0 to GELIB_HIP_MAX_L   */
+#define GELIB_HIP_MAX_OUT_PARTS 65  /* parts of the product / gradient SO3vec: l up to 2 GELIB_HIP_MAX_L */
 
 /* Message for a status code (static storage). */
 const char *gelib_hip_strerror(int status);
@@ -139,15 +143,24 @@ int gelib_hip_so3part_spharm(const gelib_part_desc *r, const float *x, const int
  * SO3linear (python/src/gelib/SO3vec.py:174-177, python/src/gelib/SO3weights.py:75-85).  adjoint != 0: w is
  * (n_out, n_in) and V = w^H: the gradient of that matmul with respect to the part (torch's autograd forms it in the
  * reference).  Row strides in complex elements.  n_in must be even and the rows of x 16-byte aligned (else
- * GELIB_HIP_ERR_ARG).  The re-packed matrix is kept in a buffer per (device, stream) that grows on demand. */
+ * GELIB_HIP_ERR_ARG).  workspace: device memory of at least gelib_hip_part_mix_workspace_bytes(0, rows, n_in, n_out)
+ * bytes, 16-byte aligned, that receives the matrix re-packed for the matrix cores; the kernels of the call read it, so
+ * it must stay untouched until they have run on `stream` (a buffer from a stream-ordered allocator does).  The library
+ * allocates nothing for this call (GELIB_HIP_ERR_WORKSPACE if the buffer is missing or too small). */
 int gelib_hip_part_mix_channels(void *r, const void *x, const void *w, int64_t rows, int n_in, int n_out,
-                                int64_t r_row_stride, int64_t x_row_stride, int adjoint, void *stream);
+                                int64_t r_row_stride, int64_t x_row_stride, int adjoint, void *workspace,
+                                uint64_t workspace_bytes, void *stream);
 /* wg[c, o] = sum over the rows of conj(x[row, c]) g[row, o], overwriting the row-major (n_in, n_out) matrix wg: the
  * gradient of the same matmul with respect to W (torch's autograd forms it in the reference).  Same conditions on
  * n_in and x.  The rows are summed in ranges whose partial sums are added in a fixed order: the result does not depend
- * on timing.  The partial sums live in the same per-(device, stream) buffer. */
+ * on timing.  workspace: at least gelib_hip_part_mix_workspace_bytes(1, rows, n_in, n_out) bytes for those partial sums,
+ * same rules as above. */
 int gelib_hip_part_mix_channels_wgrad(void *wg, const void *x, const void *g, int64_t rows, int n_in, int n_out,
-                                      int64_t x_row_stride, int64_t g_row_stride, void *stream);
+                                      int64_t x_row_stride, int64_t g_row_stride, void *workspace,
+                                      uint64_t workspace_bytes, void *stream);
+/* Bytes of workspace the two calls above need: kind 0 for gelib_hip_part_mix_channels (either value of adjoint; n_in and
+ * n_out as passed to that call), kind 1 for gelib_hip_part_mix_channels_wgrad.  0 for empty shapes or an unknown kind. */
+uint64_t gelib_hip_part_mix_workspace_bytes(int kind, int64_t rows, int n_in, int n_out);
 
 /* ---- gather: sums of slices along the batch or a grid dimension ---------------------------------------------------------
  * A gather map is a list of (source, target) pairs with 0 <= source < n_in, 0 <= target < n_out (the arguments of
@@ -185,7 +198,8 @@ int gelib_hip_synchronize(void);
 /*
  * Tuning / introspection (no counterpart in the reference).
  * gelib_hip_set_option("force_generic", 1) routes every call through the shape-agnostic kernels;
- * "check_pointers" (default 1) switches the device-pointer validation of every call off or on.
+ * "check_pointers" (default 1) switches the device-pointer validation of every call off or on (an allocation
+ * that has passed once is remembered, so repeated calls on the same buffers make no driver calls for it).
  * Tuning knobs of the fast families (0 restores the built-in choice unless noted): "unrolled_fwd" / "unrolled_bwd" /
  * "staged_fwd" / "staged_bwd" / "diag6" / "onepair" (1/0: use the family), "fwd_block_bytes", "fwd_lds_bytes", "fwd_tile",
  * "fwd_cell_tile" (cells per tile of the unrolled forward launch, 0 = one tile),

@@ -127,3 +127,47 @@ def test_host_pointer_is_refused_not_launched():
 def test_unknown_option():
     assert cabi.lib().gelib_hip_set_option(b"no_such_option", 1) != 0
     cabi.set_option("force_generic", 0)
+
+
+def test_destination_that_repeats_memory_and_negative_strides():
+    """An expanded view as destination (extent > 1, stride 0) and negative strides are refused before any pointer is
+    looked at, whatever the "check_pointers" option says."""
+    cabi.set_option("check_pointers", 0)
+    try:
+        x, y = fake(2, 3, 4), fake(2, 3, 4)
+        r = fake(2, 3, 16)
+        r.strides[0] = 0                                   # the two cells of the product share their memory
+        assert call("gelib_hip_so3part_cg_fwd", r, x, y) == 11
+        xg, g = fake(2, 3, 4), fake(2, 3, 16)
+        xg.strides[4] = 0                                  # all channels of the gradient in one place
+        assert call("gelib_hip_so3part_cg_back0", xg, g, y) == 11
+        yg = fake(2, 3, 4)
+        yg.strides[3] = 0
+        assert call("gelib_hip_so3part_cg_back1", yg, g, x) == 11
+        neg = fake(2, 3, 4)
+        neg.strides[3] = -4
+        assert call("gelib_hip_so3part_cg_fwd", fake(2, 3, 16), neg, y) == 12
+        L = cabi.lib()
+        A = cabi.PartDesc * 1
+        rr = A(fake(2, 3, 16))
+        rr[0].strides[0] = 0
+        assert L.gelib_hip_so3vec_cg_fwd(1, rr, 1, A(x), 1, A(y), 1, None) == 11
+        gg = A(fake(2, 3, 16))
+        bad = A(fake(2, 3, 4))
+        bad[0].strides[0] = 0
+        assert L.gelib_hip_so3vec_cg_bwd(bad, None, 1, gg, 1, A(x), 1, A(y), 1, None) == 11
+    finally:
+        cabi.set_option("check_pointers", 1)
+
+
+def test_part_count_limits():
+    """An SO3vec may hold every l from 0 to 32 (33 parts), its product every l up to 64 (65 parts); one more is status 9."""
+    L = cabi.lib()
+    xs = (cabi.PartDesc * 34)(*[fake(1, 2 * min(l, 32) + 1, 1) for l in range(34)])   # the last l is a repeat
+    y = (cabi.PartDesc * 1)(fake(1, 1, 1))
+    r = (cabi.PartDesc * 1)(fake(1, 1, 1))
+    assert L.gelib_hip_so3vec_cg_fwd(1, r, 34, xs, 1, y, 1, None) == 9
+    # 33 distinct parts pass the part-count check and are stopped later, by the missing channels of r
+    assert L.gelib_hip_so3vec_cg_fwd(1, (cabi.PartDesc * 1)(fake(1, 1, 0, ptr=None)), 33, xs, 1, y, 1, None) in (0, 5)
+    assert L.gelib_hip_part_mix_workspace_bytes(0, 10, 32, 16) >= 16 * 32 * 16
+    assert L.gelib_hip_part_mix_workspace_bytes(2, 10, 32, 16) == 0

@@ -170,7 +170,9 @@ def test_mix_channels_row_strides(cabi):
     w = rand((n_in, n_out), 12)
     x, r = xw[:, 8:8 + n_in], rw[:, 4:4 + n_out]
     L = cabi.lib()
-    cabi.check(L.gelib_hip_part_mix_channels(r.data_ptr(), x.data_ptr(), w.data_ptr(), rows, n_in, n_out, 24, 64, 0, None))
+    ws, nbytes = cabi.mix_workspace(0, rows, n_in, n_out, "cuda")
+    cabi.check(L.gelib_hip_part_mix_channels(r.data_ptr(), x.data_ptr(), w.data_ptr(), rows, n_in, n_out, 24, 64, 0,
+                                             ws.data_ptr(), nbytes, None))
     want = U.host(x.contiguous()).astype(np.complex128) @ U.host(w).astype(np.complex128)
     tol = 1e-6 + 4 * np.finfo(np.float32).eps * (np.abs(U.host(x.contiguous())).astype(np.float64) @ np.abs(U.host(w)).astype(np.float64))
     assert (np.abs(U.host(r.contiguous()) - want) <= tol).all()
@@ -179,6 +181,35 @@ def test_mix_channels_row_strides(cabi):
     assert float(rw[:, keep.cuda()].abs().max()) == 0.0      # nothing outside the block was written
     g = rand((rows, n_out), 13)
     wg = torch.empty(n_in, n_out, dtype=torch.complex64, device="cuda")
-    cabi.check(L.gelib_hip_part_mix_channels_wgrad(wg.data_ptr(), x.data_ptr(), g.data_ptr(), rows, n_in, n_out, 64, n_out, None))
+    ws1, nbytes1 = cabi.mix_workspace(1, rows, n_in, n_out, "cuda")
+    cabi.check(L.gelib_hip_part_mix_channels_wgrad(wg.data_ptr(), x.data_ptr(), g.data_ptr(), rows, n_in, n_out, 64, n_out,
+                                                   ws1.data_ptr(), nbytes1, None))
     hx, hg = U.host(x.contiguous()).astype(np.complex128), U.host(g).astype(np.complex128)
     assert (np.abs(U.host(wg) - hx.conj().T @ hg) <= 1e-6 + 4 * np.finfo(np.float32).eps * (np.abs(hx).T @ np.abs(hg))).all()
+
+
+def test_mix_channels_workspace_is_the_callers(cabi):
+    """The library allocates nothing for these calls: without a workspace, or with one that is too small or misaligned,
+    they return status 13 and launch nothing."""
+    rows, n_in, n_out = 64, 32, 16
+    x, w = rand((rows, n_in), 21), rand((n_in, n_out), 22)
+    r = torch.full((rows, n_out), 5.0, dtype=torch.complex64, device="cuda")
+    L = cabi.lib()
+    need = int(L.gelib_hip_part_mix_workspace_bytes(0, rows, n_in, n_out))
+    assert need > 0 and int(L.gelib_hip_part_mix_workspace_bytes(1, rows, n_in, n_out)) > 0
+    assert int(L.gelib_hip_part_mix_workspace_bytes(0, 0, n_in, n_out)) == 0
+    ws = torch.empty(need + 16, dtype=torch.uint8, device="cuda")
+    call = lambda p, n: L.gelib_hip_part_mix_channels(r.data_ptr(), x.data_ptr(), w.data_ptr(), rows, n_in, n_out,
+                                                      n_out, n_in, 0, p, n, None)
+    assert call(None, 0) == 13
+    assert call(ws.data_ptr(), 16 * n_in * n_out - 16) == 13      # less than the packed matrix itself
+    assert call(ws.data_ptr() + 4, need) == 13
+    g = rand((rows, n_out), 23)
+    wg = torch.empty(n_in, n_out, dtype=torch.complex64, device="cuda")
+    assert L.gelib_hip_part_mix_channels_wgrad(wg.data_ptr(), x.data_ptr(), g.data_ptr(), rows, n_in, n_out, n_in, n_out,
+                                               None, 0, None) == 13
+    torch.cuda.synchronize()
+    assert float((r - 5.0).abs().max()) == 0.0
+    assert call(ws.data_ptr(), need) == 0
+    torch.cuda.synchronize()
+    assert float((r - 5.0).abs().max()) > 0.0

@@ -121,3 +121,13 @@ def test_channel_counts_that_are_not_powers_of_two(cabi, case, diag):
         assert run_vec(cabi, *case, diag, seed=500, force_generic=False) == (2, 2)
     finally:
         cabi.set_option("diag6", 1)
+
+
+@pytest.mark.parametrize("case", [
+    (3, {l: 1 for l in range(17)}, {0: 2}, -1),      # 17 operand parts: more than the fused kernels' part lists hold
+    (2, {32: 1}, {32: 1}, -1),                        # 65 product parts, l = 0..64
+])
+def test_more_parts_than_the_fused_kernels_take(cabi, case):
+    """The reference's loop over triples has no limit on the number of parts (core/Gvec.hpp:311-345); vectors beyond the
+    fused kernels' argument lists run one launch per triple on the shape-agnostic kernels."""
+    assert run_vec(cabi, *case, False, seed=800, force_generic=False) == (1, 1)

@@ -18,7 +18,8 @@ SYMBOLS = [
     "gelib_hip_so3vec_cg_fwd", "gelib_hip_so3vec_cg_bwd", "gelib_hip_so3vec_diagcg_fwd",
     "gelib_hip_so3vec_diagcg_bwd", "gelib_hip_so3part_spharm", "gelib_hip_gather_map_create",
     "gelib_hip_gather_map_destroy", "gelib_hip_part_gather", "gelib_hip_part_mix_channels",
-    "gelib_hip_part_mix_channels_wgrad", "gelib_hip_part_mix_workspace_bytes", "gelib_hip_set_option",
+    "gelib_hip_part_mix_channels_static", "gelib_hip_part_mix_channels_wgrad", "gelib_hip_part_mix_workspace_bytes",
+    "gelib_hip_set_option",
     "gelib_hip_last_path",
     "gelib_hip_malloc", "gelib_hip_free", "gelib_hip_memcpy", "gelib_hip_memset", "gelib_hip_synchronize",
 ]
@@ -77,6 +78,9 @@ def lib():
                                                         ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.c_int64,
                                                         ctypes.c_int64, ctypes.c_void_p, ctypes.c_uint64,
                                                         ctypes.c_void_p]
+        L.gelib_hip_part_mix_channels_static.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+                                                         ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.c_int64,
+                                                         ctypes.c_int64, ctypes.c_int, ctypes.c_void_p]
         L.gelib_hip_part_mix_workspace_bytes.restype = ctypes.c_uint64
         L.gelib_hip_part_mix_workspace_bytes.argtypes = [ctypes.c_int, ctypes.c_int64, ctypes.c_int, ctypes.c_int]
         L.gelib_hip_set_option.argtypes = [ctypes.c_char_p, ctypes.c_int]

@@ -553,6 +553,9 @@ const char *gelib_hip_strerror(int status) {
     case GELIB_HIP_ERR_BROADCAST_DEST: return "the destination repeats memory (a dimension of extent > 1 with stride 0)";
     case GELIB_HIP_ERR_ARG: return "malformed argument";
     case GELIB_HIP_ERR_WORKSPACE: return "workspace missing, not 16-byte aligned or too small";
+    case GELIB_HIP_ERR_TOO_LARGE:
+      return "the packed matrix of n_in x n_out channels exceeds the 8 MiB array of the entry point that allocates "
+             "nothing; use gelib_hip_part_mix_channels with a workspace";
   }
   return "unknown status";
 }
@@ -752,12 +755,12 @@ int gelib_hip_part_gather(const gelib_part_desc *r, const gelib_part_desc *x, co
 }
 
 // ---- channel mixing (the linear layer that consumes a product) ------------------------------------------------------
-int gelib_hip_part_mix_channels(void *r, const void *x, const void *w, int64_t rows, int n_in, int n_out,
-                                int64_t r_row_stride, int64_t x_row_stride, int adjoint, void *workspace,
-                                uint64_t workspace_bytes, void *stream) {
-  t_last_path = kPathNone;
+namespace {
+// argument checks shared by the two forms of the product; 0 = go on, -1 = nothing to do, else a status
+int mix_check(void *r, const void *x, const void *w, int64_t rows, int n_in, int n_out, int64_t r_row_stride,
+              int64_t x_row_stride, int adjoint) {
   if (rows < 0 || n_in < 0 || n_out < 0 || r_row_stride < n_out || x_row_stride < n_in) return GELIB_HIP_ERR_ARG;
-  if (rows == 0 || n_out == 0) return GELIB_HIP_OK;
+  if (rows == 0 || n_out == 0) return -1;
   if (!r || (n_in > 0 && (!x || !w))) return GELIB_HIP_ERR_NULL;
   if (n_in == 0 || (n_in & 1) || (x_row_stride & 1) || ((uintptr_t)x & 15) || rows > (1LL << 38))
     return GELIB_HIP_ERR_ARG;
@@ -769,11 +772,32 @@ int gelib_hip_part_mix_channels(void *r, const void *x, const void *w, int64_t r
   if ((rc = check_range(r, rd, rst, 2 * sizeof(float))) || (rc = check_range(x, xd, xst, 2 * sizeof(float))) ||
       (rc = check_range(w, wd, wst, 2 * sizeof(float))))
     return rc;
+  return GELIB_HIP_OK;
+}
+}  // namespace
+
+int gelib_hip_part_mix_channels(void *r, const void *x, const void *w, int64_t rows, int n_in, int n_out,
+                                int64_t r_row_stride, int64_t x_row_stride, int adjoint, void *workspace,
+                                uint64_t workspace_bytes, void *stream) {
+  t_last_path = kPathNone;
+  int rc = mix_check(r, x, w, rows, n_in, n_out, r_row_stride, x_row_stride, adjoint);
+  if (rc) return rc < 0 ? GELIB_HIP_OK : rc;
   const int64_t sd[5] = {(int64_t)workspace_bytes, 1, 1, 1, 1}, sst[5] = {1, 0, 0, 0, 0};
   if (workspace && workspace_bytes && (rc = check_range(workspace, sd, sst, 1))) return rc;
   t_last_path = kPathGeneric;
   rc = launch_mix((float2 *)r, (const float2 *)x, (const float2 *)w, rows, n_in, n_out, x_row_stride, r_row_stride,
                   adjoint != 0, (float *)workspace, (size_t)workspace_bytes, (hipStream_t)stream);
+  return rc == 11 ? GELIB_HIP_ERR_ARG : rc;
+}
+
+int gelib_hip_part_mix_channels_static(void *r, const void *x, const void *w, int64_t rows, int n_in, int n_out,
+                                       int64_t r_row_stride, int64_t x_row_stride, int adjoint, void *stream) {
+  t_last_path = kPathNone;
+  int rc = mix_check(r, x, w, rows, n_in, n_out, r_row_stride, x_row_stride, adjoint);
+  if (rc) return rc < 0 ? GELIB_HIP_OK : rc;
+  t_last_path = kPathGeneric;
+  rc = launch_mix_static((float2 *)r, (const float2 *)x, (const float2 *)w, rows, n_in, n_out, x_row_stride,
+                         r_row_stride, adjoint != 0, (hipStream_t)stream);
   return rc == 11 ? GELIB_HIP_ERR_ARG : rc;
 }
 

@@ -66,6 +66,11 @@ int launch_gather(float2 *r, const float2 *x, const long long rs[5], const long 
 size_t mix_workspace_bytes(int n_in, int n_out);
 int launch_mix(float2 *r, const float2 *x, const float2 *w, long long rows, int n_in, int n_out, long long xs,
                long long rs, bool adjoint, float *ws, size_t ws_bytes, hipStream_t s);
+// the same with the packed matrix in an array of the library's own device image (no workspace, nothing allocated);
+// 14 when n_in and n_out need more than mix_static_scratch_bytes()
+size_t mix_static_scratch_bytes();
+int launch_mix_static(float2 *r, const float2 *x, const float2 *w, long long rows, int n_in, int n_out, long long xs,
+                      long long rs, bool adjoint, hipStream_t s);
 // wg (n_in, n_out) = sum over the rows of conj(x[row, :])^T g[row, :]; the workspace holds the partial sums
 size_t mix_wgrad_workspace_bytes(long long rows, int n_in, int n_out);
 int launch_mix_wgrad(float2 *wg, const float2 *x, const float2 *g, long long rows, int n_in, int n_out, long long xs,

@@ -24,6 +24,7 @@
 // every row) at a time: lane (i, h) reads the 16 floats of its row that start at 16 h.
 #include <algorithm>
 #include <map>
+#include <mutex>
 #include <string>
 
 #include "cg_common.h"
@@ -491,6 +492,46 @@ int launch_mix(float2 *r, const float2 *x, const float2 *w, long long rows, int 
     launch<1, 4, true>(a, s);
   }
   return hipGetLastError() == hipSuccess ? 0 : 10;
+}
+
+// ---- the same product for callers that cannot allocate -------------------------------------------------------------
+// Code under graph capture, tight serving loops and harnesses that forbid hipMalloc have no workspace to pass.  For them
+// the packed matrix goes into an array that is part of the library's device image: every GPU the library runs on holds
+// its own copy (kStaticScratchBytes, until the process ends) at its own address.  In host code the array's name is only a
+// stand-in for that address, so it is never passed to a kernel or a copy: the address is asked for once per device with
+// hipGetSymbolAddress, with that device current, and from then on only that pointer is used.  Every call on a GPU
+// shares that GPU's array: calls that overlap on one GPU (two streams, two host threads) race on it.  Nothing in it has
+// to start at zero, since the pack kernel writes every float of the region a call reads, padding included.
+constexpr size_t kStaticScratchBytes = (size_t)8 << 20;   // 16 B per pair of channels: n_in * n_out up to 524288
+static __device__ __align__(256) float scratch[kStaticScratchBytes / sizeof(float)];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+float *g_scratch_ptr[kMaxDevices] = {};
+}  // namespace
+
+size_t mix_static_scratch_bytes() { return kStaticScratchBytes; }
+
+// 0, 10, 11 as launch_mix; 14 when the packed matrix does not fit the array
+int launch_mix_static(float2 *r, const float2 *x, const float2 *w, long long rows, int n_in, int n_out, long long xs,
+                      long long rs, bool adjoint, hipStream_t s) {
+  if (rows == 0 || n_out == 0) return 0;
+  if (mix_workspace_bytes(n_in, n_out) > kStaticScratchBytes) return 14;
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 10;
+  float *ptr;
+  {
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+      float *p = nullptr;
+      const hipError_t e = hipGetSymbolAddress((void **)&p, HIP_SYMBOL(scratch));   // this device's copy
+      if (e != hipSuccess || !p) return record_hip_error(e, "hipGetSymbolAddress(scratch)");
+      g_scratch_ptr[dev] = p;
+    }
+    ptr = g_scratch_ptr[dev];
+  }
+  return launch_mix(r, x, w, rows, n_in, n_out, xs, rs, adjoint, ptr, kStaticScratchBytes, s);
 }
 
 // ---- gradient with respect to the matrix:  wg[c, o] = sum_rows conj(x[row, c]) g[row, o] ----------------------------------

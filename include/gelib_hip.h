@@ -44,7 +44,8 @@ enum gelib_hip_status {
   GELIB_HIP_ERR_RUNTIME = 10,      /* a HIP call failed; see gelib_hip_last_runtime_error()                          */
   GELIB_HIP_ERR_BROADCAST_DEST = 11, /* the destination has a dimension of extent > 1 with stride 0 (an expanded view) */
   GELIB_HIP_ERR_ARG = 12,          /* negative offset, negative stride or other malformed argument                   */
-  GELIB_HIP_ERR_WORKSPACE = 13     /* workspace missing, not 16-byte aligned or smaller than the size query says     */
+  GELIB_HIP_ERR_WORKSPACE = 13,    /* workspace missing, not 16-byte aligned or smaller than the size query says     */
+  GELIB_HIP_ERR_TOO_LARGE = 14     /* sizes beyond the stated maximum of gelib_hip_part_mix_channels_static          */
 };
 
 #define GELIB_HIP_MAX_L 32          /* largest l of an operand part                     */
@@ -150,6 +151,17 @@ int gelib_hip_so3part_spharm(const gelib_part_desc *r, const float *x, const int
 int gelib_hip_part_mix_channels(void *r, const void *x, const void *w, int64_t rows, int n_in, int n_out,
                                 int64_t r_row_stride, int64_t x_row_stride, int adjoint, void *workspace,
                                 uint64_t workspace_bytes, void *stream);
+/* gelib_hip_part_mix_channels for callers that cannot allocate device memory and so have no workspace to pass: code
+ * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the
+ * reference.  Same arguments, same kernels, same results bit for bit; the re-packed matrix goes into an 8 MiB array that
+ * is part of the library's device image (each GPU the library runs on holds its own copy until the process ends), so the
+ * call allocates nothing -- neither directly nor through any library routine.  Limit: the packed matrix must fit, i.e.
+ * gelib_hip_part_mix_workspace_bytes(0, rows, n_in, n_out) <= 8 MiB (16 bytes per pair of channels: n_in * n_out up to
+ * 524288 when both are multiples of 16), else GELIB_HIP_ERR_TOO_LARGE.  All calls on one GPU share that GPU's array:
+ * calls that may overlap there (two streams, two host threads) race on it and must be ordered by the caller.  The
+ * first call on a device asks the runtime for the array's address on that device (no allocation). */
+int gelib_hip_part_mix_channels_static(void *r, const void *x, const void *w, int64_t rows, int n_in, int n_out,
+                                       int64_t r_row_stride, int64_t x_row_stride, int adjoint, void *stream);
 /* wg[c, o] = sum over the rows of conj(x[row, c]) g[row, o], overwriting the row-major (n_in, n_out) matrix wg: the
  * gradient of the same matmul with respect to W (torch's autograd forms it in the reference).  Same conditions on
  * n_in and x.  The rows are summed in ranges whose partial sums are added in a fixed order: the result does not depend

@@ -434,6 +434,12 @@ int bwd_dispatch(const VecPlan &plan, const std::vector<View> &G, const std::vec
         return GELIB_HIP_OK;
       }
     }
+    rc = onepair_mfma_vec_bwd(plan, gd, xd, yd, xgd, ygd, accumulate != 0, s, &used);
+    if (rc) return rc;
+    if (used) {
+      t_last_path = kPathOnePair;
+      return GELIB_HIP_OK;
+    }
     rc = onepair_vec_bwd(plan, gd, xd, yd, xgd, ygd, accumulate != 0, s, &used);
     if (rc) return rc;
     if (used) {
@@ -873,6 +879,7 @@ int gelib_hip_set_option(const char *name, int value) {
   }
   if (!std::strncmp(name, "staged_", 7)) return staged_set_option(name, value);
   if (!std::strncmp(name, "diag6", 5)) return diag6_set_option(name, value);
+  if (!std::strcmp(name, "onepair_mfma")) return onepair_mfma_set_option(name, value);
   if (!std::strncmp(name, "onepair", 7)) return onepair_set_option(name, value);
   if (!std::strncmp(name, "mix_", 4)) return mix_set_option(name, value);
   return unrolled_set_option(name, value);

@@ -1,0 +1,380 @@
+// Backward pass of a product of ONE x part with ONE y part of large l, 8 x 8 channels, on the matrix cores: both
+// gradients from one pass over g (the l1 = l2 = 10, all 21 l case; any l1 <= 15, l2 <= 15, at most 22 values of l).
+//
+// For one row number m = m1 + m2 the contraction over l,
+//     Q[m1, chan] = sum_l C_l[m1, m - m1] g_l[m, chan],
+// is a real (m1 x l) matrix times the (l x 128) block of the floats of the rows g_l[m] -- GEMM-shaped, with up to 21 x 21
+// coefficients per m.  v_mfma_f32_32x32x2_f32 computes D (32 x 32) += A (32 x 2) B (2 x 32): here the rows of D are the
+// floats of the 64 channels (four tiles of 32), its columns are m1, a step of the reduction is two values of l.
+//   A: lane (i, h) = (lane % 32, lane / 32) loads 16 bytes of row g_{l(h)}[m], floats 4 i .. 4 i + 3, one for each of the
+//      four tiles: a wave's load instruction fetches the two rows of a step, 512 contiguous bytes each;
+//   B: lane (i, h) supplies C_{l(h)}[m1 = i - l1, m - m1], from a table laid out in lane order (one float per lane, step
+//      and m), zero where the pair (m1, m2) or the value of l does not exist;
+//   D: lane (i, h) ends up with Q[m1 = i - l1] of the 32 channels (a, j) with a = 2 b + h, b = 0..3, j = 0..7, real and
+//      imaginary part: register v of tile e is float 4 (8 (v / 4) + 4 h + v % 4) + e of the row.
+// So after the matrix instructions of one m a lane owns ONE m1 and with it one m2 = m - m1:
+//   x-gradient  ax[m1, a] += sum_j Q[a, j] conj(y[m2, j]): the lane's m1 never changes, the sums are eight registers;
+//   y-gradient  the lane's partial sum for ay[m2, j] (over its four a) belongs to a row m2 that moves on by one lane when
+//               m goes up by one.  The eight partial sums travel with it: after every m they are shifted one lane up
+//               (wave_shr), zeros enter at m1 = -l1, and the row that has left m1 = l1 is complete and is parked in LDS.
+// No atomics, a fixed order of additions.  The vector unit does 256 multiply-adds per m and lane (both gradients),
+// the matrix cores the 2 x (21 - |m|)^2 x 128 of the contraction; the operands of the next eight steps are always in
+// flight, across the boundaries between the m.
+#include <cstring>
+#include <map>
+#include <mutex>
+#include <vector>
+
+#include "cg_staged.h"
+#include "cg_unrolled_dev.h"
+
+namespace gelib_hip {
+
+namespace {
+
+constexpr int kNLm = 22;   // most values of l of the pair
+constexpr int kMaxLm = 15; // largest l1, l2: 2 l + 1 <= 31 columns, one spare for the row that leaves
+
+struct OnePairMfmaArgs {
+  FastPart x, y, xg, yg;
+  FastPart g[kNLm];   // by dl = l - lmin; ptr == nullptr: no such triple
+  int offs[kNLm];     // first channel of the triple's block in its part
+  const float *coef;  // device: 64 floats (lane order) per (m, step)
+  int nsteps;         // steps of all m, rounded up to a multiple of the kernel's queue length (idle steps at the end)
+  long long ncells;
+  int l1, l2, lmin, lt, nl;
+  int offs_add, accumulate;
+};
+
+typedef float f16v __attribute__((ext_vector_type(16)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef const __attribute__((address_space(1))) v4f *GlobalIn4;
+typedef const __attribute__((address_space(1))) float *GlobalIn1;
+typedef const __attribute__((address_space(4))) int *IntPtr;
+
+__device__ __forceinline__ float wave_shr1(float v) {  // lane k receives lane k - 1, lane 0 receives 0
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x138, 0xf, 0xf, true));
+}
+
+constexpr int kQueue = 6;  // steps whose operands are in flight or waiting in registers
+
+__global__ void __launch_bounds__(64) onepair_mfma_bwd_kernel(const OnePairMfmaArgs a) {
+  __shared__ unsigned long long gbase[kNLm + 1];  // address of row 0 of the cell's block in part dl; slot nl: a harmless row
+  __shared__ unsigned growb[kNLm + 1];            // distance between rows in bytes
+  __shared__ float2 ys[(2 * kMaxLm + 1) * 8];
+  __shared__ float2 accy[2][(2 * kMaxLm + 1) * 8];
+  const int lane = threadIdx.x, i = lane & 31, h = lane >> 5;
+  const int l1 = a.l1, l2 = a.l2, lmin = a.lmin, lt = a.lt, nl = a.nl;
+  const long long cell = blockIdx.x;
+  const int r1 = 2 * l1 + 1, r2 = 2 * l2 + 1;
+
+  static_for<kNLm>([&](auto dc) __attribute__((always_inline)) {
+    constexpr int dl = decltype(dc)::value;
+    if (lane == 0 && dl < nl) {
+      const FastPart P = a.g[dl];
+      const bool there = P.ptr != nullptr;
+      // a triple that is not there reads the coefficient table (finite numbers) and meets coefficients that are zero
+      gbase[dl] = there ? (unsigned long long)(P.ptr + cell * P.sb + (a.offs[dl] + a.offs_add)) : (unsigned long long)a.coef;
+      growb[dl] = there ? (unsigned)P.sm * 8u : 0u;
+    }
+  });
+  if (lane == 0) {
+    gbase[nl] = (unsigned long long)a.coef;
+    growb[nl] = 0u;
+  }
+  for (int e = lane; e < r2 * 8; e += 64) {
+    ys[e] = a.y.ptr[cell * a.y.sb + (long long)(e >> 3) * a.y.sm + (e & 7)];
+    accy[0][e] = make_float2(0.f, 0.f);
+    accy[1][e] = make_float2(0.f, 0.f);
+  }
+  // the lane's row of x: m1 = i - l1, channels 2 b + h; a lane beyond the rows holds zeros (so do its coefficients)
+  float2 xv[4];
+#pragma unroll
+  for (int b = 0; b < 4; b++)
+    xv[b] = i < r1 ? a.x.ptr[cell * a.x.sb + (long long)i * a.x.sm + (2 * b + h)] : make_float2(0.f, 0.f);
+  __syncthreads();
+
+  // The steps of all m form one sequence (two values of l per step, m ascending), padded with idle steps to a multiple
+  // of kQueue.  The operands of the next kQueue steps are always on their way: a step's registers are refilled for the
+  // step kQueue further on as soon as its matrix instructions are issued.  No load sits behind a branch.
+  const int nsteps = a.nsteps;
+  // where a step stands: its m, the first of its two dl, and how many steps of this m are left (itself included);
+  // scalar arithmetic only.  Beyond the last m the cursor idles on the harmless row.
+  struct Cursor {
+    int m, dlb, left;
+  };
+  auto start_m = [&](Cursor &c, int m) __attribute__((always_inline)) {
+    const int mabs = m < 0 ? -m : m;
+    const int dl0 = (mabs > lmin ? mabs : lmin) - lmin;  // the first l with a row m
+    c.m = m;
+    c.dlb = dl0;
+    c.left = (nl - dl0 + 1) >> 1;
+  };
+  auto next_step = [&](Cursor &c) __attribute__((always_inline)) {
+    if (--c.left > 0) {
+      c.dlb += 2;
+    } else if (c.m < lt) {
+      start_m(c, c.m + 1);
+    } else {
+      c.dlb = nl;
+      c.left = 1 << 30;
+    }
+  };
+  v4f G[kQueue];
+  float C[kQueue];
+  long long coef_at = lane;  // the lane's coefficient of the step that is fetched next
+  auto fetch = [&](const Cursor &c, v4f &g, float &cf) __attribute__((always_inline)) {
+    int dl = c.dlb + h;
+    dl = dl < nl ? dl : nl;
+    const unsigned long long base = gbase[dl];
+    const unsigned rowb = growb[dl];
+    const unsigned long long addr = base + (unsigned long long)((unsigned)(c.m + lmin + dl) * rowb) + (unsigned)i * 16u;
+    g = *(GlobalIn4)addr;
+    cf = *((GlobalIn1)a.coef + coef_at);   // the table ends with a queue's worth of idle steps
+    coef_at += 64;
+  };
+
+  float2 ax[4], S[8];
+#pragma unroll
+  for (int b = 0; b < 4; b++) ax[b] = make_float2(0.f, 0.f);
+#pragma unroll
+  for (int j = 0; j < 8; j++) S[j] = make_float2(0.f, 0.f);
+  f16v D[4];
+#pragma unroll
+  for (int e = 0; e < 4; e++)
+#pragma unroll
+    for (int v = 0; v < 16; v++) D[e][v] = 0.f;
+
+  // the sums of one m are in D: both gradients, then every row of the y-gradient moves one lane up
+  auto finish_m = [&](int m) __attribute__((always_inline)) {
+    // the lane's m2 = m - m1; outside [-l2, l2] (or m1 beyond l1) every coefficient was zero and so is Q
+    int m2 = m - (i - l1);
+    m2 = m2 < -l2 ? -l2 : (m2 > l2 ? l2 : m2);
+    const float4 *yrow = reinterpret_cast<const float4 *>(ys + (m2 + l2) * 8);
+    float2 yv[8];
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+      const float4 t = yrow[q];
+      yv[2 * q] = make_float2(t.x, t.y);
+      yv[2 * q + 1] = make_float2(t.z, t.w);
+    }
+#pragma unroll
+    for (int b = 0; b < 4; b++)
+#pragma unroll
+      for (int vv = 0; vv < 4; vv++)
+#pragma unroll
+        for (int e2 = 0; e2 < 2; e2++) {
+          const float qr = D[2 * e2][4 * b + vv], qi = D[2 * e2 + 1][4 * b + vv];
+          const int j = 2 * vv + e2;
+          ax[b].x = fmaf(qr, yv[j].x, ax[b].x);
+          ax[b].x = fmaf(qi, yv[j].y, ax[b].x);
+          ax[b].y = fmaf(qi, yv[j].x, ax[b].y);
+          ax[b].y = fmaf(-qr, yv[j].y, ax[b].y);
+          S[j].x = fmaf(qr, xv[b].x, S[j].x);
+          S[j].x = fmaf(qi, xv[b].y, S[j].x);
+          S[j].y = fmaf(qi, xv[b].x, S[j].y);
+          S[j].y = fmaf(-qr, xv[b].y, S[j].y);
+        }
+#pragma unroll
+    for (int e = 0; e < 4; e++)
+#pragma unroll
+      for (int v = 0; v < 16; v++) D[e][v] = 0.f;
+    if (m < lt) {  // the row that leaves m1 = l1 is complete; after the last m the rows stay where they are
+#pragma unroll
+      for (int j = 0; j < 8; j++) {
+        S[j].x = wave_shr1(S[j].x);
+        S[j].y = wave_shr1(S[j].y);
+      }
+      const int mdone = m - l1;  // the row now in column r1
+      if (i == r1 && mdone >= -l2 && mdone <= l2) {
+        float4 *dst = reinterpret_cast<float4 *>(accy[h] + (mdone + l2) * 8);
+#pragma unroll
+        for (int q = 0; q < 4; q++) dst[q] = make_float4(S[2 * q].x, S[2 * q].y, S[2 * q + 1].x, S[2 * q + 1].y);
+      }
+      if (i == 0 || i >= r1) {  // zeros enter at m1 = -l1; nothing travels on beyond the last column
+#pragma unroll
+        for (int j = 0; j < 8; j++) S[j] = make_float2(0.f, 0.f);
+      }
+    }
+  };
+
+  // The fences keep the loads in the order of the steps, here as in the loop: the wait in front of a step's matrix
+  // instructions then counts the loads issued after its own instead of waiting for all.
+  Cursor cf, ck;
+  start_m(cf, -lt);
+  start_m(ck, -lt);
+  static_for<kQueue>([&](auto kc) __attribute__((always_inline)) {
+    fetch(cf, G[kc.value], C[kc.value]);
+    next_step(cf);
+    __builtin_amdgcn_sched_barrier(0);
+  });
+  for (int q0 = 0; q0 < nsteps; q0 += kQueue) {
+    static_for<kQueue>([&](auto kc) __attribute__((always_inline)) {
+      constexpr int k = decltype(kc)::value;
+      const v4f g = G[k];
+      const float c = C[k];
+      D[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(g.x, c, D[0], 0, 0, 0);
+      D[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(g.y, c, D[1], 0, 0, 0);
+      D[2] = __builtin_amdgcn_mfma_f32_32x32x2f32(g.z, c, D[2], 0, 0, 0);
+      D[3] = __builtin_amdgcn_mfma_f32_32x32x2f32(g.w, c, D[3], 0, 0, 0);
+      fetch(cf, G[k], C[k]);
+      next_step(cf);
+      __builtin_amdgcn_sched_barrier(0);
+      if (ck.left == 1) finish_m(ck.m);  // uniform; an idle step never ends an m
+      next_step(ck);
+    });
+  }
+  // the rows that are still on their way are complete as well: column i holds m2 = lt - (i - l1)
+  {
+    const int m2 = lt - (i - l1);
+    if (i < r1 && m2 >= -l2 && m2 <= l2) {
+      float4 *dst = reinterpret_cast<float4 *>(accy[h] + (m2 + l2) * 8);
+#pragma unroll
+      for (int q = 0; q < 4; q++) dst[q] = make_float4(S[2 * q].x, S[2 * q].y, S[2 * q + 1].x, S[2 * q + 1].y);
+    }
+  }
+  __syncthreads();
+
+  const bool accumulate = a.accumulate != 0;
+  if (i < r1) {
+#pragma unroll
+    for (int b = 0; b < 4; b++) {
+      float2 *p = a.xg.ptr + cell * a.xg.sb + (long long)i * a.xg.sm + (2 * b + h);
+      float2 o = ax[b];
+      if (accumulate) o.x += p->x, o.y += p->y;
+      *p = o;
+    }
+  }
+  for (int e = lane; e < r2 * 8; e += 64) {
+    float2 *p = a.yg.ptr + cell * a.yg.sb + (long long)(e >> 3) * a.yg.sm + (e & 7);
+    float2 o = make_float2(accy[0][e].x + accy[1][e].x, accy[0][e].y + accy[1][e].y);
+    if (accumulate) o.x += p->x, o.y += p->y;
+    *p = o;
+  }
+}
+
+// ---- host side ---------------------------------------------------------------------------------------------------
+
+struct Tables {
+  float *coef;
+  int nsteps;
+};
+std::mutex g_mutex;
+std::map<std::vector<int>, Tables> g_tables;  // (device, l1, l2, lmin, lt, nl, present...) -> device tables
+int g_enable = 1;
+
+int device_tables(int l1, int l2, int lmin, int lt, int nl, const std::vector<int> &present, Tables *out) {
+  int dev = 0;
+  GELIB_HIP_TRY(hipGetDevice(&dev));
+  std::vector<int> key = {dev, l1, l2, lmin, lt, nl};
+  key.insert(key.end(), present.begin(), present.end());
+  std::lock_guard<std::mutex> lock(g_mutex);
+  auto it = g_tables.find(key);
+  if (it == g_tables.end()) {
+    std::vector<std::vector<float>> C(nl);
+    for (int dl = 0; dl < nl; dl++)
+      if (present[dl]) {
+        C[dl].resize((size_t)(2 * l1 + 1) * (2 * l2 + 1));
+        cg_matrix_host(l1, l2, lmin + dl, C[dl].data());
+      }
+    std::vector<float> coef;
+    int step = 0;
+    for (int m = -lt; m <= lt; m++) {
+      const int dl0 = std::max(std::abs(m), lmin) - lmin;   // the first l with a row m
+      const int nks = (nl - dl0 + 1) / 2;
+      for (int ks = 0; ks < nks; ks++, step++) {
+        for (int lane = 0; lane < 64; lane++) {
+          const int col = lane & 31, h = lane >> 5;
+          const int dl = dl0 + 2 * ks + h, m1 = col - l1, m2 = m - m1;
+          float c = 0.f;
+          if (dl < nl && present[dl] && col <= 2 * l1 && m2 >= -l2 && m2 <= l2)
+            c = C[dl][(size_t)(m1 + l1) * (2 * l2 + 1) + (m2 + l2)];
+          coef.push_back(c);
+        }
+      }
+    }
+    while (step % kQueue != 0) {  // idle steps: the harmless row against coefficients that are zero
+      coef.insert(coef.end(), 64, 0.f);
+      step++;
+    }
+    coef.insert(coef.end(), (size_t)kQueue * 64, 0.f);  // the queue runs kQueue steps ahead, also at the end; the start
+                                                          // of the table doubles as the harmless row (512 bytes at least)
+    Tables t{nullptr, step};
+    GELIB_HIP_TRY(hipMalloc((void **)&t.coef, coef.size() * sizeof(float)));
+    GELIB_HIP_TRY(hipMemcpy(t.coef, coef.data(), coef.size() * sizeof(float), hipMemcpyHostToDevice));
+    it = g_tables.emplace(key, t).first;
+  }
+  *out = it->second;
+  return GELIB_HIP_OK;
+}
+
+}  // namespace
+
+// Both gradients of a non-Diag product of one x part with one y part, 8 x 8 channels, l1, l2 <= 15.  *used = 1 if
+// the launch was made; anything else is left to the other kernels.
+int onepair_mfma_vec_bwd(const VecPlan &plan, const std::vector<const gelib_part_desc *> &g,
+                         const std::vector<const gelib_part_desc *> &x, const std::vector<const gelib_part_desc *> &y,
+                         const std::vector<const gelib_part_desc *> &xg, const std::vector<const gelib_part_desc *> &yg,
+                         bool accumulate, hipStream_t s, int *used) {
+  *used = 0;
+  if (!g_enable || plan.diag || x.size() != 1 || y.size() != 1 || xg.size() != 1 || yg.size() != 1 || plan.triples.empty())
+    return GELIB_HIP_OK;
+  std::vector<FastPart> fx, fy, fg, fxg, fyg;
+  std::vector<std::pair<int, int>> lx, ly, lg;
+  if (!lists_to_fast(x, plan.E, false, &fx, &lx) || !lists_to_fast(y, plan.E, false, &fy, &ly) ||
+      !lists_to_fast(g, plan.E, false, &fg, &lg) || !lists_to_fast(xg, plan.E, true, &fxg, nullptr) ||
+      !lists_to_fast(yg, plan.E, true, &fyg, nullptr))
+    return GELIB_HIP_OK;
+  const int l1 = lx[0].first, l2 = ly[0].first, n1 = lx[0].second, n2 = ly[0].second;
+  if (n1 != 8 || n2 != 8 || l1 > kMaxLm || l2 > kMaxLm) return GELIB_HIP_OK;
+  const int lmin = std::abs(l1 - l2);
+  int lmax = -1;
+  for (auto &t : plan.triples) lmax = std::max(lmax, t.l);
+  const int nl = lmax - lmin + 1;
+  if (nl > kNLm || nl < 4) return GELIB_HIP_OK;  // a few values of l: the other kernels do as well
+  OnePairMfmaArgs a;
+  std::memset(&a, 0, sizeof(a));
+  a.x = fx[0];
+  a.y = fy[0];
+  a.xg = fxg[0];
+  a.yg = fyg[0];
+  std::vector<int> present(nl, 0);
+  for (auto &t : plan.triples) {
+    const int dl = t.l - lmin;
+    a.g[dl] = fg[t.ri];
+    a.offs[dl] = t.offs;
+    present[dl] = 1;
+    // the lane's 16 bytes of a row must be 16-byte aligned: block offset, row and cell strides even
+    if (((t.offs) & 1) || (fg[t.ri].sm & 1) || (fg[t.ri].sb & 1) || ((uintptr_t)fg[t.ri].ptr & 15)) return GELIB_HIP_OK;
+    if ((long long)fg[t.ri].sm * 8 * (2 * t.l + 1) >= (1LL << 32)) return GELIB_HIP_OK;  // row offsets are 32 bits
+  }
+  const long long ncells = plan.E[0] * plan.E[1] * plan.E[2];
+  if (ncells > 0x7fffffffLL) return GELIB_HIP_OK;
+  Tables t;
+  const int lt = std::min(l1 + l2, lmax);
+  int rc = device_tables(l1, l2, lmin, lt, nl, present, &t);
+  if (rc) return rc;
+  a.coef = t.coef;
+  a.nsteps = t.nsteps;
+  a.ncells = ncells;
+  a.l1 = l1;
+  a.l2 = l2;
+  a.lmin = lmin;
+  a.lt = lt;
+  a.nl = nl;
+  a.accumulate = accumulate ? 1 : 0;
+  hipLaunchKernelGGL(onepair_mfma_bwd_kernel, dim3((unsigned)ncells), dim3(64), 0, s, a);
+  GELIB_HIP_TRY(hipGetLastError());
+  *used = 1;
+  return GELIB_HIP_OK;
+}
+
+int onepair_mfma_set_option(const char *name, int value) {
+  if (!std::strcmp(name, "onepair_mfma")) {
+    g_enable = value;
+    return GELIB_HIP_OK;
+  }
+  return GELIB_HIP_ERR_ARG;
+}
+
+}  // namespace gelib_hip

@@ -140,10 +140,6 @@ __global__ void __launch_bounds__(64) onepair_mfma_bwd_kernel(const OnePairMfmaA
 #pragma unroll
   for (int j = 0; j < 8; j++) S[j] = make_float2(0.f, 0.f);
   f16v D[4];
-#pragma unroll
-  for (int e = 0; e < 4; e++)
-#pragma unroll
-    for (int v = 0; v < 16; v++) D[e][v] = 0.f;
 
   // the sums of one m are in D: both gradients, then every row of the y-gradient moves one lane up
   auto finish_m = [&](int m) __attribute__((always_inline)) {
@@ -175,10 +171,6 @@ __global__ void __launch_bounds__(64) onepair_mfma_bwd_kernel(const OnePairMfmaA
           S[j].y = fmaf(qi, xv[b].x, S[j].y);
           S[j].y = fmaf(-qr, xv[b].y, S[j].y);
         }
-#pragma unroll
-    for (int e = 0; e < 4; e++)
-#pragma unroll
-      for (int v = 0; v < 16; v++) D[e][v] = 0.f;
     if (m < lt) {  // the row that leaves m1 = l1 is complete; after the last m the rows stay where they are
 #pragma unroll
       for (int j = 0; j < 8; j++) {
@@ -208,15 +200,27 @@ __global__ void __launch_bounds__(64) onepair_mfma_bwd_kernel(const OnePairMfmaA
     next_step(cf);
     __builtin_amdgcn_sched_barrier(0);
   });
+  bool fresh = true;
   for (int q0 = 0; q0 < nsteps; q0 += kQueue) {
     static_for<kQueue>([&](auto kc) __attribute__((always_inline)) {
       constexpr int k = decltype(kc)::value;
       const v4f g = G[k];
       const float c = C[k];
-      D[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(g.x, c, D[0], 0, 0, 0);
-      D[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(g.y, c, D[1], 0, 0, 0);
-      D[2] = __builtin_amdgcn_mfma_f32_32x32x2f32(g.z, c, D[2], 0, 0, 0);
-      D[3] = __builtin_amdgcn_mfma_f32_32x32x2f32(g.w, c, D[3], 0, 0, 0);
+      if (fresh) {  // uniform: the first step of an m starts from zero (a constant operand, no registers to clear)
+        f16v zero;
+#pragma unroll
+        for (int v = 0; v < 16; v++) zero[v] = 0.f;
+        D[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(g.x, c, zero, 0, 0, 0);
+        D[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(g.y, c, zero, 0, 0, 0);
+        D[2] = __builtin_amdgcn_mfma_f32_32x32x2f32(g.z, c, zero, 0, 0, 0);
+        D[3] = __builtin_amdgcn_mfma_f32_32x32x2f32(g.w, c, zero, 0, 0, 0);
+      } else {
+        D[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(g.x, c, D[0], 0, 0, 0);
+        D[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(g.y, c, D[1], 0, 0, 0);
+        D[2] = __builtin_amdgcn_mfma_f32_32x32x2f32(g.z, c, D[2], 0, 0, 0);
+        D[3] = __builtin_amdgcn_mfma_f32_32x32x2f32(g.w, c, D[3], 0, 0, 0);
+      }
+      fresh = ck.left == 1;  // the next step starts a new m
       fetch(cf, G[k], C[k]);
       next_step(cf);
       __builtin_amdgcn_sched_barrier(0);

@@ -36,11 +36,30 @@ CASES = [
     (11, 7, 20, 7, 20, -1, True),    # Diag, 20 channels padded to 32: two cells per wave
     (3, 9, 64, 6, 64, -1, True),     # Diag, a full wave per cell
     (70, 6, 1, 5, 1, -1, False),     # one channel pair: 64 cells per wave
+    # 8 x 8 channels: the contraction over l runs on the matrix cores
+    (4, 12, 8, 9, 8, -1, False),     # l1 != l2: l from 3 to 21, 19 values
+    (3, 3, 8, 15, 8, -1, False),     # few rows of x, many of y: most columns of the matrix instructions idle
+    (5, 15, 8, 4, 8, -1, False),     # 31 rows of x: every column but the spare one in use
+    (7, 10, 8, 10, 8, 14, False),    # capped: m runs to 14 only, rows of the y-gradient end their journey early
+    (2, 7, 8, 7, 8, 3, False),       # four values of l
+    (33, 10, 8, 1, 8, -1, False),    # three values of l: left to the kernel that keeps its sums in LDS
 ]
 
 
+@pytest.mark.parametrize("mfma", [1, 0])
 @pytest.mark.parametrize("B,l1,n1,l2,n2,maxl,diag", CASES)
-def test_onepair_bwd(cabi, B, l1, n1, l2, n2, maxl, diag):
+def test_onepair_bwd(cabi, B, l1, n1, l2, n2, maxl, diag, mfma):
+    """Both forms of the family: with the matrix-core kernel allowed (it takes the 8 x 8 cases) and without it."""
+    if not mfma and (n1, n2) != (8, 8):
+        pytest.skip("the same kernel either way")
+    cabi.set_option("onepair_mfma", mfma)
+    try:
+        run_onepair(cabi, B, l1, n1, l2, n2, maxl, diag)
+    finally:
+        cabi.set_option("onepair_mfma", 1)
+
+
+def run_onepair(cabi, B, l1, n1, l2, n2, maxl, diag):
     seed = 1300 + B
     xs = [U.seeded(seed, B, 2 * l1 + 1, n1)]
     ys = [U.seeded(seed + 1, B, 2 * l2 + 1, n2)]

@@ -67,6 +67,7 @@ WORKLOADS = {
     "so3vec_cg_L2_tau64_B8192_maxl2": ("vec", 8192, {l: 64 for l in range(3)}, {l: 64 for l in range(3)}, 2, False),
     "so3vec_diagcg_L4_n64_B131072_uncapped": ("vec", 131072, {l: 64 for l in range(5)}, {l: 64 for l in range(5)}, -1, True),
     "so3part_cg_1x1to1_n16_B1024": ("vec", 1024, {1: 16}, {1: 16}, 1, False),
+    "so3vec_cg_l8l10_x_l9l10_tau4_B32768_maxl12": ("vec", 32768, {8: 4, 10: 4}, {9: 4, 10: 4}, 12, False),
 }
 HEADLINE = "so3vec_cg_L4_tau16_B32768_maxl4"
 # the configurations of the baseline list other than the headline, with the size of the CPU slice each is checked on
@@ -78,7 +79,7 @@ ALIASES = {"cfg1": "so3part_cg_1x1to1_n16_B1024", "cfg4": "so3vec_cg_L4_tau16_B3
            "cfg5": "so3part_cg_10x10_all_l_n8_B16384", "diag4": "so3vec_diagcg_L4_n64_B131072",
            "diag4n16": "so3vec_diagcg_L4_n16_B524288", "cg6": "so3vec_cg_L6_tau8_B16384_maxl6",
            "diag4u": "so3vec_diagcg_L4_n64_B131072_uncapped", "cg2n64": "so3vec_cg_L2_tau64_B8192_maxl2",
-           "cg4n4": "so3vec_cg_L4_tau4_B524288_maxl4"}
+           "cg4n4": "so3vec_cg_L4_tau4_B524288_maxl4", "cg10m": "so3vec_cg_l8l10_x_l9l10_tau4_B32768_maxl12"}
 
 
 def out_type(tx, ty, maxl, diag):

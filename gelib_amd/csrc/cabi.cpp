@@ -408,6 +408,67 @@ int vec_fwd_entry(bool diag, int nr, const gelib_part_desc *r, int nx, const gel
   return fwd_dispatch(plan, R, X, Y, accumulate, s);
 }
 
+// Vectors of several parts with l above 7: one launch of the single-pair kernels per (x part, y part) pair, each adding
+// its share to the two gradient parts it touches (launches on one stream run one after the other, so the order of the
+// additions is fixed).  The any-l kernels would otherwise take such vectors in one pass that adds partial sums into LDS
+// with float atomics; g is read once either way.  Taken only when every pair is one the single-pair kernels accept.
+int g_pairwise = 1;
+int pairwise_onepair_bwd(const VecPlan &plan, const std::vector<View> &G, const std::vector<View> &X,
+                         const std::vector<View> &Y, const std::vector<View> &XG, const std::vector<View> &YG,
+                         const std::vector<const gelib_part_desc *> &gd, bool want_x, bool want_y, int accumulate,
+                         hipStream_t s, int *used) {
+  *used = 0;
+  if (!g_pairwise || !want_x || !want_y || X.size() * Y.size() < 2) return GELIB_HIP_OK;
+  int lop = 0;
+  for (auto &v : X) lop = std::max(lop, v.l);
+  for (auto &v : Y) lop = std::max(lop, v.l);
+  if (g_pairwise == 1 && lop <= 7) return GELIB_HIP_OK;   // the striped kernels (fixed order, no atomics) take those
+  struct Sub {
+    VecPlan plan;
+    int p, q;
+  };
+  std::vector<Sub> subs;
+  for (int p = 0; p < (int)X.size(); p++)
+    for (int q = 0; q < (int)Y.size(); q++) {
+      Sub sub;
+      sub.p = p;
+      sub.q = q;
+      sub.plan.diag = plan.diag;
+      for (int k = 0; k < 3; k++) sub.plan.E[k] = plan.E[k];
+      for (auto t : plan.triples)
+        if (t.xi == p && t.yi == q) {
+          t.xi = t.yi = 0;
+          sub.plan.triples.push_back(t);
+        }
+      if (!sub.plan.triples.empty()) subs.push_back(sub);
+    }
+  if (subs.empty()) return GELIB_HIP_OK;
+  int rc;
+  for (auto &sub : subs) {  // first pass: would every pair be taken?
+    int ok = 0;
+    if ((rc = onepair_vec_bwd(sub.plan, gd, {X[sub.p].d}, {Y[sub.q].d}, {XG[sub.p].d}, {YG[sub.q].d}, true, s, &ok, true)))
+      return rc;
+    if (!ok) return GELIB_HIP_OK;
+  }
+  if (!accumulate) {  // every pair adds; a part that no pair feeds is still written (zeros)
+    for (auto *L : {&XG, &YG})
+      for (auto &v : *L) {
+        long long own[3];
+        PartDev pd = to_dev(v.d, plan.E, own);
+        if ((rc = launch_zero_fill(pd, own, 2 * v.l + 1, v.n, s))) return rc;
+      }
+  }
+  for (auto &sub : subs) {
+    int ok = 0;
+    const std::vector<const gelib_part_desc *> x1 = {X[sub.p].d}, y1 = {Y[sub.q].d}, xg1 = {XG[sub.p].d}, yg1 = {YG[sub.q].d};
+    if ((rc = onepair_mfma_vec_bwd(sub.plan, gd, x1, y1, xg1, yg1, true, s, &ok))) return rc;
+    if (!ok && (rc = onepair_vec_bwd(sub.plan, gd, x1, y1, xg1, yg1, true, s, &ok))) return rc;
+    if (!ok) return GELIB_HIP_ERR_ARG;  // cannot happen: the first pass asked
+  }
+  *used = 1;
+  return GELIB_HIP_OK;
+}
+
 int bwd_dispatch(const VecPlan &plan, const std::vector<View> &G, const std::vector<View> &X, const std::vector<View> &Y,
                  const std::vector<View> &XG, const std::vector<View> &YG, bool want_x, bool want_y, int accumulate,
                  hipStream_t s, bool skip_unrolled = false) {
@@ -441,6 +502,12 @@ int bwd_dispatch(const VecPlan &plan, const std::vector<View> &G, const std::vec
       return GELIB_HIP_OK;
     }
     rc = onepair_vec_bwd(plan, gd, xd, yd, xgd, ygd, accumulate != 0, s, &used);
+    if (rc) return rc;
+    if (used) {
+      t_last_path = kPathOnePair;
+      return GELIB_HIP_OK;
+    }
+    rc = pairwise_onepair_bwd(plan, G, X, Y, XG, YG, gd, want_x, want_y, accumulate, s, &used);
     if (rc) return rc;
     if (used) {
       t_last_path = kPathOnePair;
@@ -871,6 +938,10 @@ int gelib_hip_set_option(const char *name, int value) {
   if (!name) return GELIB_HIP_ERR_NULL;
   if (!std::strcmp(name, "force_generic")) {
     g_force_generic = value;
+    return GELIB_HIP_OK;
+  }
+  if (!std::strcmp(name, "pairwise_bwd")) {  // 0 never, 1 for operand l above 7, 2 wherever every pair qualifies
+    g_pairwise = value;
     return GELIB_HIP_OK;
   }
   if (!std::strcmp(name, "check_pointers")) {

@@ -264,7 +264,7 @@ int device_tables(int l1, int l2, int lmin, int lt, const std::vector<int> &pres
 int onepair_vec_bwd(const VecPlan &plan, const std::vector<const gelib_part_desc *> &g,
                     const std::vector<const gelib_part_desc *> &x, const std::vector<const gelib_part_desc *> &y,
                     const std::vector<const gelib_part_desc *> &xg, const std::vector<const gelib_part_desc *> &yg,
-                    bool accumulate, hipStream_t s, int *used) {
+                    bool accumulate, hipStream_t s, int *used, bool dry_run) {
   *used = 0;
   if (!g_enable || x.size() != 1 || y.size() != 1 || xg.size() != 1 || yg.size() != 1 || plan.triples.empty())
     return GELIB_HIP_OK;
@@ -323,6 +323,10 @@ int onepair_vec_bwd(const VecPlan &plan, const std::vector<const gelib_part_desc
   a.rec_off = (int)lds_f2;
   const size_t lds = (size_t)lds_f2 * sizeof(float2) + (size_t)std::max(kStepsMax * kRecord, 64 * 8) * sizeof(float);
   if (lds > 64 * 1024) return GELIB_HIP_OK;
+  if (dry_run) {  // the caller only asks whether this pair is one the kernel takes
+    *used = 1;
+    return GELIB_HIP_OK;
+  }
   if (plan.diag) hipLaunchKernelGGL(onepair_bwd_kernel<true>, dim3((unsigned)nblocks), dim3(64), lds, s, a);
   else hipLaunchKernelGGL(onepair_bwd_kernel<false>, dim3((unsigned)nblocks), dim3(64), lds, s, a);
   GELIB_HIP_TRY(hipGetLastError());

@@ -88,7 +88,7 @@ int staged_set_option(const char *name, int value);
 int onepair_vec_bwd(const VecPlan &plan, const std::vector<const gelib_part_desc *> &g,
                     const std::vector<const gelib_part_desc *> &x, const std::vector<const gelib_part_desc *> &y,
                     const std::vector<const gelib_part_desc *> &xg, const std::vector<const gelib_part_desc *> &yg,
-                    bool accumulate, hipStream_t s, int *used);
+                    bool accumulate, hipStream_t s, int *used, bool dry_run = false);
 int onepair_set_option(const char *name, int value);
 // The same for 8 x 8 channels and l1, l2 <= 15 with the contraction over l on the matrix cores (cg_onepair_mfma.hip).
 int onepair_mfma_vec_bwd(const VecPlan &plan, const std::vector<const gelib_part_desc *> &g,

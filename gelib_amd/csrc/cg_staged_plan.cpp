@@ -18,7 +18,10 @@ int g_bwd_enable = 1;
 int g_fwd_tile = 0;           // 0 = widest tile that fits, else force 1 / 2 / 4 (still subject to divisibility)
 int g_fwd_coeffs_lds = 1;     // forward coefficients staged in LDS when they fit
 int g_fwd_threads = 0;        // 0 = choose from the LDS footprint
-int g_bwd_stripes = 1;       // striped (register-accumulating) backward kernels: 0 never, 1 where they pay, 2 wherever they apply
+int g_bwd_stripes = 1;       // striped (register-accumulating) backward kernels: 0 never, otherwise wherever they apply
+int g_bwd_atomic = 0;        // single-pass backward kernels that add partial sums into LDS with float atomics (results
+                             // depend on timing in their last bits): 1 where the striped kernels do not apply, 0 never
+                             // (such products then run on the shape-agnostic kernels, in a fixed order)
 int g_bwd_pairs = 0;         // pair-wise single-pass backward kernel where the striped ones are not used: 1 yes, 0 no
                              // (off: measured slower than the triple-wise kernel, 6.5 vs 5.9 ms at l1 = l2 = 10)
 int g_bwd_threads = 0;       // 0 = choose from the LDS footprint, else force 256 / 512 / 1024
@@ -344,9 +347,10 @@ int run_bwd(bool diag, const std::vector<VecTriple> &triples, const std::vector<
   const DevicePlan *plan = nullptr;
   int rc = get_plan(diag, triples, xs, ys, rls, &plan);
   if (rc) return rc;
-  // The striped kernels win where rows are short (small l: an atomic per handful of terms in the other form); with
-  // 32 register rows for g and 32 for the sums they run at low occupancy and lose to the single-pass form.
-  const bool stripes_wanted = g_bwd_stripes == 2 || (g_bwd_stripes == 1 && plan->stripe_cap == 16);
+  // The striped kernels sum in a fixed order and win where rows are short; with 32 register rows for g and 32 for the
+  // sums (own l above 7) they run at low occupancy, still 2.7 times faster than the atomic single-pass form on vectors
+  // of several parts around l = 10 (6.7 against 18.4 ms; the per-pair route of the dispatcher takes those first).
+  const bool stripes_wanted = g_bwd_stripes != 0;
   if (stripes_wanted && plan->stripes_ok && 8LL * std::max(plan->xsize, plan->ysize) + 64 <= kLdsLimit) {
     // one launch per wanted gradient; LDS holds the other operand only
     StagedArgs a;
@@ -375,6 +379,7 @@ int run_bwd(bool diag, const std::vector<VecTriple> &triples, const std::vector<
     *used = 1;
     return GELIB_HIP_OK;
   }
+  if (!g_bwd_atomic) return GELIB_HIP_OK;  // what is left adds with float atomics: only on request
   const long long cell_bytes = 16LL * (plan->xsize + plan->ysize);  // operands + gradient images
   if (cell_bytes > kLdsLimit) return GELIB_HIP_OK;
   // n2 <= 64 and power-of-two channel counts hold here; the pair-wise kernel also needs uniform slots per pair,
@@ -502,6 +507,10 @@ int staged_set_option(const char *name, int value) {
   }
   if (!std::strcmp(name, "staged_bwd_stripes")) {
     g_bwd_stripes = value;
+    return GELIB_HIP_OK;
+  }
+  if (!std::strcmp(name, "staged_bwd_atomic")) {
+    g_bwd_atomic = value;
     return GELIB_HIP_OK;
   }
   if (!std::strcmp(name, "staged_bwd_pairs")) {

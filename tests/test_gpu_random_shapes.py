@@ -81,6 +81,15 @@ def test_random_product(cabi, seed):
     torch.cuda.synchronize()
     path = cabi.last_path()
     O.check_bwd(None if dxg is None else [U.host(a) for a in dxg], [U.host(a) for a in dyg], tag + " path %d" % path)
+    # no kernel on the default dispatch adds with atomics: a second run gives the same bits, forward and backward
+    drs2 = [U.dev(a) for a in start]
+    cabi.so3vec_fwd(drs2, dxs, dys, accumulate=accumulate, diag=diag)
+    dyg2 = [torch.full_like(a, 2.0 + 1j) for a in dyg]
+    dxg2 = None if dxg is None else [torch.full_like(a, 2.0 + 1j) for a in dxg]
+    cabi.so3vec_bwd(dxg2, dyg2, dgs, dxs, dys, accumulate=False, diag=diag)
+    torch.cuda.synchronize()
+    for a, b in zip(drs + dyg + (dxg or []), drs2 + dyg2 + (dxg2 or [])):
+        assert torch.equal(torch.view_as_real(a), torch.view_as_real(b)), tag + " path %d: two runs differ" % path
 
 
 @pytest.mark.parametrize("seed", range(120))

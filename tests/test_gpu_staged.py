@@ -21,20 +21,27 @@ STAGED = 3
 def cabi(request):
     """The three backward forms of the family: one gradient per launch with sums in registers; both gradients in
     one launch, one (x part, y part) pair at a time, contracting over l first; and both gradients in one launch,
-    one triple at a time.  Each is forced wherever its conditions hold (the library picks one of them by itself)."""
+    one triple at a time.  Each is forced wherever its conditions hold.  By itself the library uses the first only: the
+    other two add partial sums with LDS float atomics and run on request ("staged_bwd_atomic")."""
     assert torch.cuda.is_available(), "GPU tests need a GPU"
     from gelib_amd import cabi as c
     c.lib()
     c.set_option("force_generic", 0)
     c.set_option("diag6", 0)   # the lane-per-channel Diag kernels would take some of these cases first
-    c.set_option("onepair", 0) # and the single-pair backward kernel others
-    c.set_option("staged_bwd_stripes", 2 if request.param == "striped" else 0)
+    c.set_option("onepair", 0) # and the single-pair backward kernels others
+    c.set_option("onepair_mfma", 0)
+    c.set_option("pairwise_bwd", 0)
+    c.set_option("staged_bwd_stripes", 1 if request.param == "striped" else 0)
+    c.set_option("staged_bwd_atomic", 1)   # the other two forms (and what the striped one leaves) add with LDS float atomics
     c.set_option("staged_bwd_pairs", int(request.param == "pairwise"))
     yield c
     c.set_option("diag6", 1)
     c.set_option("onepair", 1)
+    c.set_option("onepair_mfma", 1)
+    c.set_option("pairwise_bwd", 1)
     c.set_option("staged_bwd_threads", 0)
     c.set_option("staged_bwd_stripes", 1)
+    c.set_option("staged_bwd_atomic", 0)
     c.set_option("staged_bwd_pairs", 0)
 
 

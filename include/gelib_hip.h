@@ -216,8 +216,12 @@ int gelib_hip_synchronize(void);
  * "staged_fwd" / "staged_bwd" / "diag6" / "onepair" (1/0: use the family), "fwd_block_bytes", "fwd_lds_bytes", "fwd_tile",
  * "fwd_cell_tile" (cells per tile of the unrolled forward launch, 0 = one tile),
  * "staged_fwd_tile" (1, 2, 4), "staged_fwd_threads", "staged_fwd_coeffs_lds" (1/0), "staged_fwd_lds_target",
- * "staged_bwd_lds_target", "staged_bwd_threads" (256, 512, 1024), "staged_bwd_stripes" (0 never, 1 where they pay,
- * 2 wherever they apply), "staged_bwd_pairs" (1/0: pair-wise single-pass backward kernel, off by default).  Unknown names return GELIB_HIP_ERR_ARG.  Options are process-wide.
+ * "staged_bwd_lds_target", "staged_bwd_threads" (256, 512, 1024), "staged_bwd_stripes" (0 never, otherwise wherever they
+ * apply), "staged_bwd_atomic" (1/0: allow the single-pass backward kernels that add with LDS float atomics; off by
+ * default, so that results do not depend on timing), "staged_bwd_pairs" (1/0: the pair-wise one of those),
+ * "pairwise_bwd" (one launch of the single-pair kernels per pair of parts: 0 never, 1 for operand l above 7, 2 wherever
+ * every pair qualifies), "onepair_mfma" (1/0: the matrix-core form of the single-pair kernel).  Unknown names return
+ * GELIB_HIP_ERR_ARG.  Options are process-wide.
  * gelib_hip_last_path() tells which kernel family the last call of this thread used
  * (0 = none, 1 = generic, 2 = unrolled small-l kernels, 3 = staged any-l kernels, 4 = lane-per-channel Diag
  * kernels for operand l up to 6, 5 = single-pair backward kernel for large l).

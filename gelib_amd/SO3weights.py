@@ -91,3 +91,67 @@ class SO3linear(torch.nn.Module):
 
     def forward(self, x):
         return x * self.W
+
+
+class CGproductLinearFn(torch.autograd.Function):
+    """CGproduct(x, y, maxl) * W with the product formed and consumed inside one kernel (forward).  The backward pass
+    forms the product again, through the unfused functions, and differentiates those: nothing of the product's size is
+    kept between the two passes."""
+
+    @staticmethod
+    def forward(ctx, k1, k2, maxl, *args):
+        from gelib_amd import cabi
+        xs, ys, ws = list(args[0:k1]), list(args[k1:k1 + k2]), list(args[k1 + k2:])
+        ctx.k1, ctx.k2, ctx.maxl = k1, k2, maxl
+        ctx.save_for_backward(*args)
+        lead = list(xs[0].shape[:-2])
+        out = [torch.empty(lead + [2 * l + 1, w.shape[1]], dtype=torch.complex64, device=xs[0].device)
+               for l, w in enumerate(ws)]
+        if not cabi.so3vec_cg_linear_fwd(out, xs, ys, ws, accumulate=False):
+            raise RuntimeError("CGproduct_linear: shapes outside what the fused kernel takes")
+        return tuple(out)
+
+    @staticmethod
+    def backward(ctx, *gargs):
+        from gelib_amd.SO3vec import SO3vec
+        k1, k2 = ctx.k1, ctx.k2
+        leaves = [t.detach().requires_grad_() for t in ctx.saved_tensors]
+        with torch.enable_grad():
+            x, y = SO3vec(*leaves[0:k1]), SO3vec(*leaves[k1:k1 + k2])
+            out = x.CGproduct(y, ctx.maxl) * SO3weights(*leaves[k1 + k2:])
+            outs = list(out.parts.values())
+        wanted = [t for t, need in zip(leaves, ctx.needs_input_grad[3:]) if need]
+        got = iter(torch.autograd.grad(outs, wanted, [g.contiguous() for g in gargs]))
+        return tuple([None, None, None] + [next(got) if need else None for need in ctx.needs_input_grad[3:]])
+
+
+def fused_linear_ok(x, y, W, maxl):
+    """True when CGproduct(x, y, maxl) * W is a case of the fused kernel: complex64 parts on one GPU, contiguous, the same
+    leading dimensions, l <= 4 and at most 16 channels everywhere, a product with exactly the parts l = 0..4."""
+    xs, ys, ws = list(x.parts.values()), list(y.parts.values()), list(W.parts)
+    ts = xs + ys + ws
+    if not ts or not all(t.is_cuda and t.dtype == torch.complex64 and t.is_contiguous() and t.device == ts[0].device
+                         for t in ts):
+        return False
+    if any(t.shape[:-2] != xs[0].shape[:-2] for t in xs + ys) or xs[0].numel() == 0:
+        return False
+    if max(x.parts) > 4 or max(y.parts) > 4 or any(t.shape[-1] > 16 for t in xs + ys):
+        return False
+    from gelib_amd import cabi
+    taus = cabi.so3type_product(x.tau(), y.tau(), maxl)
+    if sorted(taus) != [0, 1, 2, 3, 4] or len(ws) != 5:
+        return False
+    return all(w.dim() == 2 and w.shape[0] == taus[l] and 1 <= w.shape[1] <= 16 for l, w in enumerate(ws))
+
+
+def CGproduct_linear(x, y, W, maxl=-1):
+    """x.CGproduct(y, maxl) * W (python/src/gelib/SO3vec.py:174-177 applied to the result of SO3vec.CGproduct).  On the GPU,
+    for the shapes fused_linear_ok accepts, one kernel forms the product and multiplies it by the matrices without
+    storing it; every other case runs the two steps one after the other."""
+    from gelib_amd.SO3vec import SO3vec
+    if fused_linear_ok(x, y, W, maxl):
+        xs = [p.as_subclass(torch.Tensor) for p in x.parts.values()]
+        ys = [p.as_subclass(torch.Tensor) for p in y.parts.values()]
+        ws = [w.as_subclass(torch.Tensor) for w in W.parts]
+        return SO3vec(*CGproductLinearFn.apply(len(xs), len(ys), maxl, *(xs + ys + ws)))
+    return x.CGproduct(y, maxl) * W

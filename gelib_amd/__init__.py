@@ -14,7 +14,7 @@ from gelib_amd.SO3part import SO3part, SO3part_CGproductFn, SO3part_DiagCGproduc
 from gelib_amd.SO3vec import SO3vec, SO3vec_CGproductFn, SO3vec_DiagCGproductFn  # noqa: F401
 from gelib_amd.SO3partArr import SO3partArr, SO3partArr_CGproductFn, SO3partArr_DiagCGproductFn  # noqa: F401
 from gelib_amd.SO3vecArr import SO3vecArr, SO3vecArr_CGproductFn, SO3vecArr_DiagCGproductFn  # noqa: F401
-from gelib_amd.SO3weights import SO3weights, SO3linear  # noqa: F401
+from gelib_amd.SO3weights import SO3weights, SO3linear, CGproduct_linear  # noqa: F401
 from gelib_amd.gather_map import gather_map  # noqa: F401
 from gelib_amd.O3 import O3element, O3irrep, O3type, O3part, O3vec, O3vec_CGproductFn, O3vec_DiagCGproductFn  # noqa: F401
 

@@ -19,6 +19,7 @@ SYMBOLS = [
     "gelib_hip_so3vec_diagcg_bwd", "gelib_hip_so3part_spharm", "gelib_hip_gather_map_create",
     "gelib_hip_gather_map_destroy", "gelib_hip_part_gather", "gelib_hip_part_mix_channels",
     "gelib_hip_part_mix_channels_static", "gelib_hip_part_mix_channels_wgrad", "gelib_hip_part_mix_workspace_bytes",
+    "gelib_hip_so3vec_cg_linear_fwd", "gelib_hip_so3vec_cg_linear_workspace_bytes",
     "gelib_hip_set_option",
     "gelib_hip_last_path",
     "gelib_hip_malloc", "gelib_hip_free", "gelib_hip_memcpy", "gelib_hip_memset", "gelib_hip_synchronize",
@@ -81,6 +82,11 @@ def lib():
         L.gelib_hip_part_mix_channels_static.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
                                                          ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.c_int64,
                                                          ctypes.c_int64, ctypes.c_int, ctypes.c_void_p]
+        L.gelib_hip_so3vec_cg_linear_fwd.argtypes = [ctypes.c_int, P, ctypes.c_int, P, ctypes.c_int, P,
+                                                     ctypes.POINTER(ctypes.c_void_p), ctypes.c_int, ctypes.c_void_p,
+                                                     ctypes.c_uint64, ctypes.c_void_p]
+        L.gelib_hip_so3vec_cg_linear_workspace_bytes.restype = ctypes.c_uint64
+        L.gelib_hip_so3vec_cg_linear_workspace_bytes.argtypes = [ctypes.c_int, P, ctypes.c_int, P, ctypes.c_int, P]
         L.gelib_hip_part_mix_workspace_bytes.restype = ctypes.c_uint64
         L.gelib_hip_part_mix_workspace_bytes.argtypes = [ctypes.c_int, ctypes.c_int64, ctypes.c_int, ctypes.c_int]
         L.gelib_hip_set_option.argtypes = [ctypes.c_char_p, ctypes.c_int]
@@ -188,6 +194,28 @@ def so3vec_bwd(xgparts, ygparts, gparts, xparts, yparts, accumulate=True, diag=F
     fn = lib().gelib_hip_so3vec_diagcg_bwd if diag else lib().gelib_hip_so3vec_cg_bwd
     check(fn(_arr(xgparts), _arr(ygparts), len(gparts), _arr(gparts), len(xparts), _arr(xparts), len(yparts),
              _arr(yparts), int(accumulate), _stream(gparts[0])))
+
+
+UNSUPPORTED = 15
+
+
+def so3vec_cg_linear_fwd(rparts, xparts, yparts, wparts, accumulate=False):
+    """rparts[k] (+)= CGproduct(x, y)[l of rparts[k]] @ wparts[k] in one pass that never stores the product.  False
+    (nothing launched) when the shapes are not ones the fused kernel takes; every other failure raises."""
+    import torch
+    L = lib()
+    ra, xa, ya = _arr(rparts), _arr(xparts), _arr(yparts)
+    nbytes = int(L.gelib_hip_so3vec_cg_linear_workspace_bytes(len(rparts), ra, len(xparts), xa, len(yparts), ya))
+    if nbytes == 0:
+        return False
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=rparts[0].device)
+    wp = (ctypes.c_void_p * len(wparts))(*[w.data_ptr() for w in wparts])
+    rc = L.gelib_hip_so3vec_cg_linear_fwd(len(rparts), ra, len(xparts), xa, len(yparts), ya, wp, int(accumulate),
+                                          ctypes.c_void_p(ws.data_ptr()), nbytes, _stream(rparts[0]))
+    if rc == UNSUPPORTED:
+        return False
+    check(rc)
+    return True
 
 
 def so3part_spharm(r, x, accumulate=True):

@@ -11,6 +11,7 @@
 #include <vector>
 
 #include "cg_common.h"
+#include "cg_linear.h"
 #include "cg_staged.h"
 #include "cg_unrolled.h"
 
@@ -252,8 +253,10 @@ int sort_parts(int n, const gelib_part_desc *parts, int max_parts, std::vector<V
   return GELIB_HIP_OK;
 }
 
+// check_channels = false: the parts of R only say which l are wanted (the fused product -> mixing entry, whose
+// destination has the mixing's output channels, not the product's)
 int build_vec_plan(bool diag, const std::vector<View> &R, const std::vector<View> &X, const std::vector<View> &Y,
-                   VecPlan &plan) {
+                   VecPlan &plan, bool check_channels = true) {
   for (auto &v : X)
     if (v.l > kMaxL) return GELIB_HIP_ERR_PARTS;
   for (auto &v : Y)
@@ -277,7 +280,8 @@ int build_vec_plan(bool diag, const std::vector<View> &R, const std::vector<View
         if (k < 0) continue;  // absent product part: skipped, offsets of other parts unaffected
         if (diag && X[p].n != Y[q].n) return GELIB_HIP_ERR_DIAG_CHANNELS;
         const long long nout = diag ? X[p].n : (long long)X[p].n * Y[q].n;
-        if (offset[l] + nout > R[k].n) return GELIB_HIP_ERR_CHANNELS;
+        if (check_channels && offset[l] + nout > R[k].n) return GELIB_HIP_ERR_CHANNELS;
+        if (offset[l] + nout > 0x7fffffffLL) return GELIB_HIP_ERR_CHANNELS;
         plan.triples.push_back({p, q, k, l1, l2, l, (int)offset[l], (int)nout});
         offset[l] += nout;
       }
@@ -605,6 +609,60 @@ int vec_bwd_entry(bool diag, const gelib_part_desc *xg, const gelib_part_desc *y
   return bwd_dispatch(plan, G, X, Y, XG, YG, xg != nullptr, yg != nullptr, accumulate, s);
 }
 
+// Channels of the product's parts (indexed like R) for a plan built with check_channels = false.
+std::vector<long long> product_channels(const VecPlan &plan, size_t nparts) {
+  std::vector<long long> tau(nparts, 0);
+  for (auto &t : plan.triples) tau[t.ri] = std::max(tau[t.ri], (long long)t.offs + t.nout);
+  return tau;
+}
+
+int linear_fwd_entry(int nr, const gelib_part_desc *r, int nx, const gelib_part_desc *x, int ny,
+                     const gelib_part_desc *y, const void *const *w, int accumulate, void *workspace,
+                     uint64_t workspace_bytes, void *stream) {
+  t_last_path = kPathNone;
+  std::vector<View> R, X, Y;
+  int rc;
+  if ((rc = sort_parts(nr, r, kMaxOutParts, R)) || (rc = sort_parts(nx, x, kMaxParts, X)) ||
+      (rc = sort_parts(ny, y, kMaxParts, Y)))
+    return rc;
+  if (R.empty() || X.empty() || Y.empty()) return GELIB_HIP_OK;
+  if (!w) return GELIB_HIP_ERR_NULL;
+  VecPlan plan;
+  if ((rc = build_vec_plan(false, R, X, Y, plan, false))) return rc;
+  const std::vector<long long> tau = product_channels(plan, R.size());
+  std::vector<const float2 *> W(R.size());
+  for (size_t k = 0; k < R.size(); k++) {
+    W[k] = (const float2 *)w[R[k].d - r];
+    if (tau[k] > 0 && R[k].n > 0 && !W[k]) return GELIB_HIP_ERR_NULL;
+  }
+  for (auto &v : R)
+    if ((rc = check_dest(v.d))) return rc;
+  for (auto &v : R)
+    if ((rc = check_pointer(v.d))) return rc;
+  for (auto &v : X)
+    if ((rc = check_pointer(v.d))) return rc;
+  for (auto &v : Y)
+    if ((rc = check_pointer(v.d))) return rc;
+  for (size_t k = 0; k < R.size(); k++) {
+    if (tau[k] == 0 || R[k].n == 0) continue;
+    const int64_t wd[5] = {tau[k], 1, 1, 1, R[k].n}, wst[5] = {R[k].n, 0, 0, 0, 1};
+    if ((rc = check_range(W[k], wd, wst, 2 * sizeof(float)))) return rc;
+  }
+  const int64_t sd[5] = {(int64_t)workspace_bytes, 1, 1, 1, 1}, sst[5] = {1, 0, 0, 0, 0};
+  if (workspace && workspace_bytes && (rc = check_range(workspace, sd, sst, 1))) return rc;
+  if (plan.E[0] * plan.E[1] * plan.E[2] == 0) return GELIB_HIP_OK;
+  std::vector<const gelib_part_desc *> rd, xd, yd;
+  for (auto &v : R) rd.push_back(v.d);
+  for (auto &v : X) xd.push_back(v.d);
+  for (auto &v : Y) yd.push_back(v.d);
+  int used = 0;
+  rc = cg_linear_fwd(plan, rd, xd, yd, W, accumulate != 0, workspace, (size_t)workspace_bytes, (hipStream_t)stream, &used);
+  if (rc) return rc;
+  if (!used) return GELIB_HIP_ERR_UNSUPPORTED;
+  t_last_path = kPathLinear;
+  return GELIB_HIP_OK;
+}
+
 }  // namespace
 }  // namespace gelib_hip
 
@@ -629,6 +687,8 @@ const char *gelib_hip_strerror(int status) {
     case GELIB_HIP_ERR_TOO_LARGE:
       return "the packed matrix of n_in x n_out channels exceeds the 8 MiB array of the entry point that allocates "
              "nothing; use gelib_hip_part_mix_channels with a workspace";
+    case GELIB_HIP_ERR_UNSUPPORTED:
+      return "shapes outside what the fused kernel takes; form the product and mix its channels in two calls";
   }
   return "unknown status";
 }
@@ -702,6 +762,27 @@ int gelib_hip_so3vec_diagcg_bwd(const gelib_part_desc *xg, const gelib_part_desc
                                 const gelib_part_desc *g, int nx, const gelib_part_desc *x, int ny,
                                 const gelib_part_desc *y, int accumulate, void *stream) {
   return vec_bwd_entry(true, xg, yg, ng, g, nx, x, ny, y, accumulate, stream);
+}
+
+int gelib_hip_so3vec_cg_linear_fwd(int nr, const gelib_part_desc *r, int nx, const gelib_part_desc *x, int ny,
+                                   const gelib_part_desc *y, const void *const *w, int accumulate, void *workspace,
+                                   uint64_t workspace_bytes, void *stream) {
+  return linear_fwd_entry(nr, r, nx, x, ny, y, w, accumulate, workspace, workspace_bytes, stream);
+}
+uint64_t gelib_hip_so3vec_cg_linear_workspace_bytes(int nr, const gelib_part_desc *r, int nx, const gelib_part_desc *x,
+                                                    int ny, const gelib_part_desc *y) {
+  std::vector<View> R, X, Y;
+  if (sort_parts(nr, r, kMaxOutParts, R) || sort_parts(nx, x, kMaxParts, X) || sort_parts(ny, y, kMaxParts, Y)) return 0;
+  VecPlan plan;
+  if (R.empty() || X.empty() || Y.empty() || build_vec_plan(false, R, X, Y, plan, false)) return 0;
+  const std::vector<long long> tau = product_channels(plan, R.size());
+  if (R.size() != (size_t)kLinL + 1) return 0;
+  long long t5[kLinL + 1];
+  for (int l = 0; l <= kLinL; l++) {
+    if (R[l].l != l) return 0;
+    t5[l] = tau[l];
+  }
+  return (uint64_t)cg_linear_workspace_bytes(t5);
 }
 
 int gelib_hip_so3part_spharm(const gelib_part_desc *r, const float *x, const int64_t xdims[5],

@@ -29,7 +29,7 @@ struct PartOp {
   bool diag;
 };
 
-enum PathId { kPathNone = 0, kPathGeneric = 1, kPathUnrolled = 2, kPathStaged = 3, kPathDiag6 = 4, kPathOnePair = 5 };
+enum PathId { kPathNone = 0, kPathGeneric = 1, kPathUnrolled = 2, kPathStaged = 3, kPathDiag6 = 4, kPathOnePair = 5, kPathLinear = 6 };
 
 // ---- coefficient bank (cg_bank.cpp) ----
 double cg_coeff(int l1, int l2, int l, int m1, int m2);

@@ -37,6 +37,10 @@ constexpr TableOffsets kTables = make_table_offsets();
 constexpr int table_off(int l1, int l2, int l) { return kTables.v[l1][l2][l]; }
 constexpr int kBankFloats = (kTables.total + 1) & ~1;  // even, so that the zeros behind it are 8-byte aligned
 
+// The bank on the current device (built and uploaded on first use, kept for the life of the process): kBankFloats
+// coefficients, table (l1, l2, l) at table_off(l1, l2, l), followed by kZeroFloats zeros.
+int cg_table_bank(const float **out);
+
 struct Diag6Args {
   FastPart x[kNP], y[kNP], xg[kNP], yg[kNP];  // by l; ptr == nullptr: no such part
   FastPart r[kNR];                            // product (forward) or its gradient (backward), by l

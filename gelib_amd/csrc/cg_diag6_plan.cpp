@@ -118,6 +118,8 @@ int make_args(const VecPlan &plan, const std::vector<const gelib_part_desc *> &r
 
 }  // namespace
 
+int cg_table_bank(const float **out) { return device_bank(out); }
+
 int diag6_vec_fwd(const VecPlan &plan, const std::vector<const gelib_part_desc *> &r,
                   const std::vector<const gelib_part_desc *> &x, const std::vector<const gelib_part_desc *> &y,
                   bool accumulate, hipStream_t s, int *used) {

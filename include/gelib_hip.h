@@ -45,7 +45,8 @@ enum gelib_hip_status {
   GELIB_HIP_ERR_BROADCAST_DEST = 11, /* the destination has a dimension of extent > 1 with stride 0 (an expanded view) */
   GELIB_HIP_ERR_ARG = 12,          /* negative offset, negative stride or other malformed argument                   */
   GELIB_HIP_ERR_WORKSPACE = 13,    /* workspace missing, not 16-byte aligned or smaller than the size query says     */
-  GELIB_HIP_ERR_TOO_LARGE = 14     /* sizes beyond the stated maximum of gelib_hip_part_mix_channels_static          */
+  GELIB_HIP_ERR_TOO_LARGE = 14,    /* sizes beyond the stated maximum of gelib_hip_part_mix_channels_static          */
+  GELIB_HIP_ERR_UNSUPPORTED = 15   /* gelib_hip_so3vec_cg_linear_fwd: shapes outside what the fused kernel takes     */
 };
 
 #define GELIB_HIP_MAX_L 32          /* largest l of an operand part                     */
@@ -173,6 +174,28 @@ int gelib_hip_part_mix_channels_wgrad(void *wg, const void *x, const void *g, in
 /* Bytes of workspace the two calls above need: kind 0 for gelib_hip_part_mix_channels (either value of adjoint; n_in and
  * n_out as passed to that call), kind 1 for gelib_hip_part_mix_channels_wgrad.  0 for empty shapes or an unknown kind. */
 uint64_t gelib_hip_part_mix_workspace_bytes(int kind, int64_t rows, int n_in, int n_out);
+
+/* ---- CGproduct followed by the weight matrices, in one pass ---------------------------------------------------------------
+ * out_l[.., m, o] (+)= sum over c of P_l[.., m, c] w_l[c, o] with P = CGproduct(x, y) restricted to the l of the parts of
+ * r, its channels c in the order of core/Gvec.hpp:311-321 -- what the model code of the reference writes as
+ * CGproduct(x, y, maxl) * W (python/src/gelib/SO3vec.py:174-177 followed by the per-part matmul of SO3vec.__mul__ with an
+ * SO3weights) -- without ever storing P.  r: nr parts (.., 2l+1, n_out_l) that receive the result; w[k] belongs to r[k]:
+ * device pointer to the row-major (tau_l, n_out_l) complex matrix, tau_l = channels of part l of the product (host array
+ * of nr pointers).  workspace: device memory of at least gelib_hip_so3vec_cg_linear_workspace_bytes(...) bytes, 16-byte
+ * aligned, for the matrices re-packed for the matrix cores (same rules as for gelib_hip_part_mix_channels; the library
+ * allocates nothing per call).  Taken by the fused kernel: r with every l = 0..4 and at most 16 channels per part,
+ * operand parts with l <= 4 and at most 16 channels, contiguous channels, leading dimensions that collapse into one
+ * index.  Anything else returns GELIB_HIP_ERR_UNSUPPORTED with nothing launched: the caller then forms the product with
+ * gelib_hip_so3vec_cg_fwd and mixes each part with gelib_hip_part_mix_channels.  The sums over c run in a fixed order
+ * (ascending c per row, in float32 on the matrix cores); results agree with the two-call form to rounding, not bit for
+ * bit. */
+int gelib_hip_so3vec_cg_linear_fwd(int nr, const gelib_part_desc *r, int nx, const gelib_part_desc *x, int ny,
+                                   const gelib_part_desc *y, const void *const *w, int accumulate, void *workspace,
+                                   uint64_t workspace_bytes, void *stream);
+/* Bytes of workspace the call above needs for these parts (256 per product channel plus 4096 per part); 0 when the
+ * descriptors are malformed or r does not have exactly the parts l = 0..4. */
+uint64_t gelib_hip_so3vec_cg_linear_workspace_bytes(int nr, const gelib_part_desc *r, int nx, const gelib_part_desc *x,
+                                                    int ny, const gelib_part_desc *y);
 
 /* ---- gather: sums of slices along the batch or a grid dimension ---------------------------------------------------------
  * A gather map is a list of (source, target) pairs with 0 <= source < n_in, 0 <= target < n_out (the arguments of

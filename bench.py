@@ -269,7 +269,110 @@ def aux_bench(torch, args, name):
     print(json.dumps(out))
 
 
-PATH_NAMES = {1: "generic", 2: "unrolled", 3: "staged", 4: "diag6", 5: "onepair"}
+FUSED_WORKLOAD = "so3vec_cg_linear_L4_tau16_to16_B32768"
+MFMA_F32_PEAK = 157.3e12
+
+
+def fused_linear_bench(torch, args):
+    """CGproduct(x, y, maxl = 4) of the headline operands followed by the per-l weight matrices (16 output channels), forward:
+    the fused entry point, which never stores the product, timed beside the two-step form (product launch + one
+    channel-mixing launch per part) on the same inputs.  The fused kernel is bound by the matrix and vector units, not by
+    memory: its roofline record counts the flops of the product (8 per complex multiply-add of a term) and of the mixing
+    against the float32 matrix-core peak."""
+    import numpy as np
+    from gelib_amd import cabi
+    dev = torch.device("cuda:0")
+    B = args.batch or 32768
+    tx = {l: 16 for l in range(5)}
+    tr = out_type(tx, tx, 4, False)
+    n_out = 16
+    xs = seeded_parts(torch, 101, B, tx, dev)
+    ys = seeded_parts(torch, 202, B, tx, dev)
+    ws = []
+    for l, n in tr.items():
+        g = torch.Generator(device=dev).manual_seed(303 + l)
+        ws.append(torch.view_as_complex(torch.randn(n, n_out, 2, generator=g, device=dev)) / float(n) ** 0.5)
+    outs = [torch.empty(B, 2 * l + 1, n_out, dtype=torch.complex64, device=dev) for l in tr]
+    outs2 = [torch.empty_like(o) for o in outs]
+    prod = [torch.empty(B, 2 * l + 1, n, dtype=torch.complex64, device=dev) for l, n in tr.items()]
+
+    def fused():
+        assert cabi.so3vec_cg_linear_fwd(outs, xs, ys, ws, accumulate=False)
+
+    def two_step():
+        cabi.so3vec_fwd(prod, xs, ys, accumulate=False)
+        for o, p, w in zip(outs2, prod, ws):
+            cabi.part_mix_channels(o, p, w)
+
+    def timed(fn):
+        for _ in range(args.warmup):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t0 = time.perf_counter()
+        e0.record()
+        for _ in range(args.steps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / args.steps, (time.perf_counter() - t0) / args.steps
+
+    fused_ms, fused_wall = timed(fused)
+    two_ms, _ = timed(two_step)
+    # terms (m1, m2) of one channel of every (l1, l2, l) block
+    terms = sum(1 for l1 in tx for l2 in tx for l in range(abs(l1 - l2), min(l1 + l2, 4) + 1)
+                for m in range(-l, l + 1) for m1 in range(-l1, l1 + 1) if abs(m - m1) <= l2)
+    flops_product = 8 * terms * 16 * 16 * B
+    flops_mix = 8 * sum((2 * l + 1) * n for l, n in tr.items()) * n_out * B
+    flops = flops_product + flops_mix
+    product_bytes = 8 * B * sum((2 * l + 1) * n for l, n in tr.items())
+    out = {"metric": "SO3vec CGproduct -> linear, forward, samples/s at L=4 (fused kernel)", "value": B / fused_wall,
+           "unit": "samples/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+           "ms_per_step": fused_wall * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+           "dtype": "f32", "data": "synthetic",
+           "config": {"workload": FUSED_WORKLOAD, "batch": B, "tau_x": tx, "tau_y": tx, "maxl": 4, "tau_product": tr,
+                      "n_out": n_out, "fused_fwd_ms": fused_ms, "two_step_fwd_ms": two_ms,
+                      "speedup_over_two_step": two_ms / fused_ms,
+                      "product_bytes_never_stored": product_bytes,
+                      "flops": {"product": flops_product, "mixing": flops_mix}},
+           "roofline": {"bound": "mfma", "kernel": "cg_linear_fwd (two launches, one per half of the rows)",
+                        "achieved": flops / (fused_ms * 1e-3) / 1e12, "peak": MFMA_F32_PEAK / 1e12, "unit": "TFLOP/s",
+                        "frac": flops / (fused_ms * 1e-3) / MFMA_F32_PEAK, "traffic": None,
+                        "algorithmic_flops_per_step": flops}}
+    if not args.no_cpu:
+        from oracle import cg_oracle as ora
+        from tests import gpu_util as U
+        ns = min(B, 2048)
+        hx = [t[:ns].cpu().numpy() for t in xs]
+        hy = [t[:ns].cpu().numpy() for t in ys]
+        hw = [w.cpu().numpy() for w in ws]
+        t0 = time.perf_counter()
+        p32 = ora.vec_fwd(hx, hy, 4, False, nthreads=1)
+        r32 = [np.matmul(p, w) for p, w in zip(p32, hw)]
+        dt = time.perf_counter() - t0
+        p64 = ora.vec_fwd(U.c128(hx), U.c128(hy), 4, False, nthreads=1)
+        r64 = [np.matmul(p, w.astype(np.complex128)) for p, w in zip(p64, hw)]
+        S = [np.matmul(s, (np.abs(w.real) + np.abs(w.imag)).astype(np.float64))
+             for s, w in zip(ora.vec_fwd_term_sums(hx, hy, 4, False, 1), hw)]
+        reps = [U.parity_counts(o[:ns].cpu().numpy(), a, b, c) for o, a, b, c in zip(outs, r32, r64, S)]
+        n = sum(r["components"] for r in reps)
+        out["cpu_baseline"] = {"value": ns / dt, "unit": "samples/s", "cores": 1, "kind": "port",
+                               "sample": "first %d samples: oracle product, then numpy complex64 matmuls, %.1f s" % (ns, dt)}
+        out["parity"] = {"ok": all(r["rejected"] == 0 for r in reps), "samples": ns, "components": n,
+                         "outside_gate": sum(r["outside_gate"] * r["components"] for r in reps) / n,
+                         "cpu_f32_outside_gate_of_f64": sum(r["cpu_f32_outside_gate_of_f64"] * r["components"] for r in reps) / n,
+                         "by_rule_B": sum(r["by_rule_B"] * r["components"] for r in reps) / n,
+                         "by_rule_C": sum(r["by_rule_C"] * r["components"] for r in reps) / n,
+                         "rejected": sum(r["rejected"] for r in reps),
+                         "max_err_over_rule_C_bound": max(r["max_err_over_rule_C_bound"] for r in reps),
+                         "two_step_vs_fused_max_abs_diff": max(float((a - b).abs().max()) for a, b in zip(outs, outs2))}
+    print(json.dumps(out))
+    if "parity" in out and not out["parity"]["ok"]:
+        print("bench.py: a fused result on the CPU slice passes none of the parity rules", file=sys.stderr)
+        sys.exit(3)
+
+
+PATH_NAMES = {1: "generic", 2: "unrolled", 3: "staged", 4: "diag6", 5: "onepair", 6: "linear"}
 
 
 def run_cg_workload(torch, cabi, name, steps, warmup, batch=0, cpu_samples=0, single_core=False, copy_probe=False,
@@ -399,6 +502,8 @@ def main():
         k, v = kv.split("=")
         cabi.set_option(k, int(v))
     name = ALIASES.get(args.workload, args.workload)
+    if name in ("fused_linear", FUSED_WORKLOAD):
+        return fused_linear_bench(torch, args)
     aux = [w for w in AUX_WORKLOADS if w == name or w.split("_")[0] == name]
     if aux:
         return aux_bench(torch, args, aux[0])

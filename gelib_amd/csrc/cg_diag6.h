@@ -54,6 +54,7 @@ struct Diag6Args {
   int offs_add;
   int accumulate;
   int want_x, want_y;  // backward: which gradients are stored (the operand of an unwanted one is never read)
+  int owner[kNP];      // backward: which of the block's four waves takes the pairs with this l2
 };
 
 int launch_diag6_fwd_l6(const Diag6Args &a, hipStream_t s);  // product l up to 6

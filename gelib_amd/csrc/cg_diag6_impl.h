@@ -326,12 +326,9 @@ __device__ __forceinline__ void store_rows(const float2 *v, int vstride, const F
   }
 }
 
-// Which of the four waves of a block owns the pairs with this l2: {6}, {5,0}, {4,1}, {3,2} -- 13, 12, 12 and 12 rows
-// of y, so the waves finish every l1 at about the same time.
-constexpr int owner_of(int l2) { return l2 == 6 ? 0 : (l2 == 5 || l2 == 0) ? 1 : (l2 == 4 || l2 == 1) ? 2 : 3; }
-
-// The four waves of a block share one cell and channel group.  Each owns the pairs of its l2 set, so its rows of the
-// y-gradient image are its own (plain read-add-write).  The x-gradient of part l1 gets a partial sum from every
+// The four waves of a block share one cell and channel group.  Each owns the pairs of its set of l2 (a.owner[l2], dealt
+// by the host so that the waves get about the same number of rows of y: {6}, {5,0}, {4,1}, {3,2} when every part up to
+// l = 6 is there), so its rows of the y-gradient image are its own (plain read-add-write).  The x-gradient of part l1 gets a partial sum from every
 // wave; the partials meet in LDS after the last pair of l1, are added in the order of the waves and written out, the
 // rows dealt round-robin to the waves.  Pairs (l1, l2) and (l1, l2 +- 1) read neighbouring 512-byte blocks of the same
 // rows of g, and they are in flight at about the same time.
@@ -366,7 +363,7 @@ __global__ void __launch_bounds__(256) diag6_bwd_kernel(const Diag6Args a) {
       for (int m1 = 0; m1 <= 2 * L1; m1++) ax[m1] = make_float2(0.f, 0.f);
       static_for<kNP>([&](auto l2c) __attribute__((always_inline)) {
         constexpr int L2 = kL6 - decltype(l2c)::value;  // descending, so that neighbours in l2 run at the same time
-        if (owner_of(L2) == wave && a.y[L2].ptr != nullptr) {
+        if (a.owner[L2] == wave && a.y[L2].ptr != nullptr) {
           float2 yv[2 * L2 + 1];
           if (wx) {
             load_rows<L2, PACKED>(yv, a.y[L2], q);
@@ -405,7 +402,7 @@ __global__ void __launch_bounds__(256) diag6_bwd_kernel(const Diag6Args a) {
   static_for<kNP>([&](auto l2c) __attribute__((always_inline)) {
     constexpr int L2 = decltype(l2c)::value;
     const FastPart YG = a.yg[L2];
-    if (wy && owner_of(L2) == wave && YG.ptr != nullptr)
+    if (wy && a.owner[L2] == wave && YG.ptr != nullptr)
       store_rows<L2, PACKED>(yimg + (L2 * L2) * 64 + lane, 64, YG, q, accumulate);
   });
 }

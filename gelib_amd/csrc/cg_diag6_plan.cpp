@@ -81,6 +81,20 @@ int make_args(const VecPlan &plan, const std::vector<const gelib_part_desc *> &r
   for (size_t i = 0; i < fr.size(); i++) a->r[lr[i].first] = fr[i];
   for (size_t i = 0; i < fxg.size(); i++) a->xg[lx[i].first] = fxg[i];
   for (size_t i = 0; i < fyg.size(); i++) a->yg[ly[i].first] = fyg[i];
+  {
+    // deal the parts of y to the four waves of a backward block, largest first, each to the wave with the fewest rows
+    // so far: the waves then finish every l1 at about the same time
+    int rows[4] = {0, 0, 0, 0};
+    for (int l2 = kL6; l2 >= 0; l2--) {
+      a->owner[l2] = 0;
+      if (!a->y[l2].ptr) continue;
+      int w = 0;
+      for (int k = 1; k < 4; k++)
+        if (rows[k] < rows[w]) w = k;
+      a->owner[l2] = w;
+      rows[w] += 2 * l2 + 1;
+    }
+  }
   std::vector<int> offs((size_t)kNP * kNP * kNR, -1);
   *lcap = 0;
   for (auto &t : plan.triples) {

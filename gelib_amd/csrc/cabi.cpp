@@ -356,6 +356,12 @@ int fwd_dispatch(const VecPlan &plan, const std::vector<View> &R, const std::vec
       t_last_path = kPathUnrolled;
       return GELIB_HIP_OK;
     }
+    rc = onepair_mfma_vec_fwd(plan, rd, xd, yd, accumulate != 0, s, &used);
+    if (rc) return rc;
+    if (used) {
+      t_last_path = kPathOnePair;
+      return GELIB_HIP_OK;
+    }
     rc = staged_vec_fwd(plan, rd, xd, yd, accumulate != 0, s, &used);
     if (rc) return rc;
     if (used) {
@@ -1031,7 +1037,7 @@ int gelib_hip_set_option(const char *name, int value) {
   }
   if (!std::strncmp(name, "staged_", 7)) return staged_set_option(name, value);
   if (!std::strncmp(name, "diag6", 5)) return diag6_set_option(name, value);
-  if (!std::strcmp(name, "onepair_mfma")) return onepair_mfma_set_option(name, value);
+  if (!std::strncmp(name, "onepair_mfma", 12)) return onepair_mfma_set_option(name, value);
   if (!std::strncmp(name, "onepair", 7)) return onepair_set_option(name, value);
   if (!std::strncmp(name, "mix_", 4)) return mix_set_option(name, value);
   return unrolled_set_option(name, value);

@@ -20,6 +20,18 @@
 // No atomics, a fixed order of additions.  The vector unit does 256 multiply-adds per m and lane (both gradients),
 // the matrix cores the 2 x (21 - |m|)^2 x 128 of the contraction; the operands of the next eight steps are always in
 // flight, across the boundaries between the m.
+//
+// The forward pass of the same product (second kernel of this file) is the mirror image: for one m
+//     r_l[m, chan] = sum_m1 P_m[chan, m1] C_l[m1, m - m1],   P_m[chan, m1] = x[m1, a] y[m - m1, j],
+// here the ROWS of D are the l and its columns the floats of the 64 channels (four tiles of 32 columns), a step of the
+// reduction is two values of m1.  Lane (i, h) supplies C_{lmin + i}[m1(h), m - m1(h)] from a table in lane order (the A
+// operand) and forms four floats of the product x[m1(h)] y[m - m1(h)] from LDS (the B operands of the four tiles): column
+// i of tile t is float 4 i + t of the row, i.e. the lane's floats are the real and imaginary parts of channels 2 i and
+// 2 i + 1 = (a, j) and (a, j + 1) with a = i / 4: one x, two neighbouring y, eight operations.  After the steps of one m
+// register v of the four tiles holds floats 4 i .. 4 i + 3 of row r_l[m] with l = lmin + 8 (v / 4) + 4 h + v % 4: one
+// 16-byte store per lane, and a store instruction writes one complete 512-byte row for each half of the wave.  (With
+// the channels as rows and the l as columns a lane owned 16-byte pieces of 21 different rows and the stores left as
+// 32-byte pieces: 1.47 ms instead of the any-l kernel's 1.05.)
 #include <cstring>
 #include <map>
 #include <mutex>
@@ -41,6 +53,8 @@ struct OnePairMfmaArgs {
   int offs[kNLm];     // first channel of the triple's block in its part
   const float *coef;  // device: 64 floats (lane order) per (m, step)
   int nsteps;         // steps of all m, rounded up to a multiple of the kernel's queue length (idle steps at the end)
+  const float *coef_fwd;  // the same for the forward kernel (steps over m1, columns l)
+  int nsteps_fwd;
   long long ncells;
   int l1, l2, lmin, lt, nl;
   int offs_add, accumulate;
@@ -49,6 +63,7 @@ struct OnePairMfmaArgs {
 typedef float f16v __attribute__((ext_vector_type(16)));
 typedef float v4f __attribute__((ext_vector_type(4)));
 typedef const __attribute__((address_space(1))) v4f *GlobalIn4;
+typedef __attribute__((address_space(1))) v4f *GlobalOut4;
 typedef const __attribute__((address_space(1))) float *GlobalIn1;
 typedef const __attribute__((address_space(4))) int *IntPtr;
 
@@ -257,15 +272,130 @@ __global__ void __launch_bounds__(64) onepair_mfma_bwd_kernel(const OnePairMfmaA
   }
 }
 
+
+constexpr int kStepsM = (2 * kMaxLm + 2) / 2;  // most steps of one m (forward): two values of m1 per step
+constexpr int kColsF = 24;                     // columns (values of l) the forward coefficient table keeps per step and m1
+constexpr int kCellsF = 4;                     // cells (waves) per block of the forward kernel
+
+// Forward: g[] are the parts of the product (written), x and y the operands.  A block of four waves takes four cells and
+// shares one copy of the coefficient table in LDS (2 x 24 floats per step, 44 KB at l1 = l2 = 10), loaded by all of
+// its threads while the waves set up their cells.  Nothing is loaded from memory once the rows are being stored: loads
+// and stores return through one in-order counter, and a wait for a load issued behind stores waits for the stores to
+// be acknowledged (with the coefficients fetched from memory step by step the waves spent a third of their time so).
+__global__ void __launch_bounds__(64 * kCellsF) onepair_mfma_fwd_kernel(const OnePairMfmaArgs a) {
+  extern __shared__ float4 smem4[];
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63, i = lane & 31, h = lane >> 5;
+  const int l1 = a.l1, l2 = a.l2, lmin = a.lmin, lt = a.lt, nl = a.nl;
+  const int r1 = 2 * l1 + 1, r2 = 2 * l2 + 1;
+  float *ctab = reinterpret_cast<float *>(smem4);
+  const int tab4 = a.nsteps_fwd * (2 * kColsF / 4);  // float4s of the table
+  float2 *xs = reinterpret_cast<float2 *>(smem4 + tab4) + wave * ((r1 + r2) * 8);
+  float2 *ys = xs + r1 * 8;  // r1 * 8 float2 = a multiple of 16 bytes
+  {
+    const float4 *src = reinterpret_cast<const float4 *>(a.coef_fwd);
+    for (int e = threadIdx.x; e < tab4; e += 64 * kCellsF) smem4[e] = src[e];
+  }
+  long long cell = (long long)blockIdx.x * kCellsF + wave;
+  const bool live = cell < a.ncells;  // a wave beyond the last cell repeats it and stores nothing
+  cell = live ? cell : a.ncells - 1;
+  for (int e = lane; e < r1 * 8; e += 64) xs[e] = a.x.ptr[cell * a.x.sb + (long long)(e >> 3) * a.x.sm + (e & 7)];
+  for (int e = lane; e < r2 * 8; e += 64) ys[e] = a.y.ptr[cell * a.y.sb + (long long)(e >> 3) * a.y.sm + (e & 7)];
+  // Register v of a tile belongs to part l = lmin + 8 (v / 4) + 4 h + v % 4.  cur[v]: the lane's 16 bytes of row m of
+  // that part for the m at hand (the rows of a part start at m = -l; before that the address is not used), advanced by
+  // the part's row length after every m.  A part that is not there has lrow[v] = -1.
+  unsigned long long cur[16];
+  unsigned rowb[16];
+  int lrow[16];
+  static_for<16>([&](auto vc) __attribute__((always_inline)) {
+    constexpr int v = decltype(vc)::value;
+    cur[v] = 0;
+    rowb[v] = 0;
+    lrow[v] = -1;
+    static_for<2>([&](auto hc) __attribute__((always_inline)) {
+      constexpr int dl = 8 * (v / 4) + 4 * decltype(hc)::value + (v % 4);
+      if constexpr (dl < kNLm) {
+        if (hc.value == h && dl < nl && live && a.g[dl].ptr != nullptr) {
+          const FastPart P = a.g[dl];
+          rowb[v] = (unsigned)P.sm * 8u;
+          cur[v] = (unsigned long long)(P.ptr + cell * P.sb + (a.offs[dl] + a.offs_add)) +
+                   (unsigned long long)((long long)(lmin + dl - lt) * (long long)rowb[v]) + (unsigned)i * 16u;
+          lrow[v] = lmin + dl;
+        }
+      }
+    });
+  });
+  const float2 *xmine = xs + (i >> 2);                                              // row r: xmine[r * 8]
+  const float4 *ymine = reinterpret_cast<const float4 *>(ys) + (i & 3);           // row r: ymine[r * 4] = y[r, j], y[r, j + 1]
+  // the lane's coefficient of step s: ctab[s * 48 + cslot]; columns beyond the table hold no part (coefficient zero)
+  const bool has_col = i < kColsF;
+  const float *cmine = ctab + h * kColsF + (has_col ? i : 0);
+  __syncthreads();
+
+  const bool accumulate = a.accumulate != 0;
+  f16v D[4];
+  int at = 0;  // first step of the m at hand in the table
+  for (int m = -lt; m <= lt; m++) {
+    const int lo = (m - l2 > -l1) ? m - l2 : -l1, hi = (m + l2 < l1) ? m + l2 : l1;
+    const int nst = (hi - lo + 2) >> 1;
+    static_for<kStepsM>([&](auto kc) __attribute__((always_inline)) {
+      constexpr int k = decltype(kc)::value;
+      if (k < nst) {  // uniform
+        // the lane's m1 of this step (the second of an odd count is clamped: its coefficient is zero) and its m2
+        int m1 = lo + 2 * k + h;
+        m1 = m1 > l1 ? l1 : m1;
+        int m2 = m - m1;
+        m2 = m2 < -l2 ? -l2 : (m2 > l2 ? l2 : m2);
+        const float2 xv = xmine[(m1 + l1) * 8];
+        const float4 yv = ymine[(m2 + l2) * 4];
+        const float cl = cmine[(at + k) * (2 * kColsF)];
+        const float c = has_col ? cl : 0.f;
+        const float p0 = fmaf(-xv.y, yv.y, xv.x * yv.x), p1 = fmaf(xv.y, yv.x, xv.x * yv.y);
+        const float p2 = fmaf(-xv.y, yv.w, xv.x * yv.z), p3 = fmaf(xv.y, yv.z, xv.x * yv.w);
+        if constexpr (k == 0) {  // the first step of an m starts from zero (a constant operand, no registers to clear)
+          f16v zero;
+#pragma unroll
+          for (int v = 0; v < 16; v++) zero[v] = 0.f;
+          D[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(c, p0, zero, 0, 0, 0);
+          D[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(c, p1, zero, 0, 0, 0);
+          D[2] = __builtin_amdgcn_mfma_f32_32x32x2f32(c, p2, zero, 0, 0, 0);
+          D[3] = __builtin_amdgcn_mfma_f32_32x32x2f32(c, p3, zero, 0, 0, 0);
+        } else {
+          D[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(c, p0, D[0], 0, 0, 0);
+          D[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(c, p1, D[1], 0, 0, 0);
+          D[2] = __builtin_amdgcn_mfma_f32_32x32x2f32(c, p2, D[2], 0, 0, 0);
+          D[3] = __builtin_amdgcn_mfma_f32_32x32x2f32(c, p3, D[3], 0, 0, 0);
+        }
+      }
+    });
+    // register v of the four tiles: floats 4 i .. 4 i + 3 of row m of part lrow[v]
+    const int mabs = m < 0 ? -m : m;
+#pragma unroll
+    for (int v = 0; v < 16; v++) {
+      if (lrow[v] >= mabs) {
+        GlobalOut4 p = (GlobalOut4)cur[v];
+        v4f o;
+        o.x = D[0][v], o.y = D[1][v], o.z = D[2][v], o.w = D[3][v];
+        if (accumulate) o += *p;
+        *p = o;
+      }
+      cur[v] += rowb[v];
+    }
+    at += nst;
+  }
+}
+
 // ---- host side ---------------------------------------------------------------------------------------------------
 
 struct Tables {
   float *coef;
   int nsteps;
+  float *coef_fwd;
+  int nsteps_fwd;
 };
 std::mutex g_mutex;
 std::map<std::vector<int>, Tables> g_tables;  // (device, l1, l2, lmin, lt, nl, present...) -> device tables
-int g_enable = 1;
+int g_enable = 1, g_enable_fwd = 1;
 
 int device_tables(int l1, int l2, int lmin, int lt, int nl, const std::vector<int> &present, Tables *out) {
   int dev = 0;
@@ -303,9 +433,27 @@ int device_tables(int l1, int l2, int lmin, int lt, int nl, const std::vector<in
     }
     coef.insert(coef.end(), (size_t)kQueue * 64, 0.f);  // the queue runs kQueue steps ahead, also at the end; the start
                                                           // of the table doubles as the harmless row (512 bytes at least)
-    Tables t{nullptr, step};
+    // forward: steps over m1 (two per step), 24 columns (l) per m1: [step][h][column]
+    std::vector<float> cfwd;
+    int fstep = 0;
+    for (int m = -lt; m <= lt; m++) {
+      const int lo = std::max(-l1, m - l2), hi = std::min(l1, m + l2);
+      const int nks = (hi - lo + 2) / 2;
+      for (int ks = 0; ks < nks; ks++, fstep++)
+        for (int h = 0; h < 2; h++)
+          for (int dl = 0; dl < kColsF; dl++) {
+            const int m1 = lo + 2 * ks + h, m2 = m - m1;
+            float c = 0.f;
+            if (dl < nl && present[dl] && m1 <= hi && std::abs(m) <= lmin + dl)
+              c = C[dl][(size_t)(m1 + l1) * (2 * l2 + 1) + (m2 + l2)];
+            cfwd.push_back(c);
+          }
+    }
+    Tables t{nullptr, step, nullptr, fstep};
     GELIB_HIP_TRY(hipMalloc((void **)&t.coef, coef.size() * sizeof(float)));
     GELIB_HIP_TRY(hipMemcpy(t.coef, coef.data(), coef.size() * sizeof(float), hipMemcpyHostToDevice));
+    GELIB_HIP_TRY(hipMalloc((void **)&t.coef_fwd, cfwd.size() * sizeof(float)));
+    GELIB_HIP_TRY(hipMemcpy(t.coef_fwd, cfwd.data(), cfwd.size() * sizeof(float), hipMemcpyHostToDevice));
     it = g_tables.emplace(key, t).first;
   }
   *out = it->second;
@@ -373,7 +521,67 @@ int onepair_mfma_vec_bwd(const VecPlan &plan, const std::vector<const gelib_part
   return GELIB_HIP_OK;
 }
 
+// The product itself for the same shapes (non-Diag, 8 x 8 channels, l1, l2 <= 15, 4 to 22 values of l).
+int onepair_mfma_vec_fwd(const VecPlan &plan, const std::vector<const gelib_part_desc *> &r,
+                         const std::vector<const gelib_part_desc *> &x, const std::vector<const gelib_part_desc *> &y,
+                         bool accumulate, hipStream_t s, int *used) {
+  *used = 0;
+  if (!g_enable_fwd || plan.diag || x.size() != 1 || y.size() != 1 || plan.triples.empty()) return GELIB_HIP_OK;
+  std::vector<FastPart> fx, fy, fr;
+  std::vector<std::pair<int, int>> lx, ly, lr;
+  if (!lists_to_fast(x, plan.E, false, &fx, &lx) || !lists_to_fast(y, plan.E, false, &fy, &ly) ||
+      !lists_to_fast(r, plan.E, true, &fr, &lr))
+    return GELIB_HIP_OK;
+  const int l1 = lx[0].first, l2 = ly[0].first, n1 = lx[0].second, n2 = ly[0].second;
+  if (n1 != 8 || n2 != 8 || l1 > kMaxLm || l2 > kMaxLm) return GELIB_HIP_OK;
+  const int lmin = std::abs(l1 - l2);
+  int lmax = -1;
+  for (auto &t : plan.triples) lmax = std::max(lmax, t.l);
+  const int nl = lmax - lmin + 1;
+  if (nl > kNLm || nl < 4) return GELIB_HIP_OK;
+  static_assert(kNLm <= kColsF, "the forward table keeps one column per value of l");
+  OnePairMfmaArgs a;
+  std::memset(&a, 0, sizeof(a));
+  a.x = fx[0];
+  a.y = fy[0];
+  std::vector<int> present(nl, 0);
+  for (auto &t : plan.triples) {
+    const int dl = t.l - lmin;
+    a.g[dl] = fr[t.ri];
+    a.offs[dl] = t.offs;
+    present[dl] = 1;
+    // a lane stores 16 bytes at a time: block offset, row and cell strides even, base aligned
+    if (((t.offs) & 1) || (fr[t.ri].sm & 1) || (fr[t.ri].sb & 1) || ((uintptr_t)fr[t.ri].ptr & 15)) return GELIB_HIP_OK;
+  }
+  const long long ncells = plan.E[0] * plan.E[1] * plan.E[2];
+  if (ncells > 0x7fffffffLL) return GELIB_HIP_OK;
+  Tables t;
+  const int lt = std::min(l1 + l2, lmax);
+  int rc = device_tables(l1, l2, lmin, lt, nl, present, &t);
+  if (rc) return rc;
+  a.coef_fwd = t.coef_fwd;
+  a.nsteps_fwd = t.nsteps_fwd;
+  a.ncells = ncells;
+  a.l1 = l1;
+  a.l2 = l2;
+  a.lmin = lmin;
+  a.lt = lt;
+  a.nl = nl;
+  a.accumulate = accumulate ? 1 : 0;
+  // LDS of a block: the table and four cells' operands; beyond what a block may ask for, the any-l kernels take the pair
+  const size_t lds = (size_t)t.nsteps_fwd * 2 * kColsF * 4 + (size_t)kCellsF * (2 * l1 + 1 + 2 * l2 + 1) * 64;
+  if (lds > 64 * 1024) return GELIB_HIP_OK;
+  hipLaunchKernelGGL(onepair_mfma_fwd_kernel, dim3((unsigned)((ncells + kCellsF - 1) / kCellsF)), dim3(64 * kCellsF), lds, s, a);
+  GELIB_HIP_TRY(hipGetLastError());
+  *used = 1;
+  return GELIB_HIP_OK;
+}
+
 int onepair_mfma_set_option(const char *name, int value) {
+  if (!std::strcmp(name, "onepair_mfma_fwd")) {
+    g_enable_fwd = value;
+    return GELIB_HIP_OK;
+  }
   if (!std::strcmp(name, "onepair_mfma")) {
     g_enable = value;
     return GELIB_HIP_OK;

@@ -95,6 +95,10 @@ int onepair_mfma_vec_bwd(const VecPlan &plan, const std::vector<const gelib_part
                          const std::vector<const gelib_part_desc *> &x, const std::vector<const gelib_part_desc *> &y,
                          const std::vector<const gelib_part_desc *> &xg, const std::vector<const gelib_part_desc *> &yg,
                          bool accumulate, hipStream_t s, int *used);
-int onepair_mfma_set_option(const char *name, int value);
+// The forward pass of the same shapes on the matrix cores (the reduction over m1).
+int onepair_mfma_vec_fwd(const VecPlan &plan, const std::vector<const gelib_part_desc *> &r,
+                         const std::vector<const gelib_part_desc *> &x, const std::vector<const gelib_part_desc *> &y,
+                         bool accumulate, hipStream_t s, int *used);
+int onepair_mfma_set_option(const char *name, int value);  // "onepair_mfma", "onepair_mfma_fwd": 0 switches the kernel off
 
 }  // namespace gelib_hip

@@ -1,5 +1,6 @@
-"""GPU parity of the backward kernel for products of ONE x part with ONE y part of large l (l1 + l2 <= 21, at most 64
-channel slots per cell): gelib_hip_last_path() == 5, gradients against the CPU oracle in float32 and float64."""
+"""GPU parity of the kernels for products of ONE x part with ONE y part of large l (l1 + l2 <= 21, at most 64 channel
+slots per cell): gelib_hip_last_path() == 5, gradients (and, for 8 x 8 channels, the product itself on the matrix
+cores) against the CPU oracle in float32 and float64."""
 import numpy as np
 import pytest
 
@@ -97,3 +98,41 @@ def test_onepair_leaves_the_rest_alone(cabi):
     xg11, yg11 = [torch.zeros_like(x11[0])], [torch.zeros_like(y11[0])]
     cabi.so3vec_bwd(xg11, yg11, g11, x11, y11, accumulate=False)
     assert cabi.last_path() != ONEPAIR
+
+
+FWD_CASES = [c for c in CASES if (c[2], c[4]) == (8, 8) and not c[6] and c[1] + c[3] >= 3 and c[0] != 33]
+
+
+@pytest.mark.parametrize("B,l1,n1,l2,n2,maxl,diag", FWD_CASES)
+def test_onepair_fwd_on_the_matrix_cores(cabi, B, l1, n1, l2, n2, maxl, diag):
+    """The product itself for 8 x 8 channels: overwrite into garbage, accumulate on top, a block at a channel offset of a
+    wider part (the other channels must stay as they were), and the same bits on a second run."""
+    seed = 1700 + B
+    xs = [U.seeded(seed, B, 2 * l1 + 1, n1)]
+    ys = [U.seeded(seed + 1, B, 2 * l2 + 1, n2)]
+    O = U.VecOracle(xs, ys, maxl, diag)
+    dxs, dys = [U.dev(a) for a in xs], [U.dev(a) for a in ys]
+    drs = [torch.full(p.shape, 7.0 + 1j, dtype=torch.complex64, device="cuda") for p in O.r32]
+    cabi.so3vec_fwd(drs, dxs, dys, accumulate=False, diag=diag)
+    assert cabi.last_path() == ONEPAIR
+    torch.cuda.synchronize()
+    tag = "fwd B%d (%d,%d)x(%d,%d) maxl %d" % (B, l1, n1, l2, n2, maxl)
+    O.check_fwd([U.host(a) for a in drs], tag)
+    start = [U.seeded(seed + 20 + k, *p.shape) for k, p in enumerate(O.r32)]
+    drs2 = [U.dev(a) for a in start]
+    cabi.so3vec_fwd(drs2, dxs, dys, accumulate=True, diag=diag)
+    assert cabi.last_path() == ONEPAIR
+    drs3 = [torch.empty_like(t) for t in drs]
+    cabi.so3vec_fwd(drs3, dxs, dys, accumulate=False, diag=diag)
+    torch.cuda.synchronize()
+    O.check_fwd_onto([U.host(a) for a in drs2], start, tag + " onto")
+    assert all(torch.equal(a.view(torch.float32), b.view(torch.float32)) for a, b in zip(drs, drs3))
+    # part-level calls with a channel offset into wider parts
+    l = min(l1 + l2, maxl if maxl >= 0 else l1 + l2)
+    wide = torch.full((B, 2 * l + 1, 64 + 6), 5.0 - 3j, dtype=torch.complex64, device="cuda")
+    cabi.so3part_cg_fwd(wide, dxs[0], dys[0], offs=4, accumulate=False)
+    torch.cuda.synchronize()
+    hw = U.host(wide)
+    k = [p.shape[1] for p in O.r32].index(2 * l + 1)
+    U.assert_parity(hw[:, :, 4:68], O.r32[k], O.r64[k], O.Sr[k], tag + " offset block")
+    assert np.all(hw[:, :, :4] == np.complex64(5.0 - 3j)) and np.all(hw[:, :, 68:] == np.complex64(5.0 - 3j))

@@ -30,6 +30,7 @@ def cabi(request):
     c.set_option("diag6", 0)   # the lane-per-channel Diag kernels would take some of these cases first
     c.set_option("onepair", 0) # and the single-pair backward kernels others
     c.set_option("onepair_mfma", 0)
+    c.set_option("onepair_mfma_fwd", 0)
     c.set_option("pairwise_bwd", 0)
     c.set_option("staged_bwd_stripes", 1 if request.param == "striped" else 0)
     c.set_option("staged_bwd_atomic", 1)   # the other two forms (and what the striped one leaves) add with LDS float atomics
@@ -38,6 +39,7 @@ def cabi(request):
     c.set_option("diag6", 1)
     c.set_option("onepair", 1)
     c.set_option("onepair_mfma", 1)
+    c.set_option("onepair_mfma_fwd", 1)
     c.set_option("pairwise_bwd", 1)
     c.set_option("staged_bwd_threads", 0)
     c.set_option("staged_bwd_stripes", 1)

@@ -55,6 +55,7 @@ struct OnePairMfmaArgs {
   int nsteps;         // steps of all m, rounded up to a multiple of the kernel's queue length (idle steps at the end)
   const float *coef_fwd;  // the same for the forward kernel (steps over m1, columns l)
   int nsteps_fwd;
+  long long rowb;         // forward: bytes between the rows of every part of the product
   long long ncells;
   int l1, l2, lmin, lt, nl;
   int offs_add, accumulate;
@@ -275,13 +276,14 @@ __global__ void __launch_bounds__(64) onepair_mfma_bwd_kernel(const OnePairMfmaA
 
 constexpr int kStepsM = (2 * kMaxLm + 2) / 2;  // most steps of one m (forward): two values of m1 per step
 constexpr int kColsF = 24;                     // columns (values of l) the forward coefficient table keeps per step and m1
-constexpr int kCellsF = 4;                     // cells (waves) per block of the forward kernel
+constexpr int kCellsF = 8;                     // cells (waves) per block of the forward kernel
 
-// Forward: g[] are the parts of the product (written), x and y the operands.  A block of four waves takes four cells and
-// shares one copy of the coefficient table in LDS (2 x 24 floats per step, 44 KB at l1 = l2 = 10), loaded by all of
+// Forward: g[] are the parts of the product (written), x and y the operands.  A block of eight waves takes eight cells
+// and shares one copy of the coefficient table in LDS (2 x 24 floats per step, 44 KB at l1 = l2 = 10), loaded by all of
 // its threads while the waves set up their cells.  Nothing is loaded from memory once the rows are being stored: loads
 // and stores return through one in-order counter, and a wait for a load issued behind stores waits for the stores to
 // be acknowledged (with the coefficients fetched from memory step by step the waves spent a third of their time so).
+// All parts have the same row length (a.rowb; the host sends other cases to the any-l kernels).
 __global__ void __launch_bounds__(64 * kCellsF) onepair_mfma_fwd_kernel(const OnePairMfmaArgs a) {
   extern __shared__ float4 smem4[];
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -290,8 +292,11 @@ __global__ void __launch_bounds__(64 * kCellsF) onepair_mfma_fwd_kernel(const On
   const int r1 = 2 * l1 + 1, r2 = 2 * l2 + 1;
   float *ctab = reinterpret_cast<float *>(smem4);
   const int tab4 = a.nsteps_fwd * (2 * kColsF / 4);  // float4s of the table
-  float2 *xs = reinterpret_cast<float2 *>(smem4 + tab4) + wave * ((r1 + r2) * 8);
-  float2 *ys = xs + r1 * 8;  // r1 * 8 float2 = a multiple of 16 bytes
+  // per wave: x with one row of zeros behind it, y with one row of zeros on either side (the second m1 of an odd count
+  // reads one row too far; its coefficient is zero, so the row must only be finite)
+  const int wave4 = (r1 + 1 + r2 + 2) * 4;  // float4s: a row is 8 complex = 4 float4
+  float2 *xs = reinterpret_cast<float2 *>(smem4 + tab4 + wave * wave4);
+  float2 *ys = xs + (r1 + 1) * 8 + 8;  // row 0 of y; the zero row sits in front of it
   {
     const float4 *src = reinterpret_cast<const float4 *>(a.coef_fwd);
     for (int e = threadIdx.x; e < tab4; e += 64 * kCellsF) smem4[e] = src[e];
@@ -301,35 +306,37 @@ __global__ void __launch_bounds__(64 * kCellsF) onepair_mfma_fwd_kernel(const On
   cell = live ? cell : a.ncells - 1;
   for (int e = lane; e < r1 * 8; e += 64) xs[e] = a.x.ptr[cell * a.x.sb + (long long)(e >> 3) * a.x.sm + (e & 7)];
   for (int e = lane; e < r2 * 8; e += 64) ys[e] = a.y.ptr[cell * a.y.sb + (long long)(e >> 3) * a.y.sm + (e & 7)];
+  if (lane < 8) {
+    xs[r1 * 8 + lane] = make_float2(0.f, 0.f);
+    ys[lane - 8] = make_float2(0.f, 0.f);
+    ys[r2 * 8 + lane] = make_float2(0.f, 0.f);
+  }
   // Register v of a tile belongs to part l = lmin + 8 (v / 4) + 4 h + v % 4.  cur[v]: the lane's 16 bytes of row m of
   // that part for the m at hand (the rows of a part start at m = -l; before that the address is not used), advanced by
-  // the part's row length after every m.  A part that is not there has lrow[v] = -1.
+  // the row length after every m.  Bit v of `there`: the part exists and the wave has a cell.
+  const long long rowb = a.rowb;
   unsigned long long cur[16];
-  unsigned rowb[16];
-  int lrow[16];
+  unsigned there = 0;
   static_for<16>([&](auto vc) __attribute__((always_inline)) {
     constexpr int v = decltype(vc)::value;
     cur[v] = 0;
-    rowb[v] = 0;
-    lrow[v] = -1;
     static_for<2>([&](auto hc) __attribute__((always_inline)) {
       constexpr int dl = 8 * (v / 4) + 4 * decltype(hc)::value + (v % 4);
       if constexpr (dl < kNLm) {
         if (hc.value == h && dl < nl && live && a.g[dl].ptr != nullptr) {
           const FastPart P = a.g[dl];
-          rowb[v] = (unsigned)P.sm * 8u;
           cur[v] = (unsigned long long)(P.ptr + cell * P.sb + (a.offs[dl] + a.offs_add)) +
-                   (unsigned long long)((long long)(lmin + dl - lt) * (long long)rowb[v]) + (unsigned)i * 16u;
-          lrow[v] = lmin + dl;
+                   (unsigned long long)((long long)(lmin + dl - lt) * rowb) + (unsigned)i * 16u;
+          there |= 1u << v;
         }
       }
     });
   });
-  const float2 *xmine = xs + (i >> 2);                                              // row r: xmine[r * 8]
-  const float4 *ymine = reinterpret_cast<const float4 *>(ys) + (i & 3);           // row r: ymine[r * 4] = y[r, j], y[r, j + 1]
-  // the lane's coefficient of step s: ctab[s * 48 + cslot]; columns beyond the table hold no part (coefficient zero)
-  const bool has_col = i < kColsF;
-  const float *cmine = ctab + h * kColsF + (has_col ? i : 0);
+  const int lbase = lmin + 4 * h;  // l of register v: lbase + 8 (v / 4) + v % 4
+  const char *xmine = reinterpret_cast<const char *>(xs + (i >> 2));   // row r: + r * 64 bytes
+  const char *ymine = reinterpret_cast<const char *>(ys) + (i & 3) * 16;  // row r: + r * 64: y[r, j], y[r, j + 1]
+  // the lane's coefficient of step s: 192 s bytes on; the columns beyond the table's read its last one, which is zero
+  const char *cmine = reinterpret_cast<const char *>(ctab + h * kColsF + (i < kColsF ? i : kColsF - 1));
   __syncthreads();
 
   const bool accumulate = a.accumulate != 0;
@@ -338,18 +345,17 @@ __global__ void __launch_bounds__(64 * kCellsF) onepair_mfma_fwd_kernel(const On
   for (int m = -lt; m <= lt; m++) {
     const int lo = (m - l2 > -l1) ? m - l2 : -l1, hi = (m + l2 < l1) ? m + l2 : l1;
     const int nst = (hi - lo + 2) >> 1;
+    // step k: m1 = lo + 2 k + h, m2 = m - m1: the addresses of a step are those of step 0 plus constants (y runs
+    // backwards: its base is the row of the last unrolled step, so that the constants are not negative)
+    const char *xm = xmine + (lo + h + l1) * 64;
+    const char *ym = ymine + (m - lo - h + l2 - 2 * (kStepsM - 1)) * 64;
+    const char *cm = cmine + at * (2 * kColsF * 4);
     static_for<kStepsM>([&](auto kc) __attribute__((always_inline)) {
       constexpr int k = decltype(kc)::value;
       if (k < nst) {  // uniform
-        // the lane's m1 of this step (the second of an odd count is clamped: its coefficient is zero) and its m2
-        int m1 = lo + 2 * k + h;
-        m1 = m1 > l1 ? l1 : m1;
-        int m2 = m - m1;
-        m2 = m2 < -l2 ? -l2 : (m2 > l2 ? l2 : m2);
-        const float2 xv = xmine[(m1 + l1) * 8];
-        const float4 yv = ymine[(m2 + l2) * 4];
-        const float cl = cmine[(at + k) * (2 * kColsF)];
-        const float c = has_col ? cl : 0.f;
+        const float2 xv = *reinterpret_cast<const float2 *>(xm + k * 128);
+        const float4 yv = *reinterpret_cast<const float4 *>(ym + (kStepsM - 1 - k) * 128);
+        const float c = *reinterpret_cast<const float *>(cm + k * (2 * kColsF * 4));
         const float p0 = fmaf(-xv.y, yv.y, xv.x * yv.x), p1 = fmaf(xv.y, yv.x, xv.x * yv.y);
         const float p2 = fmaf(-xv.y, yv.w, xv.x * yv.z), p3 = fmaf(xv.y, yv.z, xv.x * yv.w);
         if constexpr (k == 0) {  // the first step of an m starts from zero (a constant operand, no registers to clear)
@@ -368,18 +374,18 @@ __global__ void __launch_bounds__(64 * kCellsF) onepair_mfma_fwd_kernel(const On
         }
       }
     });
-    // register v of the four tiles: floats 4 i .. 4 i + 3 of row m of part lrow[v]
+    // register v of the four tiles: floats 4 i .. 4 i + 3 of row m of its part
     const int mabs = m < 0 ? -m : m;
 #pragma unroll
     for (int v = 0; v < 16; v++) {
-      if (lrow[v] >= mabs) {
+      if (((there >> v) & 1u) && lbase + (8 * (v / 4) + v % 4) >= mabs) {
         GlobalOut4 p = (GlobalOut4)cur[v];
         v4f o;
         o.x = D[0][v], o.y = D[1][v], o.z = D[2][v], o.w = D[3][v];
         if (accumulate) o += *p;
         *p = o;
       }
-      cur[v] += rowb[v];
+      cur[v] += rowb;
     }
     at += nst;
   }
@@ -552,6 +558,9 @@ int onepair_mfma_vec_fwd(const VecPlan &plan, const std::vector<const gelib_part
     present[dl] = 1;
     // a lane stores 16 bytes at a time: block offset, row and cell strides even, base aligned
     if (((t.offs) & 1) || (fr[t.ri].sm & 1) || (fr[t.ri].sb & 1) || ((uintptr_t)fr[t.ri].ptr & 15)) return GELIB_HIP_OK;
+    // one row length for every part (true whenever the parts hold just this pair's block)
+    if (a.rowb == 0) a.rowb = (long long)fr[t.ri].sm * 8;
+    if (a.rowb != (long long)fr[t.ri].sm * 8) return GELIB_HIP_OK;
   }
   const long long ncells = plan.E[0] * plan.E[1] * plan.E[2];
   if (ncells > 0x7fffffffLL) return GELIB_HIP_OK;
@@ -568,9 +577,21 @@ int onepair_mfma_vec_fwd(const VecPlan &plan, const std::vector<const gelib_part
   a.lt = lt;
   a.nl = nl;
   a.accumulate = accumulate ? 1 : 0;
-  // LDS of a block: the table and four cells' operands; beyond what a block may ask for, the any-l kernels take the pair
-  const size_t lds = (size_t)t.nsteps_fwd * 2 * kColsF * 4 + (size_t)kCellsF * (2 * l1 + 1 + 2 * l2 + 1) * 64;
-  if (lds > 64 * 1024) return GELIB_HIP_OK;
+  // LDS of a block: the table and eight cells' operands (with their rows of zeros); two blocks per compute unit fit
+  // up to 80 KB each, beyond that the any-l kernels take the pair
+  const size_t lds = (size_t)t.nsteps_fwd * 2 * kColsF * 4 + (size_t)kCellsF * (2 * l1 + 1 + 2 * l2 + 1 + 3) * 64;
+  if (lds > 80 * 1024) return GELIB_HIP_OK;
+  {
+    static std::mutex attr_mutex;
+    static std::map<int, size_t> attr_set;  // device -> largest size asked for so far
+    int dev = 0;
+    GELIB_HIP_TRY(hipGetDevice(&dev));
+    std::lock_guard<std::mutex> lock(attr_mutex);
+    if (attr_set[dev] < lds) {
+      GELIB_HIP_TRY(hipFuncSetAttribute((const void *)onepair_mfma_fwd_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)(80 * 1024)));
+      attr_set[dev] = 80 * 1024;
+    }
+  }
   hipLaunchKernelGGL(onepair_mfma_fwd_kernel, dim3((unsigned)((ncells + kCellsF - 1) / kCellsF)), dim3(64 * kCellsF), lds, s, a);
   GELIB_HIP_TRY(hipGetLastError());
   *used = 1;

@@ -788,7 +788,9 @@ uint64_t gelib_hip_so3vec_cg_linear_workspace_bytes(int nr, const gelib_part_des
     if (R[l].l != l) return 0;
     t5[l] = tau[l];
   }
-  return (uint64_t)cg_linear_workspace_bytes(t5);
+  long long x_elems = 0;
+  for (auto &v : X) x_elems += (long long)(2 * v.l + 1) * v.n;
+  return (uint64_t)cg_linear_workspace_bytes(t5, x_elems, plan.E[0] * plan.E[1] * plan.E[2]);
 }
 
 int gelib_hip_so3part_spharm(const gelib_part_desc *r, const float *x, const int64_t xdims[5],

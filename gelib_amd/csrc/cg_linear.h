@@ -12,8 +12,9 @@ constexpr int kLinMaxN = 16;     // most channels of an operand part
 constexpr int kLinMaxOut = 16;   // most output channels of a product part
 constexpr int kLinCells = 32;    // cells per block: the rows of one matrix-core tile
 
-// Bytes of workspace for the re-packed matrices of a product with tau[l] channels in part l (l = 0..kLinL).
-size_t cg_linear_workspace_bytes(const long long tau[kLinL + 1]);
+// Bytes of workspace: the re-packed matrices of a product with tau[l] channels in part l (l = 0..kLinL) and a copy of
+// the first operand (x_elems_per_cell complex numbers per cell) transposed per group of kLinCells cells.
+size_t cg_linear_workspace_bytes(const long long tau[kLinL + 1], long long x_elems_per_cell, long long ncells);
 
 // out_l[cell, m, :] (+)= P_l[cell, m, :] W_l with P = CGproduct(x, y) never stored.  w[k] belongs to r[k] (both l-sorted):
 // (tau_l, n_out_l) complex, row-major, device memory.  *used = 0 when the shapes are not ones the kernel takes (nothing

@@ -1,0 +1,10 @@
+// Fused product -> linear forward: the launch for the rows of pass 1 (see cg_linear_impl.h).
+#include "cg_linear_impl.h"
+
+namespace gelib_hip {
+
+int launch_cg_linear_pass1(const LinArgs &a, long long nblocks, hipStream_t s) {
+  return launch_cg_linear_pass_impl<1>(a, nblocks, s);
+}
+
+}  // namespace gelib_hip

@@ -192,7 +192,8 @@ uint64_t gelib_hip_part_mix_workspace_bytes(int kind, int64_t rows, int n_in, in
 int gelib_hip_so3vec_cg_linear_fwd(int nr, const gelib_part_desc *r, int nx, const gelib_part_desc *x, int ny,
                                    const gelib_part_desc *y, const void *const *w, int accumulate, void *workspace,
                                    uint64_t workspace_bytes, void *stream);
-/* Bytes of workspace the call above needs for these parts (256 per product channel plus 4096 per part); 0 when the
+/* Bytes of workspace the call above needs for these parts (256 per product channel plus 4096 per part, and a copy of x
+ * rounded up to groups of 32 cells); 0 when the
  * descriptors are malformed or r does not have exactly the parts l = 0..4. */
 uint64_t gelib_hip_so3vec_cg_linear_workspace_bytes(int nr, const gelib_part_desc *r, int nx, const gelib_part_desc *x,
                                                     int ny, const gelib_part_desc *y);

@@ -108,7 +108,8 @@ def test_workspace_rules(cabi):
     L = cabi.lib()
     ra, xa, ya = cabi._arr(outs), cabi._arr(xs), cabi._arr(ys)
     need = int(L.gelib_hip_so3vec_cg_linear_workspace_bytes(5, ra, 5, xa, 5, ya))
-    assert need == sum((taus[l] + 16) * 256 for l in range(5))
+    # the packed matrices (16 channels of padding per part) and x transposed, rounded up to a group of 32 cells
+    assert need == sum((taus[l] + 16) * 256 for l in range(5)) + 32 * sum((2 * l + 1) * 2 for l in range(5)) * 8
     wp = (ctypes.c_void_p * 5)(*[w.data_ptr() for w in ws])
     buf = torch.empty(need, dtype=torch.uint8, device="cuda")
     st = cabi._stream(outs[0])

@@ -88,7 +88,7 @@ constexpr bool pair_needed(int pass, int l1, int l2) {
 
 template <int L1, int L2, int PASS, int U>
 __device__ __forceinline__ void pair_body(const LinArgs &a, f16v (&acc)[kTiles], const v2f *ys, long long cell,
-                                          int slot, int h, int lane) {
+                                          int slot, int h, int lane, int zero) {
   constexpr int lmin = iabs(L1 - L2), lmax = imin(L1 + L2, kLinL);
   constexpr int R1 = 2 * L1 + 1, R2 = 2 * L2 + 1, NLP = lmax - lmin + 1;
   if constexpr (!pair_needed(PASS, L1, L2)) return;
@@ -98,7 +98,6 @@ __device__ __forceinline__ void pair_body(const LinArgs &a, f16v (&acc)[kTiles],
   // the part itself -- eight bytes per cell, a cell's row apart -- the gathers of the waves of an XCD kept more lines
   // alive than its L2 cache holds and pushed the matrices out of it)
   const GlobalC xp = (GlobalC)(a.xt[L1] + (long long)blockIdx.x * (R1 * X.n) * kLinCells + slot);
-  const CoeffPtr bank = (CoeffPtr)a.bank;
   GlobalF wl[NLP];
   static_for<NLP>([&](auto dc) __attribute__((always_inline)) {
     constexpr int l = lmin + decltype(dc)::value;
@@ -106,7 +105,11 @@ __device__ __forceinline__ void pair_body(const LinArgs &a, f16v (&acc)[kTiles],
   });
 
   // The coefficients of the pair's l of this pass, one register each (the same value in every lane): the scalar
-  // registers cannot hold them all, and scalar loads inside the loop would each have to be waited for.
+  // registers cannot hold them all, and scalar loads inside the loop would each have to be waited for.  They are
+  // fetched with VECTOR loads, all in flight at once: as scalar loads into one register each was loaded, waited for and
+  // copied in turn (up to 97 round trips to the scalar cache per pair).  The lane offset `zero` is 0, but opaque to the
+  // compiler, which would otherwise make scalar loads of them again.
+  const GlobalF bankv = (GlobalF)a.bank + zero;
   float C[NLP][2 * (L1 + L2) + 1][R1];
   static_for<NLP>([&](auto dc) __attribute__((always_inline)) {
     constexpr int l = lmin + decltype(dc)::value;
@@ -116,9 +119,7 @@ __device__ __forceinline__ void pair_body(const LinArgs &a, f16v (&acc)[kTiles],
         static_for<R1>([&](auto kc) __attribute__((always_inline)) {
           constexpr int k = decltype(kc)::value, m2 = m - (k - L1);
           if constexpr (m2 >= -L2 && m2 <= L2) {
-            float c = bank[table_off(L1, L2, l) + k * R2 + (m2 + L2)];
-            asm volatile("" : "+v"(c));
-            C[dc.value][m + L1 + L2][k] = c;
+            C[dc.value][m + L1 + L2][k] = bankv[table_off(L1, L2, l) + k * R2 + (m2 + L2)];
           }
         });
       }
@@ -162,7 +163,9 @@ __device__ __forceinline__ void pair_body(const LinArgs &a, f16v (&acc)[kTiles],
         const int jn = j + sub + 1 < n2 ? j + sub + 1 : 0;
 #pragma unroll
         for (int k = 0; k < R2; k++) yq[nxt][k] = ys[(k * n2 + jn) * kLinCells + slot];
-        __builtin_amdgcn_sched_barrier(0);  // the loads stay ahead of the arithmetic that hides them
+        __builtin_amdgcn_sched_barrier(0);  // the loads stay ahead of the arithmetic that hides them (fences between the
+                                            // rows, or in front of the refill below, cost 5 %: the chains of one row
+                                            // depend on each other, and with one wave per SIMD nothing else fills in)
 
         static_for<2 * (L1 + L2) + 1>([&](auto mc) __attribute__((always_inline)) {
           constexpr int m = decltype(mc)::value - (L1 + L2);
@@ -190,10 +193,8 @@ __device__ __forceinline__ void pair_body(const LinArgs &a, f16v (&acc)[kTiles],
                 acc[tile] = __builtin_amdgcn_mfma_f32_32x32x2f32(P, bq[sub][dc.value], acc[tile], 0, 0, 0);
               }
             });
-            __builtin_amdgcn_sched_barrier(0);  // one row's products at a time: few registers
           }
         });
-        __builtin_amdgcn_sched_barrier(0);
         // refill the slot (the B operands past the block's last channel are the next block's or padding)
         static_for<NLP>([&](auto dc) __attribute__((always_inline)) {
           if constexpr (l_in_pass(PASS, lmin + decltype(dc)::value))
@@ -212,6 +213,8 @@ template <int PASS>
 __global__ void __launch_bounds__(64) cg_linear_fwd_kernel(const LinArgs a) {
   __shared__ v2f ys[(2 * kLinL + 1) * kLinMaxN * kLinCells];
   const int lane = threadIdx.x, slot = lane & 31, h = lane >> 5;
+  int zero;
+  asm volatile("v_mov_b32 %0, 0" : "=v"(zero));
   const long long cell0 = (long long)blockIdx.x * kLinCells;
   long long cell = cell0 + slot;
   if (cell >= a.ncells) cell = a.ncells - 1;  // the last block's spare rows repeat the last cell and are not stored
@@ -237,8 +240,8 @@ __global__ void __launch_bounds__(64) cg_linear_fwd_kernel(const LinArgs a) {
           constexpr int UW = wide_u(PASS, L1, L2);
           // the second operand's channel count must be a multiple of the ring length; any other count takes one
           // channel pair per trip and waits for every load (correct, slow)
-          if ((Y.n & (UW - 1)) == 0) pair_body<L1, L2, PASS, UW>(a, acc, ys, cell, slot, h, lane);
-          else pair_body<L1, L2, PASS, 1>(a, acc, ys, cell, slot, h, lane);
+          if ((Y.n & (UW - 1)) == 0) pair_body<L1, L2, PASS, UW>(a, acc, ys, cell, slot, h, lane, zero);
+          else pair_body<L1, L2, PASS, 1>(a, acc, ys, cell, slot, h, lane, zero);
         }
       });
     }

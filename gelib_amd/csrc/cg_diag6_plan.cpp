@@ -1,5 +1,6 @@
 // Host side of the lane-per-channel Diag kernels: which products they take, the coefficient table with its fixed
 // layout, the per-type offset table (both cached on the device), and the argument block.
+#include <algorithm>
 #include <cstring>
 #include <map>
 #include <mutex>
@@ -82,17 +83,32 @@ int make_args(const VecPlan &plan, const std::vector<const gelib_part_desc *> &r
   for (size_t i = 0; i < fxg.size(); i++) a->xg[lx[i].first] = fxg[i];
   for (size_t i = 0; i < fyg.size(); i++) a->yg[ly[i].first] = fyg[i];
   {
-    // deal the parts of y to the four waves of a backward block, largest first, each to the wave with the fewest rows
-    // so far: the waves then finish every l1 at about the same time
-    int rows[4] = {0, 0, 0, 0};
-    for (int l2 = kL6; l2 >= 0; l2--) {
-      a->owner[l2] = 0;
-      if (!a->y[l2].ptr) continue;
+    // Deal the parts of y to the four waves of a backward block, heaviest first, each to the wave with the least work so
+    // far, so that the waves finish every l1 at about the same time.  Work of a pair: two multiply-adds per term of each
+    // of its triples (the contraction over l) and eight per (m1, m2).
+    long long cost[kNP] = {0, 0, 0, 0, 0, 0, 0};
+    bool pair_seen[kNP][kNP] = {};
+    for (auto &t : plan.triples) {
+      long long terms = 0;
+      for (int m = -t.l; m <= t.l; m++) terms += std::min(t.l1, m + t.l2) - std::max(-t.l1, m - t.l2) + 1;
+      cost[t.l2] += 2 * terms;
+      if (!pair_seen[t.l1][t.l2]) {
+        pair_seen[t.l1][t.l2] = true;
+        cost[t.l2] += 8LL * (2 * t.l1 + 1) * (2 * t.l2 + 1);
+      }
+    }
+    long long load[4] = {0, 0, 0, 0};
+    bool dealt[kNP] = {};
+    for (int n = 0; n < kNP; n++) {
+      int best = -1;
+      for (int l2 = 0; l2 < kNP; l2++)
+        if (!dealt[l2] && (best < 0 || cost[l2] > cost[best])) best = l2;
+      dealt[best] = true;
       int w = 0;
       for (int k = 1; k < 4; k++)
-        if (rows[k] < rows[w]) w = k;
-      a->owner[l2] = w;
-      rows[w] += 2 * l2 + 1;
+        if (load[k] < load[w]) w = k;
+      a->owner[best] = w;
+      load[w] += cost[best];
     }
   }
   std::vector<int> offs((size_t)kNP * kNP * kNR, -1);

@@ -39,6 +39,8 @@ struct DevicePlan {
   int lmax_out = 0;
   int fwd_len = 0;           // floats of the forward coefficient stream (the first region of the bank)
   bool stripes_ok = false;   // the striped backward kernels apply
+  bool stripes_skip_parts = false;  // ... but only when accumulating: some gradient part gets nothing from these triples
+                                    // and would stay unwritten
   int stripe_cap = 0;        // register rows they need (16 or 32)
   std::vector<int> stripes;  // host copy of the table
   int npairs = 0;            // (x part, y part) pairs; their table follows the stripe tables
@@ -182,9 +184,10 @@ int get_plan(bool diag, const std::vector<VecTriple> &triples, const std::vector
           n_other = no;
         }
         table[3 * k + 1] = filled - table[3 * k];
-        // a part that no triple feeds has a zero gradient; a stripe without units would leave it unwritten, so such
-        // types go to the kernels that write every part from their images
-        if (table[3 * k + 1] == 0) ok = false;
+        // a part that no triple feeds has a zero gradient; a stripe without units leaves it as it is, which is right
+        // when the call accumulates (the second half of a product split between two kernel families) and wrong when it
+        // overwrites
+        if (table[3 * k + 1] == 0) plan.stripes_skip_parts = true;
         // lane slots: channel counts rounded up to powers of two
         const int lgu = diag ? ilog2(std::max(1, n_own)) : ilog2(std::max(1, n_own)) + ilog2(std::max(1, n_other));
         if (lgu > 20) ok = false;
@@ -351,7 +354,8 @@ int run_bwd(bool diag, const std::vector<VecTriple> &triples, const std::vector<
   // sums (own l above 7) they run at low occupancy, still 2.7 times faster than the atomic single-pass form on vectors
   // of several parts around l = 10 (6.7 against 18.4 ms; the per-pair route of the dispatcher takes those first).
   const bool stripes_wanted = g_bwd_stripes != 0;
-  if (stripes_wanted && plan->stripes_ok && 8LL * std::max(plan->xsize, plan->ysize) + 64 <= kLdsLimit) {
+  if (stripes_wanted && plan->stripes_ok && (accumulate || !plan->stripes_skip_parts) &&
+      8LL * std::max(plan->xsize, plan->ysize) + 64 <= kLdsLimit) {
     // one launch per wanted gradient; LDS holds the other operand only
     StagedArgs a;
     fill_args(a, *plan, f, xs, ys, ncells, offs_add, accumulate);

@@ -1,0 +1,75 @@
+"""The entry points inside a captured HIP graph: product forward and backward, channel mixing (workspace from the
+caller, and the variant that allocates nothing) and the fused product -> linear call are recorded once (after an eager
+call that uploads the tables of the type signature) and replayed several times on new input values, with eager work and
+synchronisations between the replays; every replay must give the bits of the eager calls on the same values."""
+import pytest
+
+from tests import gpu_util as U
+
+pytestmark = pytest.mark.gpu
+
+torch = pytest.importorskip("torch")
+
+
+@pytest.fixture(scope="module")
+def cabi():
+    assert torch.cuda.is_available(), "GPU tests need a GPU"
+    from gelib_amd import cabi as c
+    c.lib()
+    return c
+
+
+def bits(ts):
+    return [t.view(torch.float32).clone() for t in ts]
+
+
+def test_replays_match_eager_calls(cabi):
+    import ctypes
+    B, n, n_out = 96, 16, 16
+    tau = {l: n for l in range(5)}
+    taus = cabi.so3type_product(tau, tau, 4)
+    xs = [U.dev(U.seeded(10 + l, B, 2 * l + 1, n)) for l in range(5)]
+    ys = [U.dev(U.seeded(20 + l, B, 2 * l + 1, n)) for l in range(5)]
+    ws = [U.dev(U.seeded(30 + l, taus[l], n_out, scale=0.05)) for l in range(5)]
+    rs = [torch.empty(B, 2 * l + 1, taus[l], dtype=torch.complex64, device="cuda") for l in range(5)]
+    xg, yg = [torch.empty_like(t) for t in xs], [torch.empty_like(t) for t in ys]
+    mixed = torch.empty(B, 9, n_out, dtype=torch.complex64, device="cuda")
+    mixed_static = torch.empty_like(mixed)
+    fused = [torch.empty(B, 2 * l + 1, n_out, dtype=torch.complex64, device="cuda") for l in range(5)]
+    L = cabi.lib()
+
+    def static_mix(stream):
+        rows = B * 9
+        cabi.check(L.gelib_hip_part_mix_channels_static(mixed_static.data_ptr(), rs[4].data_ptr(), ws[4].data_ptr(), rows,
+                                                        taus[4], n_out, n_out, taus[4], 0, stream))
+
+    def work():
+        cabi.so3vec_fwd(rs, xs, ys, accumulate=False)
+        cabi.so3vec_bwd(xg, yg, rs, xs, ys, accumulate=False)      # the product itself as the incoming gradient
+        cabi.part_mix_channels(mixed, rs[4], ws[4])
+        static_mix(ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+        assert cabi.so3vec_cg_linear_fwd(fused, xs, ys, ws, accumulate=False)
+
+    outputs = lambda: bits(rs + xg + yg + [mixed, mixed_static] + fused)
+    work()                      # eager: uploads the tables, validates the allocations
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        work()
+    torch.cuda.synchronize()
+    for k in range(3):
+        for l in range(5):      # new values in the buffers the graph reads
+            xs[l].copy_(U.dev(U.seeded(100 + 10 * k + l, B, 2 * l + 1, n)))
+            ys[l].copy_(U.dev(U.seeded(200 + 10 * k + l, B, 2 * l + 1, n)))
+        work()
+        torch.cuda.synchronize()
+        want = outputs()
+        for t in rs + xg + yg + [mixed, mixed_static] + fused:
+            t.fill_(7.0)
+        junk = torch.randn(1 << 20, device="cuda").sum()      # unrelated eager work between the replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        got = outputs()
+        assert all(torch.equal(a, b) for a, b in zip(got, want)), "replay %d" % k
+        assert bool(torch.isfinite(junk))

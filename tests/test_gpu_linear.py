@@ -81,6 +81,29 @@ def test_fused_forward_matches_product_then_matmul(cabi, case):
     assert all(torch.equal(a.view(torch.float32), b.view(torch.float32)) for a, b in zip(outs, outs3))
 
 
+def test_grid_dimensions_collapse_into_cells(cabi):
+    """Parts with grid dimensions (batch, grid0, grid1, 2l+1, n), contiguous: 3 x 4 x 5 = 60 cells."""
+    lead, n, n_out = (3, 4, 5), 4, 6
+    B = 60
+    xs = [U.seeded(700 + l, B, 2 * l + 1, n) for l in range(5)]
+    ys = [U.seeded(750 + l, B, 2 * l + 1, n) for l in range(5)]
+    O = U.VecOracle(xs, ys, 4, False)
+    taus = [p.shape[2] for p in O.r32]
+    ws = weights(800, taus, [n_out] * 5)
+    r32, r64, S = oracle_linear(O, ws)
+    dxs = [U.dev(a).reshape(*lead, 2 * l + 1, n) for l, a in enumerate(xs)]
+    dys = [U.dev(a).reshape(*lead, 2 * l + 1, n) for l, a in enumerate(ys)]
+    dws = [U.dev(a) for a in ws]
+    outs = [torch.full((*lead, 2 * l + 1, n_out), 7.0 + 1j, dtype=torch.complex64, device="cuda") for l in range(5)]
+    assert cabi.so3vec_cg_linear_fwd(outs, dxs, dys, dws, accumulate=False)
+    torch.cuda.synchronize()
+    for l in range(5):
+        U.assert_parity(U.host(outs[l]).reshape(B, 2 * l + 1, n_out), r32[l], r64[l], S[l], "grid l=%d" % l)
+    # an operand that broadcasts over the grid is not a case of the fused kernel
+    bx = [t[:, :1, :1].expand(*lead, -1, -1) for t in dxs]
+    assert cabi.so3vec_cg_linear_fwd(outs, bx, dys, dws, accumulate=False) is False
+
+
 def test_shapes_the_fused_kernel_does_not_take(cabi):
     B = 4
     xs = [U.dev(U.seeded(1 + l, B, 2 * l + 1, 4)) for l in range(3)]

@@ -12,6 +12,7 @@ int launch_unrolled_bwd_cg4_pad(const BwdArgs &a, int nblocks, size_t lds_bytes,
 int launch_unrolled_bwd_cg8_pad(const BwdArgs &a, int nblocks, size_t lds_bytes, hipStream_t s);
 int launch_unrolled_bwd_diag4_pad(const BwdArgs &a, int nblocks, size_t lds_bytes, hipStream_t s);
 int launch_unrolled_bwd_diag8_pad(const BwdArgs &a, int nblocks, size_t lds_bytes, hipStream_t s);
+int launch_unrolled_bwd_cg6_l6(const BwdArgs &a, int nblocks, size_t lds_bytes, hipStream_t s);
 
 size_t unrolled_bwd_lds_bytes(int bank_len, int xsize, int ysize, int cells_per_block) {
   const int waves = kBlock / kWave;
@@ -19,9 +20,18 @@ size_t unrolled_bwd_lds_bytes(int bank_len, int xsize, int ysize, int cells_per_
   return sizeof(float2) * (size_t)(1 + waves) * cells_per_block * ((size_t)xsize + ysize);
 }
 
+// Operands up to l = 4: every product (l up to 8), Diag or not, any channel counts.  Operands up to l = 6: CGproduct
+// capped at l = 6 with power-of-two channel counts (one instantiation, five minutes of compile time; a kernel for the
+// uncapped product, l up to 12, is not built).
+bool unrolled_bwd_takes(bool diag, bool padded, int lcap, int lop) {
+  if (lop <= kLT) return lcap <= 2 * kLT;
+  return lop <= kLTMax && !diag && !padded && lcap <= kLTMax;
+}
+
 // lcap: largest l present in the gradient; code for l above 4 is left out when the product is capped there
-int launch_unrolled_bwd(const BwdArgs &a, bool diag, int lcap, int nblocks, size_t lds_bytes, hipStream_t s) {
+int launch_unrolled_bwd(const BwdArgs &a, bool diag, int lcap, int lop, int nblocks, size_t lds_bytes, hipStream_t s) {
   if (nblocks <= 0) return GELIB_HIP_OK;
+  if (lop > kLT) return launch_unrolled_bwd_cg6_l6(a, nblocks, lds_bytes, s);
   if (a.padded) {
     if (diag) return lcap <= kLT ? launch_unrolled_bwd_diag4_pad(a, nblocks, lds_bytes, s)
                                  : launch_unrolled_bwd_diag8_pad(a, nblocks, lds_bytes, s);

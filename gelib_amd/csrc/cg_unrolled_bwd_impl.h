@@ -1,4 +1,5 @@
-// Backward CG / DiagCG product for l1, l2 <= kLT: both gradients from one pass over g, all triples in one launch.
+// Backward CG / DiagCG product for l1, l2 <= kLT (one instantiation: <= kLTMax): both gradients from one pass over g,
+// all triples in one launch.
 //
 // Work split.  A block owns a few whole cells (one cell when a cell has >= 256 channel slots).  The operands x, y
 // of those cells are staged once in LDS next to the coefficient bank.  For every (l1,l2) pair the flattened
@@ -136,7 +137,7 @@ __device__ __forceinline__ void pair_bwd(const GParts<LCAP> &gp, PairPtr pr, Coe
   // them (the wave then waits once per pair, and 16 waves per compute unit keep enough bytes in flight to cover
   // the memory latency), otherwise as many m as fit the budget.  The kernels for l up to 8 hold more sums and are
   // near the register limit of three waves per SIMD already, so their budget is smaller.
-  constexpr int kRowBudget = LCAP <= 4 ? 32 : 14;
+  constexpr int kRowBudget = LCAP <= 4 ? 32 : ((L1 > kLT || L2 > kLT) ? 8 : 14);  // pairs with l = 5, 6 hold 26 sums more
   constexpr int ROWS = (LTOP + 1) * (LTOP + 1) - LMIN * LMIN;  // sum of 2l+1 over the l of the pair
   constexpr int PF = ROWS <= kRowBudget ? 2 * LTOP + 1 : (kRowBudget / NLP > 1 ? kRowBudget / NLP : 1);
   float2 gq[PF][NLP];
@@ -282,7 +283,8 @@ __device__ __forceinline__ void copy_image(const FastPart (&parts)[kFastIn], con
   });
 }
 
-template <int LCAP, bool DIAG, bool WX, bool WY, bool PAD>
+// LT: largest operand l of the pairs the kernel has code for.
+template <int LCAP, bool DIAG, bool WX, bool WY, bool PAD, int LT>
 __global__ void __launch_bounds__(kBlock) unrolled_bwd_kernel(const BwdArgs a) {
   constexpr int KR = 2 * LCAP + 1;
   extern __shared__ float lds[];
@@ -328,13 +330,15 @@ __global__ void __launch_bounds__(kBlock) unrolled_bwd_kernel(const BwdArgs a) {
     dealt += nruns;
     for (int run = first; run < nruns; run += kWaves) {
       const LanePos q = lane_pos(run, lane, p->log2_u, ncell);
-      switch (p->l1 * (kLT + 1) + p->l2) {
+      switch (p->l1 * (kLTMax + 1) + p->l2) {
 #define GELIB_CASE(A, B)                                                                                      \
-  case A * (kLT + 1) + B:                                                                                     \
-    pair_bwd<A, B, LCAP, DIAG, WX, WY, PAD>(gp, p, C, Zc, zrows, xs, ys, xacc, yacc, xsize, ysize, cell0, offs_add, q); \
+  case A * (kLTMax + 1) + B:                                                                                  \
+    if constexpr (A <= LT && B <= LT)                                                                         \
+      pair_bwd<A, B, LCAP, DIAG, WX, WY, PAD>(gp, p, C, Zc, zrows, xs, ys, xacc, yacc, xsize, ysize, cell0, offs_add, q); \
     break;
-#define GELIB_ROW(A) GELIB_CASE(A, 0) GELIB_CASE(A, 1) GELIB_CASE(A, 2) GELIB_CASE(A, 3) GELIB_CASE(A, 4)
-        GELIB_ROW(0) GELIB_ROW(1) GELIB_ROW(2) GELIB_ROW(3) GELIB_ROW(4)
+#define GELIB_ROW(A) \
+  GELIB_CASE(A, 0) GELIB_CASE(A, 1) GELIB_CASE(A, 2) GELIB_CASE(A, 3) GELIB_CASE(A, 4) GELIB_CASE(A, 5) GELIB_CASE(A, 6)
+        GELIB_ROW(0) GELIB_ROW(1) GELIB_ROW(2) GELIB_ROW(3) GELIB_ROW(4) GELIB_ROW(5) GELIB_ROW(6)
 #undef GELIB_ROW
 #undef GELIB_CASE
         default: break;
@@ -347,9 +351,9 @@ __global__ void __launch_bounds__(kBlock) unrolled_bwd_kernel(const BwdArgs a) {
   if (WY) copy_image<false>(a.yg, a.yrows, a.ny, yacc_all, ysize, cell0, ncell, kWaves, cpb * ysize, a.accumulate != 0);
 }
 
-template <int LCAP, bool DIAG, bool WX, bool WY, bool PAD>
+template <int LCAP, bool DIAG, bool WX, bool WY, bool PAD, int LT>
 int launch_variant(const BwdArgs &a, int nblocks, size_t lds, hipStream_t s) {
-  auto kern = unrolled_bwd_kernel<LCAP, DIAG, WX, WY, PAD>;
+  auto kern = unrolled_bwd_kernel<LCAP, DIAG, WX, WY, PAD, LT>;
   static bool attr_set = false;  // benign race: setting the attribute twice is harmless
   if (!attr_set) {
     GELIB_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -362,13 +366,13 @@ int launch_variant(const BwdArgs &a, int nblocks, size_t lds, hipStream_t s) {
 }
 
 // want_x / want_y select which gradients are computed
-template <int LCAP, bool DIAG, bool PAD>
+template <int LCAP, bool DIAG, bool PAD, int LT = kLT>
 int launch_bwd_variants(const BwdArgs &a, int nblocks, size_t lds_bytes, hipStream_t s) {
-  static_assert(kLT == 4, "the case table above lists l1, l2 = 0..4");
+  static_assert(kLTMax == 6 && LT <= kLTMax, "the case table above lists l1, l2 = 0..6");
   const bool wx = a.want_x != 0, wy = a.want_y != 0;
-  if (wx && wy) return launch_variant<LCAP, DIAG, true, true, PAD>(a, nblocks, lds_bytes, s);
-  if (wx) return launch_variant<LCAP, DIAG, true, false, PAD>(a, nblocks, lds_bytes, s);
-  return launch_variant<LCAP, DIAG, false, true, PAD>(a, nblocks, lds_bytes, s);
+  if (wx && wy) return launch_variant<LCAP, DIAG, true, true, PAD, LT>(a, nblocks, lds_bytes, s);
+  if (wx) return launch_variant<LCAP, DIAG, true, false, PAD, LT>(a, nblocks, lds_bytes, s);
+  return launch_variant<LCAP, DIAG, false, true, PAD, LT>(a, nblocks, lds_bytes, s);
 }
 
 }  // namespace

@@ -8,8 +8,8 @@
 
 namespace gelib_hip {
 
-constexpr int kFastIn = kLT + 1;       // operand parts l = 0..kLT
-constexpr int kFastOut = 2 * kLT + 1;  // product parts l = 0..2*kLT
+constexpr int kFastIn = kLTMax + 1;       // operand parts l = 0..kLTMax
+constexpr int kFastOut = 2 * kLTMax + 1;  // product parts l = 0..2*kLTMax
 constexpr int kBlock = 256;
 
 struct FwdArgs {
@@ -90,7 +90,9 @@ __device__ __forceinline__ int pick_int(const int (&arr)[N], int i) {
 
 // ti: channels of the first operand handled per thread (1, 2 or 4); must divide every n1.
 int launch_unrolled_fwd(const FwdArgs &a, bool diag, int ti, int lcap, int nblocks, size_t lds_bytes, hipStream_t s);
-// lcap: largest l present in the gradient
-int launch_unrolled_bwd(const BwdArgs &a, bool diag, int lcap, int nblocks, size_t lds_bytes, hipStream_t s);
+// lcap: largest l present in the gradient; lop: largest l of an operand (above kLT: the kernel for l up to kLTMax, which
+// exists for CGproduct with power-of-two channel counts and lcap <= kLTMax only -- unrolled_bwd_takes says so)
+bool unrolled_bwd_takes(bool diag, bool padded, int lcap, int lop);
+int launch_unrolled_bwd(const BwdArgs &a, bool diag, int lcap, int lop, int nblocks, size_t lds_bytes, hipStream_t s);
 
 }  // namespace gelib_hip

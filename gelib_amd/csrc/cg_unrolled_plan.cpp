@@ -17,6 +17,7 @@ int g_fwd_lds_bytes = 16 * 1024;     // LDS one forward block may use for its st
 int g_fwd_cell_tile = 64;             // cells per tile of the forward launch (0 = all cells in one tile)
 int g_fwd_ti = 0;                    // 0 = widest tile that divides every n1, else force 1 / 2 / 4
 int g_bwd_enable = 1;
+int g_bwd_l6_enable = 1;  // the backward kernel for operands up to l = 6
 int g_fwd_enable = 1;
 
 struct DevicePlan {
@@ -165,7 +166,7 @@ int get_plan(bool diag, const std::vector<VecTriple> &triples, const std::vector
   }
   if (bank.size() % 2) bank.push_back(0.f);
   plan.zero_off = (int)bank.size();
-  bank.resize(bank.size() + (2 * kLT + 1) * (2 * kLT + 1) + 1, 0.f);
+  bank.resize(bank.size() + (2 * kLTMax + 1) * (2 * kLTMax + 1) + 1, 0.f);
   plan.bank_len = (int)bank.size();
   const size_t pair_bytes = plan.pairs.size() * sizeof(PairRec);
   const size_t bank_bytes = bank.size() * sizeof(float);
@@ -264,6 +265,14 @@ int run_bwd(bool diag, const std::vector<VecTriple> &triples, const std::vector<
             const std::vector<std::pair<int, int>> &ys, const std::vector<int> &rls, const FastLists &f,
             long long ncells, int offs_add, bool accumulate, bool want_x, bool want_y, hipStream_t s, int *used) {
   *used = 0;
+  int lcap = 0, lop = 0;
+  bool padded = false;
+  for (auto &t : triples) {
+    lcap = std::max(lcap, t.l);
+    lop = std::max(lop, std::max(t.l1, t.l2));
+    padded = padded || !is_pow2(xs[t.xi].second) || (!diag && !is_pow2(ys[t.yi].second));
+  }
+  if (!unrolled_bwd_takes(diag, padded, lcap, lop) || (lop > kLT && !g_bwd_l6_enable)) return GELIB_HIP_OK;
   // lane slots are the channel counts rounded up to powers of two; the reduced operand must fit a wave
   int u_min = 1 << 30;
   for (auto &t : triples) {
@@ -310,9 +319,7 @@ int run_bwd(bool diag, const std::vector<VecTriple> &triples, const std::vector<
   a.cells_per_block = cpb;
   const long long nblocks = (ncells + cpb - 1) / cpb;
   if (nblocks > 0x7fffffffLL) return GELIB_HIP_ERR_ARG;
-  int lcap = 0;
-  for (auto &t : triples) lcap = std::max(lcap, t.l);
-  rc = launch_unrolled_bwd(a, diag, lcap, (int)nblocks, lds, s);
+  rc = launch_unrolled_bwd(a, diag, lcap, lop, (int)nblocks, lds, s);
   if (rc) return rc;
   *used = 1;
   return GELIB_HIP_OK;
@@ -388,9 +395,11 @@ int unrolled_vec_bwd(const VecPlan &plan, const std::vector<const gelib_part_des
   if (!g_bwd_enable) return GELIB_HIP_OK;
   if (x.size() > (size_t)kFastIn || y.size() > (size_t)kFastIn || g.size() > (size_t)kFastOut) return GELIB_HIP_OK;
   for (auto *d : x)
-    if ((d->dims[3] - 1) / 2 > kLT) return GELIB_HIP_OK;
+    if ((d->dims[3] - 1) / 2 > kLTMax) return GELIB_HIP_OK;
   for (auto *d : y)
-    if ((d->dims[3] - 1) / 2 > kLT) return GELIB_HIP_OK;
+    if ((d->dims[3] - 1) / 2 > kLTMax) return GELIB_HIP_OK;
+  for (auto *d : g)
+    if ((d->dims[3] - 1) / 2 > 2 * kLTMax) return GELIB_HIP_OK;
   FastLists f;
   std::vector<std::pair<int, int>> xs, ys, rs;
   if (!lists_to_fast(x, plan.E, false, &f.x, &xs) || !lists_to_fast(y, plan.E, false, &f.y, &ys) ||
@@ -426,6 +435,10 @@ int unrolled_set_option(const char *name, int value) {
   }
   if (!std::strcmp(name, "unrolled_fwd")) {
     g_fwd_enable = value;
+    return GELIB_HIP_OK;
+  }
+  if (!std::strcmp(name, "unrolled_bwd_l6")) {
+    g_bwd_l6_enable = value;
     return GELIB_HIP_OK;
   }
   if (!std::strcmp(name, "unrolled_bwd")) {

@@ -31,6 +31,7 @@ def cabi(request):
     c.set_option("onepair", 0) # and the single-pair backward kernels others
     c.set_option("onepair_mfma", 0)
     c.set_option("onepair_mfma_fwd", 0)
+    c.set_option("unrolled_bwd_l6", 0)   # the unrolled backward kernel for operands up to l = 6 would take some too
     c.set_option("pairwise_bwd", 0)
     c.set_option("staged_bwd_stripes", 1 if request.param == "striped" else 0)
     c.set_option("staged_bwd_atomic", 1)   # the other two forms (and what the striped one leaves) add with LDS float atomics
@@ -40,6 +41,7 @@ def cabi(request):
     c.set_option("onepair", 1)
     c.set_option("onepair_mfma", 1)
     c.set_option("onepair_mfma_fwd", 1)
+    c.set_option("unrolled_bwd_l6", 1)
     c.set_option("pairwise_bwd", 1)
     c.set_option("staged_bwd_threads", 0)
     c.set_option("staged_bwd_stripes", 1)

@@ -27,6 +27,8 @@ CASES = [
     (3, {l: 4 for l in range(3)}, {l: 4 for l in range(3)}, 2),
     (2, {10: 8}, {10: 8}, -1),                                           # configuration 5 type
     (5, {l: 8 for l in range(7)}, {l: 8 for l in range(7)}, 6),
+    (6, {0: 2, 3: 4, 5: 8, 6: 2}, {1: 4, 4: 2, 6: 8}, 6),                # operands up to l = 6, mixed channel counts
+    (3, {5: 16}, {6: 4}, 5),                                             # one pair with l1, l2 above 4, capped
 ]
 
 

@@ -52,6 +52,7 @@ struct PairRec {
   int log2_u;        // log2 of the lane slots per cell: n1p*n2p (Diag: n1p) with n1p, n2p the channel counts rounded up
                      // to powers of two; -1 when that exceeds 2^20
   int lg_n2p;        // log2 of n2p
+  int rec_off;       // offset (floats) in the bank of the pair's step records (kernel for operands up to l = kLTMax), or -1
 };
 
 // Helpers shared by the kernel families that need contiguous channels and one cell index (cg_unrolled_plan.cpp).

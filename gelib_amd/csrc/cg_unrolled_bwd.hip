@@ -28,6 +28,12 @@ bool unrolled_bwd_takes(bool diag, bool padded, int lcap, int lop) {
   return lop <= kLTMax && !diag && !padded && lcap <= kLTMax;
 }
 
+int unrolled_bwd_cap(int lcap, int lop) {
+  if (lop > kLTMax || lcap > 2 * kLTMax) return -1;
+  if (lop > kLT) return lcap <= kLTMax ? kLTMax : -1;
+  return lcap <= kLT ? kLT : 2 * kLT;
+}
+
 // lcap: largest l present in the gradient; code for l above 4 is left out when the product is capped there
 int launch_unrolled_bwd(const BwdArgs &a, bool diag, int lcap, int lop, int nblocks, size_t lds_bytes, hipStream_t s) {
   if (nblocks <= 0) return GELIB_HIP_OK;

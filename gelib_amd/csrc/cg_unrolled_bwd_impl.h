@@ -28,6 +28,21 @@ namespace {
 constexpr int cabs_(int a) { return a < 0 ? -a : a; }
 constexpr int cmin_(int a, int b) { return a < b ? a : b; }
 constexpr int kWaves = kBlock / kWave;
+constexpr int pow2ceil_(int v) {
+  int p = 1;
+  while (p < v) p *= 2;
+  return p;
+}
+// (m1,m2) steps of one row number m = m1 + m2, and steps of all row numbers below m (rows run from -ltop up)
+constexpr int steps_of(int l1, int l2, int m) {
+  const int lo = -l1 > m - l2 ? -l1 : m - l2, hi = l1 < m + l2 ? l1 : m + l2;
+  return hi >= lo ? hi - lo + 1 : 0;
+}
+constexpr int steps_below(int l1, int l2, int ltop, int m) {
+  int s = 0;
+  for (int k = -ltop; k < m; k++) s += steps_of(l1, l2, k);
+  return s;
+}
 
 // All g, x, y pointers that the arithmetic loops dereference are typed as global memory, so the loads are
 // global_load (vmcnt only) rather than flat_load (which also ties up the LDS counter).
@@ -72,7 +87,17 @@ __device__ __forceinline__ LanePos lane_pos(int run, int lane, int log2_u, int n
 // reads a row of zeros and a table of zeros (zrows, Zc) instead, so the code has no branches.
 // PAD: channel counts are not all powers of two.  Lane slots are then n1p x n2p with the counts rounded up; a lane
 // whose (i, j) lies beyond the real channels reads channel 0, has its g forced to zero and never writes.
-template <int L1, int L2, int LCAP, bool DIAG, bool WX, bool WY, bool PAD>
+// REC: the coefficients come from the pair's step records instead of its tables: one record per (m1,m2) step in the
+// order the steps run, holding C_l[m1,m2] of every l of the pair (zero for an absent l), padded to a power of two.
+// Sixteen floats of records are fetched by one scalar load, a group ahead of their use, into one of two register
+// groups.  (Read from the tables, the coefficients of a step lie in up to seven places; the compiler merges the loads
+// of neighbouring steps' entries into long ones issued far ahead of their use and spills their registers, and a wave
+// waits for a load at every step once the tables outgrow the scalar cache.)  Used by the kernel for operands up to
+// l = kLTMax (L=6, 8 channels, 16384 cells: 5.2 -> 4.6 ms, and 3.8 ms with the registers this frees: three waves per
+// SIMD).  The kernels for operands up to l = 4 keep the tables: with records the product capped at l = 4 runs at the
+// same speed and the uncapped one slower (7.8 -> 9.6 ms; its records are 16 floats, one load per step, waited for
+// one step later).
+template <int L1, int L2, int LCAP, bool DIAG, bool WX, bool WY, bool PAD, bool REC>
 __device__ __forceinline__ void pair_bwd(const GParts<LCAP> &gp, PairPtr pr, CoeffPtr Cs, CoeffPtr Zc, GlobalRows zrows,
                                          const float2 *xs, const float2 *ys, float2 *xacc, float2 *yacc, int xsize,
                                          int ysize, long long cell0, int offs_add, const LanePos q) {
@@ -120,6 +145,18 @@ __device__ __forceinline__ void pair_bwd(const GParts<LCAP> &gp, PairPtr pr, Coe
     gsm[dl] = present ? G.sm : 0;
     cl[dl] = present ? Cs + p.cg[dl] : Zc;
   });
+  constexpr int RECW = pow2ceil_(NLP);                 // floats per record
+  constexpr int kGroup = 16;                           // floats per load
+  constexpr int PER = kGroup / RECW;                   // steps per group
+  constexpr int NSTEPS = steps_below(L1, L2, LTOP, LTOP + 1);
+  constexpr int NGROUPS = (NSTEPS * RECW + kGroup - 1) / kGroup;
+  const CoeffPtr recs = Cs - p.cg_base + (REC ? p.rec_off : 0);   // Cs is the bank plus cg_base
+  float cb[2][kGroup];
+  auto load_group = [&](auto gc, float(&dst)[kGroup]) __attribute__((always_inline)) {
+#pragma unroll
+    for (int t = 0; t < kGroup; t++) dst[t] = recs[decltype(gc)::value * kGroup + t];
+  };
+  if constexpr (REC) load_group(std::integral_constant<int, 0>{}, cb[0]);
   // rows of one m at a time, the rows of the next m requested before the arithmetic of this one; the scheduling
   // barrier between steps keeps the compiler from hoisting every load of the pair to the top (twice the registers)
   auto load_m = [&](auto mc, float2(&dst)[NLP]) __attribute__((always_inline)) {
@@ -137,7 +174,7 @@ __device__ __forceinline__ void pair_bwd(const GParts<LCAP> &gp, PairPtr pr, Coe
   // them (the wave then waits once per pair, and 16 waves per compute unit keep enough bytes in flight to cover
   // the memory latency), otherwise as many m as fit the budget.  The kernels for l up to 8 hold more sums and are
   // near the register limit of three waves per SIMD already, so their budget is smaller.
-  constexpr int kRowBudget = LCAP <= 4 ? 32 : ((L1 > kLT || L2 > kLT) ? 8 : 14);  // pairs with l = 5, 6 hold 26 sums more
+  constexpr int kRowBudget = LCAP <= 4 ? 32 : LCAP == kLTMax ? ((L1 > kLT || L2 > kLT) ? 16 : 32) : 14;
   constexpr int ROWS = (LTOP + 1) * (LTOP + 1) - LMIN * LMIN;  // sum of 2l+1 over the l of the pair
   constexpr int PF = ROWS <= kRowBudget ? 2 * LTOP + 1 : (kRowBudget / NLP > 1 ? kRowBudget / NLP : 1);
   float2 gq[PF][NLP];
@@ -161,14 +198,25 @@ __device__ __forceinline__ void pair_bwd(const GParts<LCAP> &gp, PairPtr pr, Coe
       constexpr int m1 = M1LO + decltype(kc)::value;
       constexpr int m2 = m - m1;
       float qr = 0.f, qi = 0.f;
+      constexpr int step = steps_below(L1, L2, LTOP, m) + decltype(kc)::value;
+      constexpr int grp = step / PER, slot = step % PER;
       static_for<NLP>([&](auto dl_c) __attribute__((always_inline)) {
         constexpr int dl = decltype(dl_c)::value;
         if constexpr (LMIN + dl >= MABS) {
-          const float c = cl[dl][(m1 + L1) * (2 * L2 + 1) + (m2 + L2)];
+          float c;
+          if constexpr (REC) c = cb[grp & 1][slot * RECW + dl];
+          else c = cl[dl][(m1 + L1) * (2 * L2 + 1) + (m2 + L2)];
           qr = fmaf(c, gl[dl].x, qr);
           qi = fmaf(c, gl[dl].y, qi);
         }
       });
+      if constexpr (REC && slot == 0 && grp + 1 < NGROUPS) {
+        // the next group is requested only after this one has been waited for: scalar loads return in any order, so
+        // a wait for one of them is a wait for all that are in flight
+        __builtin_amdgcn_sched_barrier(0);
+        load_group(std::integral_constant<int, grp + 1>{}, cb[(grp + 1) & 1]);
+        __builtin_amdgcn_sched_barrier(0);
+      }
       if (WX) {
         const float2 yc = yv[m2 + L2];
         ax[m1 + L1].x = fmaf(qr, yc.x, ax[m1 + L1].x);
@@ -284,8 +332,10 @@ __device__ __forceinline__ void copy_image(const FastPart (&parts)[kFastIn], con
 }
 
 // LT: largest operand l of the pairs the kernel has code for.
+// The kernel for operands above kLT is asked to fit three waves per SIMD (168 registers): left alone it takes 169.
 template <int LCAP, bool DIAG, bool WX, bool WY, bool PAD, int LT>
-__global__ void __launch_bounds__(kBlock) unrolled_bwd_kernel(const BwdArgs a) {
+__global__ void __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(LT > kLT ? 3 : 1)))
+unrolled_bwd_kernel(const BwdArgs a) {
   constexpr int KR = 2 * LCAP + 1;
   extern __shared__ float lds[];
   const int xsize = a.xsize, ysize = a.ysize, cpb = a.cells_per_block;
@@ -334,7 +384,8 @@ __global__ void __launch_bounds__(kBlock) unrolled_bwd_kernel(const BwdArgs a) {
 #define GELIB_CASE(A, B)                                                                                      \
   case A * (kLTMax + 1) + B:                                                                                  \
     if constexpr (A <= LT && B <= LT)                                                                         \
-      pair_bwd<A, B, LCAP, DIAG, WX, WY, PAD>(gp, p, C, Zc, zrows, xs, ys, xacc, yacc, xsize, ysize, cell0, offs_add, q); \
+      pair_bwd<A, B, LCAP, DIAG, WX, WY, PAD, (LT > kLT)>(gp, p, C, Zc, zrows, xs, ys, xacc, yacc, xsize, ysize, cell0, \
+                                                            offs_add, q);                                      \
     break;
 #define GELIB_ROW(A) \
   GELIB_CASE(A, 0) GELIB_CASE(A, 1) GELIB_CASE(A, 2) GELIB_CASE(A, 3) GELIB_CASE(A, 4) GELIB_CASE(A, 5) GELIB_CASE(A, 6)

@@ -93,6 +93,9 @@ int launch_unrolled_fwd(const FwdArgs &a, bool diag, int ti, int lcap, int nbloc
 // lcap: largest l present in the gradient; lop: largest l of an operand (above kLT: the kernel for l up to kLTMax, which
 // exists for CGproduct with power-of-two channel counts and lcap <= kLTMax only -- unrolled_bwd_takes says so)
 bool unrolled_bwd_takes(bool diag, bool padded, int lcap, int lop);
+// largest l the backward kernel that launch_unrolled_bwd picks has code for (its step records are laid out for it),
+// or -1 when no backward kernel takes the vector
+int unrolled_bwd_cap(int lcap, int lop);
 int launch_unrolled_bwd(const BwdArgs &a, bool diag, int lcap, int lop, int nblocks, size_t lds_bytes, hipStream_t s);
 
 }  // namespace gelib_hip

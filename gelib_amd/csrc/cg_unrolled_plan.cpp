@@ -14,10 +14,11 @@ namespace {
 
 int g_fwd_block_bytes = 96 * 1024;   // product bytes one forward block aims to write
 int g_fwd_lds_bytes = 16 * 1024;     // LDS one forward block may use for its staged operands
-int g_fwd_cell_tile = 64;             // cells per tile of the forward launch (0 = all cells in one tile)
+int g_fwd_cell_tile = -1;            // cells per tile of the forward launch (0 = all cells in one tile, -1 = by channels)
 int g_fwd_ti = 0;                    // 0 = widest tile that divides every n1, else force 1 / 2 / 4
 int g_bwd_enable = 1;
 int g_bwd_l6_enable = 1;  // the backward kernel for operands up to l = 6
+int g_bwd_lds_target = 40 * 1024;  // LDS bytes per block the backward kernel aims at when it picks the cells per block
 int g_fwd_enable = 1;
 
 struct DevicePlan {
@@ -100,6 +101,37 @@ int ilog2(int v) {
 
 namespace {
 
+// Step records for the backward kernels: for every pair, one record per (m1,m2) step in the order the kernel runs
+// them (row number m = m1 + m2 rising from -ltop, m1 rising inside a row), holding C_l[m1,m2] for
+// l = |l1-l2| .. ltop = min(l1+l2, cap) -- zero where the part is absent or l < |m| -- padded to a power of two floats.
+// cap is the largest l the kernel that will run has code for (unrolled_bwd_cap).  A pair's records start on a 64-byte
+// boundary of the device allocation and are padded to whole 64-byte groups, the unit the kernel loads.
+void append_step_records(bool diag, int cap, size_t pair_bytes, std::vector<PairRec> *pairs, std::vector<float> *bank) {
+  (void)diag;
+  for (auto &p : *pairs) p.rec_off = -1;
+  if (cap < 0) return;
+  while ((pair_bytes + bank->size() * sizeof(float)) % 64) bank->push_back(0.f);
+  for (auto &p : *pairs) {
+    const int lmin = std::abs(p.l1 - p.l2), ltop = std::min(p.l1 + p.l2, cap);
+    if (lmin > ltop) continue;
+    const int nl = ltop - lmin + 1, w2 = 2 * p.l2 + 1;
+    int recw = 1;
+    while (recw < nl) recw *= 2;
+    p.rec_off = (int)bank->size();
+    for (int m = -ltop; m <= ltop; m++)
+      for (int m1 = std::max(-p.l1, m - p.l2); m1 <= std::min(p.l1, m + p.l2); m1++) {
+        const int m2 = m - m1;
+        for (int dl = 0; dl < recw; dl++) {
+          float c = 0.f;
+          if (dl < nl && dl < kMaxDl && p.ri[dl] >= 0 && lmin + dl >= std::abs(m))
+            c = (*bank)[p.cg_base + p.cg[dl] + (m1 + p.l1) * w2 + (m2 + p.l2)];
+          bank->push_back(c);
+        }
+      }
+    while (bank->size() % 16) bank->push_back(0.f);
+  }
+}
+
 // Build (or fetch) the device tables for a list of triples.  xs/ys/rs give (l, n) of the l-sorted parts.
 int get_plan(bool diag, const std::vector<VecTriple> &triples, const std::vector<std::pair<int, int>> &xs,
              const std::vector<std::pair<int, int>> &ys, const std::vector<int> &rls, const DevicePlan **out) {
@@ -167,8 +199,13 @@ int get_plan(bool diag, const std::vector<VecTriple> &triples, const std::vector
   if (bank.size() % 2) bank.push_back(0.f);
   plan.zero_off = (int)bank.size();
   bank.resize(bank.size() + (2 * kLTMax + 1) * (2 * kLTMax + 1) + 1, 0.f);
-  plan.bank_len = (int)bank.size();
   const size_t pair_bytes = plan.pairs.size() * sizeof(PairRec);
+  {
+    int lcap = 0, lop = 0;
+    for (auto &t : triples) lcap = std::max(lcap, t.l), lop = std::max(lop, std::max(t.l1, t.l2));
+    append_step_records(diag, unrolled_bwd_cap(lcap, lop), pair_bytes, &plan.pairs, &bank);
+  }
+  plan.bank_len = (int)bank.size();
   const size_t bank_bytes = bank.size() * sizeof(float);
   char *d = nullptr;
   GELIB_HIP_TRY(hipMalloc((void **)&d, pair_bytes + bank_bytes));
@@ -229,7 +266,14 @@ int run_fwd(bool diag, const std::vector<VecTriple> &triples, const std::vector<
   for (auto &t : triples) lcap = std::max(lcap, t.l);
   // The cells are cut into tiles; the blocks of a tile (every pair, every run of cells inside the tile) have
   // consecutive indices, so blocks that run at the same time write into the same neighbourhood of every product part.
-  const long long tile = g_fwd_cell_tile > 0 ? std::min<long long>(g_fwd_cell_tile, ncells) : ncells;
+  // Measured in one process, forward pass: L=4 with 16 channels 4.41 ms at 64 cells per tile, 4.30 at 32, 4.56 at 128;
+  // 8 channels 4.34 at 32 and 64, 4.89 at 4096; 4 channels (128-byte pieces per pair and row) 7.0 at 64, 6.7 at 1024,
+  // 5.85 at 4096, 7.9 with all cells in one tile.
+  long long auto_tile = 4096;
+  for (auto &p : plan->pairs)
+    if ((long long)p.n1 * (diag ? 1 : p.n2) >= 64) auto_tile = 32;
+  const long long want_tile = g_fwd_cell_tile < 0 ? auto_tile : g_fwd_cell_tile;
+  const long long tile = want_tile > 0 ? std::min<long long>(want_tile, ncells) : ncells;
   for (int i = 0; i < a.npairs; i++) {
     const PairRec &p = plan->pairs[i];
     long long rows = 0;
@@ -313,7 +357,20 @@ int run_bwd(bool diag, const std::vector<VecTriple> &triples, const std::vector<
   for (size_t i = 0; i < ys.size(); i++) a.yrows[i] = 2 * ys[i].first + 1;
   // enough cells per block to give every wave a full run of 64 slots, as far as LDS allows
   int cpb = std::max(1, kBlock / std::min(kBlock, u_min));
-  while (cpb > 1 && unrolled_bwd_lds_bytes(a.bank_len, a.xsize, a.ysize, cpb) > 64 * 1024) cpb >>= 1;
+  // ... but no more than leave LDS for the blocks the registers allow on a compute unit (four; three for the kernel
+  // for operands above kLT), as long as the block keeps at least two runs per wave; 64 KB at most in any case
+  const size_t lds_target = lop > kLT ? 52 * 1024 : (size_t)g_bwd_lds_target;
+  auto runs_at = [&](int c) {
+    long long runs = 0;
+    for (auto &p : plan->pairs) runs += (((long long)c << p.log2_u) + kWave - 1) / kWave;
+    return runs;
+  };
+  while (cpb > 1) {
+    const size_t need = unrolled_bwd_lds_bytes(a.bank_len, a.xsize, a.ysize, cpb);
+    if (need <= lds_target) break;
+    if (need <= 64 * 1024 && runs_at(cpb / 2) < 2 * (kBlock / kWave)) break;
+    cpb >>= 1;
+  }
   const size_t lds = unrolled_bwd_lds_bytes(a.bank_len, a.xsize, a.ysize, cpb);
   if (lds > 150 * 1024) return GELIB_HIP_OK;
   a.cells_per_block = cpb;
@@ -425,7 +482,7 @@ int unrolled_set_option(const char *name, int value) {
     return GELIB_HIP_OK;
   }
   if (!std::strcmp(name, "fwd_cell_tile")) {
-    if (value < 0) return GELIB_HIP_ERR_ARG;
+    if (value < -1) return GELIB_HIP_ERR_ARG;
     g_fwd_cell_tile = value;
     return GELIB_HIP_OK;
   }
@@ -435,6 +492,11 @@ int unrolled_set_option(const char *name, int value) {
   }
   if (!std::strcmp(name, "unrolled_fwd")) {
     g_fwd_enable = value;
+    return GELIB_HIP_OK;
+  }
+  if (!std::strcmp(name, "bwd_lds_target")) {
+    if (value < 1024 || value > 150 * 1024) return GELIB_HIP_ERR_ARG;
+    g_bwd_lds_target = value;
     return GELIB_HIP_OK;
   }
   if (!std::strcmp(name, "unrolled_bwd_l6")) {

@@ -57,7 +57,10 @@ WORKLOADS = {
     # name: (kind, B, tau_x, tau_y, maxl, diag)
     "so3vec_cg_L4_tau16_B32768_maxl4": ("vec", 32768, {l: 16 for l in range(5)}, {l: 16 for l in range(5)}, 4, False),
     "so3vec_cg_L4_tau16_B32768_uncapped": ("vec", 32768, {l: 16 for l in range(5)}, {l: 16 for l in range(5)}, -1, False),
-    "so3part_cg_2x3to4_n32_B65536": ("vec", 65536, {2: 32}, {3: 32}, 4, False),
+    # kind "part": ONE triple through the part-level entry points (forward; backward = back0 + back1, two calls, as
+    # the reference's SO3part operator makes them); the fifth field is the l of the triple
+    "so3part_cg_2x3to4_n32_B65536": ("part", 65536, {2: 32}, {3: 32}, 4, False),
+    "so3vec_cg_l2_x_l3_n32_B65536_maxl4": ("vec", 65536, {2: 32}, {3: 32}, 4, False),   # the same pair into l = 1..4
     "so3vec_diagcg_L6_n64_B131072": ("vec", 131072, {l: 64 for l in range(7)}, {l: 64 for l in range(7)}, 6, True),
     "so3part_cg_10x10_all_l_n8_B16384": ("vec", 16384, {10: 8}, {10: 8}, -1, False),
     "so3vec_diagcg_L4_n64_B131072": ("vec", 131072, {l: 64 for l in range(5)}, {l: 64 for l in range(5)}, 4, True),
@@ -66,7 +69,7 @@ WORKLOADS = {
     "so3vec_cg_L4_tau4_B524288_maxl4": ("vec", 524288, {l: 4 for l in range(5)}, {l: 4 for l in range(5)}, 4, False),
     "so3vec_cg_L2_tau64_B8192_maxl2": ("vec", 8192, {l: 64 for l in range(3)}, {l: 64 for l in range(3)}, 2, False),
     "so3vec_diagcg_L4_n64_B131072_uncapped": ("vec", 131072, {l: 64 for l in range(5)}, {l: 64 for l in range(5)}, -1, True),
-    "so3part_cg_1x1to1_n16_B1024": ("vec", 1024, {1: 16}, {1: 16}, 1, False),
+    "so3part_cg_1x1to1_n16_B1024": ("part", 1024, {1: 16}, {1: 16}, 1, False),
     "so3vec_cg_l8l10_x_l9l10_tau4_B32768_maxl12": ("vec", 32768, {8: 4, 10: 4}, {9: 4, 10: 4}, 12, False),
 }
 HEADLINE = "so3vec_cg_L4_tau16_B32768_maxl4"
@@ -74,7 +77,7 @@ HEADLINE = "so3vec_cg_L4_tau16_B32768_maxl4"
 OTHER_CONFIGS = [("so3part_cg_1x1to1_n16_B1024", 1024), ("so3part_cg_2x3to4_n32_B65536", 512),
                  ("so3vec_diagcg_L6_n64_B131072", 64), ("so3vec_cg_L4_tau16_B32768_uncapped", 256),
                  ("so3part_cg_10x10_all_l_n8_B16384", 64)]
-ALIASES = {"cfg1": "so3part_cg_1x1to1_n16_B1024", "cfg4": "so3vec_cg_L4_tau16_B32768_maxl4", "cfg4u": "so3vec_cg_L4_tau16_B32768_uncapped",
+ALIASES = {"cg23": "so3vec_cg_l2_x_l3_n32_B65536_maxl4", "cfg1": "so3part_cg_1x1to1_n16_B1024", "cfg4": "so3vec_cg_L4_tau16_B32768_maxl4", "cfg4u": "so3vec_cg_L4_tau16_B32768_uncapped",
            "cfg2": "so3part_cg_2x3to4_n32_B65536", "cfg3": "so3vec_diagcg_L6_n64_B131072",
            "cfg5": "so3part_cg_10x10_all_l_n8_B16384", "diag4": "so3vec_diagcg_L4_n64_B131072",
            "diag4n16": "so3vec_diagcg_L4_n16_B524288", "cg6": "so3vec_cg_L6_tau8_B16384_maxl6",
@@ -109,7 +112,7 @@ def seeded_parts(torch, seed, B, tau, device, scale=1.0):
     return parts
 
 
-def cpu_slice(torch, xs, ys, gs, rs, xgs, ygs, maxl, diag, nsample, single_core):
+def cpu_slice(torch, xs, ys, gs, rs, xgs, ygs, maxl, diag, nsample, single_core, part=False):
     """The oracle on the first `nsample` samples: timed (one thread, if single_core, and with the batch loop split over
     the host's cores, which is what the reference's MultiLoop would do) and used as the checker of the GPU results for
     that slice.  Every real component is held to the parity rules of tests/gpu_util.py (gate, or one of the two stated
@@ -123,19 +126,34 @@ def cpu_slice(torch, xs, ys, gs, rs, xgs, ygs, maxl, diag, nsample, single_core)
     ora.lib()
     nth = max(1, min(16, ora.max_threads(), os.cpu_count() or 1))
     dt1 = None
-    if single_core:
+    if part:   # one triple: maxl is its l
+        def both(g, x, y, nthreads):
+            r = ora.cg_fwd(x[0], y[0], maxl, diag, nthreads)
+            a, b = ora.cg_bwd(g[0], x[0], y[0], diag, nthreads)
+            return [r], [a], [b]
+        if single_core:
+            t0 = time.perf_counter()
+            both(hg, hx, hy, 1)
+            dt1 = time.perf_counter() - t0
         t0 = time.perf_counter()
-        ora.vec_fwd(hx, hy, maxl, diag, nthreads=1)
-        ora.vec_bwd(hg, hx, hy, diag, nthreads=1)
-        dt1 = time.perf_counter() - t0
-    t0 = time.perf_counter()
-    r = ora.vec_fwd(hx, hy, maxl, diag, nthreads=nth)
-    xg, yg = ora.vec_bwd(hg, hx, hy, diag, nthreads=nth)
-    dt_all = time.perf_counter() - t0
-    r64 = ora.vec_fwd(U.c128(hx), U.c128(hy), maxl, diag, nthreads=nth)
-    xg64, yg64 = ora.vec_bwd(U.c128(hg), U.c128(hx), U.c128(hy), diag, nthreads=nth)
-    Sr = ora.vec_fwd_term_sums(hx, hy, maxl, diag, nthreads=nth)
-    Sx, Sy = ora.vec_bwd_term_sums(hg, hx, hy, diag, nthreads=nth)
+        r, xg, yg = both(hg, hx, hy, nth)
+        dt_all = time.perf_counter() - t0
+        r64, xg64, yg64 = both(U.c128(hg), U.c128(hx), U.c128(hy), nth)
+        Sr, Sx, Sy = ([a] for a in ora.cg_term_sums(hg[0], hx[0], hy[0], maxl, diag, nth))
+    else:
+        if single_core:
+            t0 = time.perf_counter()
+            ora.vec_fwd(hx, hy, maxl, diag, nthreads=1)
+            ora.vec_bwd(hg, hx, hy, diag, nthreads=1)
+            dt1 = time.perf_counter() - t0
+        t0 = time.perf_counter()
+        r = ora.vec_fwd(hx, hy, maxl, diag, nthreads=nth)
+        xg, yg = ora.vec_bwd(hg, hx, hy, diag, nthreads=nth)
+        dt_all = time.perf_counter() - t0
+        r64 = ora.vec_fwd(U.c128(hx), U.c128(hy), maxl, diag, nthreads=nth)
+        xg64, yg64 = ora.vec_bwd(U.c128(hg), U.c128(hx), U.c128(hy), diag, nthreads=nth)
+        Sr = ora.vec_fwd_term_sums(hx, hy, maxl, diag, nthreads=nth)
+        Sx, Sy = ora.vec_bwd_term_sums(hg, hx, hy, diag, nthreads=nth)
 
     def merge(gpu_parts, c32, c64, S):
         tot = {"components": 0, "outside_gate": 0.0, "cpu_f32_outside_gate_of_f64": 0.0, "by_rule_B": 0.0,
@@ -385,6 +403,9 @@ def run_cg_workload(torch, cabi, name, steps, warmup, batch=0, cpu_samples=0, si
     if batch:
         B = batch
     tr = out_type(tx, ty, maxl, diag)
+    part = kind == "part"
+    if part:
+        tr = {maxl: tr[maxl]}
     fwd_bytes, bwd_bytes = algorithmic_bytes(B, tx, ty, tr)
     scale_y = 1e-3 if "10x10" in name else 1.0
     xs = seeded_parts(torch, 1004, B, tx, dev)
@@ -395,10 +416,17 @@ def run_cg_workload(torch, cabi, name, steps, warmup, batch=0, cpu_samples=0, si
     ygs = [torch.empty_like(t) for t in ys]
 
     def fwd():
-        cabi.so3vec_fwd(rs, xs, ys, accumulate=False, diag=diag)
+        if part:
+            cabi.so3part_cg_fwd(rs[0], xs[0], ys[0], 0, accumulate=False)
+        else:
+            cabi.so3vec_fwd(rs, xs, ys, accumulate=False, diag=diag)
 
-    def bwd():
+    def bwd():   # for one triple too: both gradients from one pass over g, as gelib_amd.SO3part.CGproduct's backward does
         cabi.so3vec_bwd(xgs, ygs, gs, xs, ys, accumulate=False, diag=diag)
+
+    def bwd_two_calls():   # the reference's form: back0 and back1, each reading g
+        cabi.so3part_cg_back0(xgs[0], gs[0], ys[0], 0, accumulate=False)
+        cabi.so3part_cg_back1(ygs[0], gs[0], xs[0], 0, accumulate=False)
 
     if copy_probe:
         src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
@@ -429,6 +457,8 @@ def run_cg_workload(torch, cabi, name, steps, warmup, batch=0, cpu_samples=0, si
     full = B == WORKLOADS[name][1]
     rec = {"workload": name, "batch": B, "tau_x": {str(k): v for k, v in tx.items()},
            "tau_y": {str(k): v for k, v in ty.items()}, "maxl": maxl, "diag": diag,
+           "entry_points": ("gelib_hip_so3part_cg_fwd; gelib_hip_so3vec_cg_bwd on one-part vectors (both gradients from "
+                            "one pass over g)") if part else "gelib_hip_so3vec_cg_fwd; gelib_hip_so3vec_cg_bwd",
            "triples": sum(1 for l1 in tx for l2 in ty for l in range(abs(l1 - l2), l1 + l2 + 1) if l in tr),
            "kernel_path": {"fwd": PATH_NAMES.get(path_fwd, str(path_fwd)), "bwd": PATH_NAMES.get(path_bwd, str(path_bwd))},
            "timed_steps": steps, "ms_per_step_wall": wall * 1e3 / steps, "samples_per_s": B / (wall / steps),
@@ -442,9 +472,22 @@ def run_cg_workload(torch, cabi, name, steps, warmup, batch=0, cpu_samples=0, si
            "fwd_bwd_frac_of_peak": (fwd_bytes + bwd_bytes) / ((fwd_ms + bwd_ms) * 1e-3) / HBM_PEAK,
            "fwd_traffic_bytes": measured_traffic(name, "so3vec_fwd") if full else None,
            "bwd_traffic_bytes": measured_traffic(name, "so3vec_bwd") if full else None}
+    if part:
+        # the two part-level calls of the reference's operator, timed after the main loop (their results are the same
+        # gradients; the CPU slice below checks what they left in the buffers)
+        bwd_two_calls()
+        torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(steps):
+            bwd_two_calls()
+        b.record()
+        torch.cuda.synchronize()
+        rec["bwd_back0_plus_back1_ms"] = a.elapsed_time(b) / steps
+        rec["bwd_back0_plus_back1_algorithmic_bytes"] = 2 * fwd_bytes
     if cpu_samples:
         ns = min(cpu_samples, B)
-        c = cpu_slice(torch, xs, ys, gs, rs, xgs, ygs, maxl, diag, ns, single_core)
+        c = cpu_slice(torch, xs, ys, gs, rs, xgs, ygs, maxl, diag, ns, single_core, part)
         rec["parity"] = c["parity"]
         rec["cpu"] = {"samples": ns, "cores": c["cores"], "all_cores_samples_per_s": ns / c["all_cores_s"],
                       "single_core_samples_per_s": ns / c["single_core_s"] if c["single_core_s"] else None,

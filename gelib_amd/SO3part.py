@@ -89,6 +89,15 @@ class SO3part_CGproductFn(torch.autograd.Function):
     def backward(ctx, g):
         x, y = ctx.saved_tensors
         g = g.contiguous()
+        if x.shape[:-2] == g.shape[:-2] and y.shape[:-2] == g.shape[:-2]:
+            # no broadcast operand: both gradients from ONE pass over g (the vector-level backward on one-part
+            # vectors); the reference makes the two calls below, each of which reads g
+            gb = backend()
+            xg = torch.empty_like(x)
+            yg = torch.empty_like(y)
+            vec = gb.SO3vec.view
+            gb.SO3vec.setCGproduct_back(vec([xg]), vec([yg]), vec([g]), vec([x]), vec([y]))
+            return xg, yg, None
         xg = torch.zeros_like(x)
         yg = torch.zeros_like(y)
         _view(xg).add_CGproduct_back0(_view(g), _view(y))

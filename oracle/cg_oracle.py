@@ -206,6 +206,18 @@ def vec_bwd_term_sums(gparts, xparts, yparts, diag=False, nthreads=1):
         lib().ora_set_abs_coeffs(0)
 
 
+def cg_term_sums(g, x, y, l, diag=False, nthreads=1):
+    """The same for one triple: the sums for the product part l and for the two gradients of g."""
+    lib().ora_set_abs_coeffs(1)
+    try:
+        (mg,), (mx,), (my,) = _moduli([g]), _moduli([x]), _moduli([y])
+        r = cg_fwd(mx, my, l, diag, nthreads)
+        xg, yg = cg_bwd(mg, mx, my, diag, nthreads)
+        return r.real.copy(), xg.real.copy(), yg.real.copy()
+    finally:
+        lib().ora_set_abs_coeffs(0)
+
+
 def spharm(l, x, batch=None):
     """(B or 1, 3, n) float32 vectors -> (B, 2l+1, n) complex64 spherical harmonics, the reference's add_spharm into zeros."""
     x = np.ascontiguousarray(x, dtype=np.float32)

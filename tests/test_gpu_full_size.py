@@ -113,3 +113,39 @@ def test_full_size(cabi, name):
         for s in range(0, B, step):     # a slab at a time: the flipped copy of a whole part would double the footprint
             hi = min(B, s + step)
             assert torch.equal(b[s:hi], a[B - hi:B - s].flip(0)), name
+
+
+@pytest.mark.parametrize("case", [(1024, 1, 16, 1, 16, 1), (65536, 2, 32, 3, 32, 4)])
+def test_single_triple_configs(cabi, case):
+    """Configurations 1 and 2 exactly as listed: ONE (l1, l2, l) triple at full batch through the part-level entry
+    points (the reference's SO3part operator: add_CGproduct, add_CGproduct_back0, add_CGproduct_back1), and both
+    gradients once more from one pass over g (what the Python operator runs when no operand is broadcast).  Slices of
+    the batch are checked against the oracle's loops for the single triple."""
+    B, l1, n1, l2, n2, l = case
+    (x,), (y,) = parts(B, {l1: n1}, 21), parts(B, {l2: n2}, 22)
+    (g,) = parts(B, {l: n1 * n2}, 23)
+    r = torch.full((B, 2 * l + 1, n1 * n2), 3.0 - 1j, dtype=torch.complex64, device="cuda")
+    cabi.so3part_cg_fwd(r, x, y, 0, accumulate=False)
+    xg0 = torch.full_like(x, 5.0)
+    yg0 = torch.full_like(y, 5.0)
+    cabi.so3part_cg_back0(xg0, g, y, 0, accumulate=False)
+    cabi.so3part_cg_back1(yg0, g, x, 0, accumulate=False)
+    xg1, yg1 = torch.full_like(x, 7.0), torch.full_like(y, 7.0)
+    cabi.so3vec_bwd([xg1], [yg1], [g], [x], [y], accumulate=False)
+    torch.cuda.synchronize()
+    rng = np.random.default_rng(6)
+    k = 16
+    idx = np.unique(np.concatenate([np.arange(k), np.arange(B - k, B), rng.integers(0, B, k)]))
+    tidx = torch.from_numpy(idx).cuda()
+    hx, hy, hg = U.host(x[tidx]), U.host(y[tidx]), U.host(g[tidx])
+    r32 = ora.cg_fwd(hx, hy, l)
+    r64 = ora.cg_fwd(*U.c128([hx, hy]), l)
+    xg32, yg32 = ora.cg_bwd(hg, hx, hy)
+    xg64, yg64 = ora.cg_bwd(*U.c128([hg, hx, hy]))
+    Sr, Sx, Sy = ora.cg_term_sums(hg, hx, hy, l)
+    what = "triple (%d,%d,%d) n %dx%d B %d" % (l1, l2, l, n1, n2, B)
+    rep = U.assert_parity(U.host(r[tidx]), r32, r64, Sr, "fwd " + what)
+    assert rep["outside_gate"] * rep["components"] <= 1 + 1e-7 * rep["components"], rep
+    for got_x, got_y, tag in ((xg0, yg0, "back0/back1"), (xg1, yg1, "one pass")):
+        U.assert_parity(U.host(got_x[tidx]), xg32, xg64, Sx, "xg %s %s" % (tag, what))
+        U.assert_parity(U.host(got_y[tidx]), yg32, yg64, Sy, "yg %s %s" % (tag, what))

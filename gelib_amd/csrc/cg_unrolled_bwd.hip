@@ -13,6 +13,7 @@ int launch_unrolled_bwd_cg8_pad(const BwdArgs &a, int nblocks, size_t lds_bytes,
 int launch_unrolled_bwd_diag4_pad(const BwdArgs &a, int nblocks, size_t lds_bytes, hipStream_t s);
 int launch_unrolled_bwd_diag8_pad(const BwdArgs &a, int nblocks, size_t lds_bytes, hipStream_t s);
 int launch_unrolled_bwd_cg6_l6(const BwdArgs &a, int nblocks, size_t lds_bytes, hipStream_t s);
+int launch_unrolled_bwd_one(const BwdArgs &a, int nblocks, size_t lds_bytes, hipStream_t s);
 
 size_t unrolled_bwd_lds_bytes(int bank_len, int xsize, int ysize, int cells_per_block) {
   const int waves = kBlock / kWave;
@@ -38,6 +39,7 @@ int unrolled_bwd_cap(int lcap, int lop) {
 int launch_unrolled_bwd(const BwdArgs &a, bool diag, int lcap, int lop, int nblocks, size_t lds_bytes, hipStream_t s) {
   if (nblocks <= 0) return GELIB_HIP_OK;
   if (lop > kLT) return launch_unrolled_bwd_cg6_l6(a, nblocks, lds_bytes, s);
+  if (a.only_dl >= 0 && !diag && !a.padded) return launch_unrolled_bwd_one(a, nblocks, lds_bytes, s);
   if (a.padded) {
     if (diag) return lcap <= kLT ? launch_unrolled_bwd_diag4_pad(a, nblocks, lds_bytes, s)
                                  : launch_unrolled_bwd_diag8_pad(a, nblocks, lds_bytes, s);

@@ -97,13 +97,19 @@ __device__ __forceinline__ LanePos lane_pos(int run, int lane, int log2_u, int n
 // SIMD).  The kernels for operands up to l = 4 keep the tables: with records the product capped at l = 4 runs at the
 // same speed and the uncapped one slower (7.8 -> 9.6 ms; its records are 16 floats, one load per step, waited for
 // one step later).
-template <int L1, int L2, int LCAP, bool DIAG, bool WX, bool WY, bool PAD, bool REC>
+// ONLY >= 0: the call has ONE triple, l = |L1 - L2| + ONLY (a part-level call, or a vector call on one-part vectors):
+// the code for the other l of the pair is left out.  (The branch-free form reads rows of zeros and multiplies by
+// tables of zeros for the l that are absent: for (2, 3) -> 4 with 32 x 32 channels that is 510 multiply-adds per lane
+// and run where 350 are needed, and 24 row loads where 9 are.)
+template <int L1, int L2, int LCAP, bool DIAG, bool WX, bool WY, bool PAD, bool REC, int ONLY = -1>
 __device__ __forceinline__ void pair_bwd(const GParts<LCAP> &gp, PairPtr pr, CoeffPtr Cs, CoeffPtr Zc, GlobalRows zrows,
                                          const float2 *xs, const float2 *ys, float2 *xacc, float2 *yacc, int xsize,
                                          int ysize, long long cell0, int offs_add, const LanePos q) {
-  constexpr int LMIN = cabs_(L1 - L2);
-  constexpr int LTOP = cmin_(L1 + L2, LCAP);
-  if constexpr (LMIN > LCAP) return;  // no l of this pair can be present
+  constexpr int DL0 = ONLY >= 0 ? ONLY : 0;  // the pair's tables are indexed by dl = l - |L1 - L2|; the first one used
+  constexpr int LMIN = cabs_(L1 - L2) + DL0;
+  constexpr int LTOP = ONLY >= 0 ? LMIN : cmin_(L1 + L2, LCAP);
+  if constexpr (LMIN > LCAP || LMIN > L1 + L2) return;  // no l of this pair can be present
+  static_assert(!(REC && ONLY >= 0), "the step records hold every l of the pair");
   constexpr int NLP = LTOP - LMIN + 1;
   // scalar loads: the record sits in constant memory and the pointer is uniform
   const __attribute__((address_space(4))) PairRec &p = *pr;
@@ -139,11 +145,11 @@ __device__ __forceinline__ void pair_bwd(const GParts<LCAP> &gp, PairPtr pr, Coe
   CoeffPtr cl[NLP];
   static_for<NLP>([&](auto dl_c) __attribute__((always_inline)) {
     constexpr int dl = decltype(dl_c)::value;
-    const bool present = p.ri[dl] >= 0;
+    const bool present = p.ri[DL0 + dl] >= 0;
     const FastPart G = gp.G[LMIN + dl];
-    gptr[dl] = present ? (GlobalRows)G.ptr + cell * G.sb + (p.offs[dl] + offs_add + chan) : zrows;
+    gptr[dl] = present ? (GlobalRows)G.ptr + cell * G.sb + (p.offs[DL0 + dl] + offs_add + chan) : zrows;
     gsm[dl] = present ? G.sm : 0;
-    cl[dl] = present ? Cs + p.cg[dl] : Zc;
+    cl[dl] = present ? Cs + p.cg[DL0 + dl] : Zc;
   });
   constexpr int RECW = pow2ceil_(NLP);                 // floats per record
   constexpr int kGroup = 16;                           // floats per load
@@ -174,7 +180,8 @@ __device__ __forceinline__ void pair_bwd(const GParts<LCAP> &gp, PairPtr pr, Coe
   // them (the wave then waits once per pair, and 16 waves per compute unit keep enough bytes in flight to cover
   // the memory latency), otherwise as many m as fit the budget.  The kernels for l up to 8 hold more sums and are
   // near the register limit of three waves per SIMD already, so their budget is smaller.
-  constexpr int kRowBudget = LCAP <= 4 ? 32 : LCAP == kLTMax ? ((L1 > kLT || L2 > kLT) ? 16 : 32) : 14;
+  constexpr int kRowBudget =
+      (LCAP <= 4 || ONLY >= 0) ? 32 : LCAP == kLTMax ? ((L1 > kLT || L2 > kLT) ? 16 : 32) : 14;
   constexpr int ROWS = (LTOP + 1) * (LTOP + 1) - LMIN * LMIN;  // sum of 2l+1 over the l of the pair
   constexpr int PF = ROWS <= kRowBudget ? 2 * LTOP + 1 : (kRowBudget / NLP > 1 ? kRowBudget / NLP : 1);
   float2 gq[PF][NLP];
@@ -333,7 +340,21 @@ __device__ __forceinline__ void copy_image(const FastPart (&parts)[kFastIn], con
 
 // LT: largest operand l of the pairs the kernel has code for.
 // The kernel for operands above kLT is asked to fit three waves per SIMD (168 registers): left alone it takes 169.
-template <int LCAP, bool DIAG, bool WX, bool WY, bool PAD, int LT>
+// ONE: the call has one triple (a.only_dl says which l of its pair).
+template <int L1, int L2, int LCAP, bool DIAG, bool WX, bool WY, bool PAD>
+__device__ __forceinline__ void pair_bwd_one(int only_dl, const GParts<LCAP> &gp, PairPtr pr, CoeffPtr Cs, CoeffPtr Zc,
+                                             GlobalRows zrows, const float2 *xs, const float2 *ys, float2 *xacc,
+                                             float2 *yacc, int xsize, int ysize, long long cell0, int offs_add,
+                                             const LanePos q) {
+  static_for<2 * cmin_(L1, L2) + 1>([&](auto dc) __attribute__((always_inline)) {
+    constexpr int D = decltype(dc)::value;
+    if (only_dl == D)  // uniform
+      pair_bwd<L1, L2, LCAP, DIAG, WX, WY, PAD, false, D>(gp, pr, Cs, Zc, zrows, xs, ys, xacc, yacc, xsize, ysize, cell0,
+                                                           offs_add, q);
+  });
+}
+
+template <int LCAP, bool DIAG, bool WX, bool WY, bool PAD, int LT, bool ONE>
 __global__ void __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(LT > kLT ? 3 : 1)))
 unrolled_bwd_kernel(const BwdArgs a) {
   constexpr int KR = 2 * LCAP + 1;
@@ -364,7 +385,8 @@ unrolled_bwd_kernel(const BwdArgs a) {
 
   // The wave's visits: for each pair in turn, runs wave, wave+4, ... of the pair's cpb*U slots.
   const PairPtr pairs = (PairPtr)a.pairs;
-  const int npairs = a.npairs, offs_add = a.offs_add;
+  const int npairs = a.npairs, offs_add = a.offs_add, only_dl = a.only_dl;
+  (void)only_dl;
   auto runs_of = [&](int k) { return ((cpb << pairs[k].log2_u) + kWave - 1) >> 6; };
   GParts<LCAP> gp;
   static_for<LCAP + 1>([&](auto l) __attribute__((always_inline)) { gp.G[l.value] = a.g[l.value]; });
@@ -383,9 +405,14 @@ unrolled_bwd_kernel(const BwdArgs a) {
       switch (p->l1 * (kLTMax + 1) + p->l2) {
 #define GELIB_CASE(A, B)                                                                                      \
   case A * (kLTMax + 1) + B:                                                                                  \
-    if constexpr (A <= LT && B <= LT)                                                                         \
-      pair_bwd<A, B, LCAP, DIAG, WX, WY, PAD, (LT > kLT)>(gp, p, C, Zc, zrows, xs, ys, xacc, yacc, xsize, ysize, cell0, \
-                                                            offs_add, q);                                      \
+    if constexpr (A <= LT && B <= LT) {                                                                       \
+      if constexpr (ONE)                                                                                      \
+        pair_bwd_one<A, B, LCAP, DIAG, WX, WY, PAD>(only_dl, gp, p, C, Zc, zrows, xs, ys, xacc, yacc, xsize, ysize,   \
+                                                    cell0, offs_add, q);                                      \
+      else                                                                                                    \
+        pair_bwd<A, B, LCAP, DIAG, WX, WY, PAD, (LT > kLT)>(gp, p, C, Zc, zrows, xs, ys, xacc, yacc, xsize, ysize,    \
+                                                              cell0, offs_add, q);                            \
+    }                                                                                                         \
     break;
 #define GELIB_ROW(A) \
   GELIB_CASE(A, 0) GELIB_CASE(A, 1) GELIB_CASE(A, 2) GELIB_CASE(A, 3) GELIB_CASE(A, 4) GELIB_CASE(A, 5) GELIB_CASE(A, 6)
@@ -402,9 +429,9 @@ unrolled_bwd_kernel(const BwdArgs a) {
   if (WY) copy_image<false>(a.yg, a.yrows, a.ny, yacc_all, ysize, cell0, ncell, kWaves, cpb * ysize, a.accumulate != 0);
 }
 
-template <int LCAP, bool DIAG, bool WX, bool WY, bool PAD, int LT>
+template <int LCAP, bool DIAG, bool WX, bool WY, bool PAD, int LT, bool ONE>
 int launch_variant(const BwdArgs &a, int nblocks, size_t lds, hipStream_t s) {
-  auto kern = unrolled_bwd_kernel<LCAP, DIAG, WX, WY, PAD, LT>;
+  auto kern = unrolled_bwd_kernel<LCAP, DIAG, WX, WY, PAD, LT, ONE>;
   static bool attr_set = false;  // benign race: setting the attribute twice is harmless
   if (!attr_set) {
     GELIB_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -417,13 +444,13 @@ int launch_variant(const BwdArgs &a, int nblocks, size_t lds, hipStream_t s) {
 }
 
 // want_x / want_y select which gradients are computed
-template <int LCAP, bool DIAG, bool PAD, int LT = kLT>
+template <int LCAP, bool DIAG, bool PAD, int LT = kLT, bool ONE = false>
 int launch_bwd_variants(const BwdArgs &a, int nblocks, size_t lds_bytes, hipStream_t s) {
   static_assert(kLTMax == 6 && LT <= kLTMax, "the case table above lists l1, l2 = 0..6");
   const bool wx = a.want_x != 0, wy = a.want_y != 0;
-  if (wx && wy) return launch_variant<LCAP, DIAG, true, true, PAD, LT>(a, nblocks, lds_bytes, s);
-  if (wx) return launch_variant<LCAP, DIAG, true, false, PAD, LT>(a, nblocks, lds_bytes, s);
-  return launch_variant<LCAP, DIAG, false, true, PAD, LT>(a, nblocks, lds_bytes, s);
+  if (wx && wy) return launch_variant<LCAP, DIAG, true, true, PAD, LT, ONE>(a, nblocks, lds_bytes, s);
+  if (wx) return launch_variant<LCAP, DIAG, true, false, PAD, LT, ONE>(a, nblocks, lds_bytes, s);
+  return launch_variant<LCAP, DIAG, false, true, PAD, LT, ONE>(a, nblocks, lds_bytes, s);
 }
 
 }  // namespace

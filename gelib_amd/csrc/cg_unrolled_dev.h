@@ -44,6 +44,7 @@ struct BwdArgs {
   int xsize, ysize; // complex elements of one cell's packed x / y image
   int xrows[kFastIn], yrows[kFastIn];  // 2l+1 of each x / y part
   int cells_per_block;
+  int only_dl;      // -1, or: the call has one triple, l = |l1 - l2| + only_dl (the kernel built for that case)
 };
 
 size_t unrolled_bwd_lds_bytes(int bank_len, int xsize, int ysize, int cells_per_block);

@@ -17,6 +17,7 @@ int g_fwd_lds_bytes = 16 * 1024;     // LDS one forward block may use for its st
 int g_fwd_cell_tile = -1;            // cells per tile of the forward launch (0 = all cells in one tile, -1 = by channels)
 int g_fwd_ti = 0;                    // 0 = widest tile that divides every n1, else force 1 / 2 / 4
 int g_bwd_enable = 1;
+int g_bwd_one_enable = 1; // the backward kernel for calls with one triple
 int g_bwd_l6_enable = 1;  // the backward kernel for operands up to l = 6
 int g_bwd_lds_target = 40 * 1024;  // LDS bytes per block the backward kernel aims at when it picks the cells per block
 int g_fwd_enable = 1;
@@ -378,6 +379,9 @@ int run_bwd(bool diag, const std::vector<VecTriple> &triples, const std::vector<
   const size_t lds = unrolled_bwd_lds_bytes(a.bank_len, a.xsize, a.ysize, cpb);
   if (lds > 150 * 1024) return GELIB_HIP_OK;
   a.cells_per_block = cpb;
+  a.only_dl = -1;
+  if (triples.size() == 1 && !diag && !plan->padded && lop <= kLT && g_bwd_one_enable)
+    a.only_dl = triples[0].l - std::abs(triples[0].l1 - triples[0].l2);
   const long long nblocks = (ncells + cpb - 1) / cpb;
   if (nblocks > 0x7fffffffLL) return GELIB_HIP_ERR_ARG;
   rc = launch_unrolled_bwd(a, diag, lcap, lop, (int)nblocks, lds, s);
@@ -501,6 +505,10 @@ int unrolled_set_option(const char *name, int value) {
   if (!std::strcmp(name, "bwd_lds_target")) {
     if (value < 1024 || value > 150 * 1024) return GELIB_HIP_ERR_ARG;
     g_bwd_lds_target = value;
+    return GELIB_HIP_OK;
+  }
+  if (!std::strcmp(name, "unrolled_bwd_one")) {
+    g_bwd_one_enable = value;
     return GELIB_HIP_OK;
   }
   if (!std::strcmp(name, "unrolled_bwd_l6")) {

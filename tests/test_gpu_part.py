@@ -34,6 +34,11 @@ SHAPES = [
     (2, 10, 10, 7, 8, 8),        # large l: shape-agnostic kernels
     (1, 2, 2, 2, 70, 3),         # n1*n2 not a multiple of the wave
     (300, 1, 2, 3, 2, 2),
+    (3, 4, 4, 8, 4, 4),          # the largest and the smallest l of the (4, 4) pair
+    (3, 4, 4, 0, 8, 8),
+    (9, 0, 3, 3, 16, 4),
+    (2, 6, 6, 6, 2, 4),          # operands above l = 4, product l up to 6
+    (2, 5, 6, 1, 8, 2),
 ]
 
 

@@ -59,6 +59,7 @@ struct OnePairMfmaArgs {
   long long ncells;
   int l1, l2, lmin, lt, nl;
   int offs_add, accumulate;
+  int paired;  // backward: the row numbers run in pairs (m, m + 2 l1 + 1), see the kernel
 };
 
 typedef float f16v __attribute__((ext_vector_type(16)));
@@ -126,11 +127,23 @@ __global__ void __launch_bounds__(64) onepair_mfma_bwd_kernel(const OnePairMfmaA
     c.dlb = dl0;
     c.left = (nl - dl0 + 1) >> 1;
   };
+  // Order of the row numbers.  Plain: -lt .. lt.  Paired (l1 = l2, every l up to 2 l1 possible): -lt, 1, -lt + 1, 2,
+  // ..., -1, lt, 0.  For m < 0 the pairs (m1, m2) with m1 + m2 = m occupy the columns m1 = -l1 .. m + l2, for
+  // m' = m + 2 l1 + 1 > 0 the columns m1 = m' - l2 .. l1 = m + l1 + 1 .. l1: the two sets are complementary, and the
+  // coefficient of a column that has no pair for the row number of a step is zero.  So the matrix steps of m and of m'
+  // add into ONE set of sums (different columns), and the vector work that follows the matrix steps -- the same number
+  // of instructions whether 1 or 21 columns hold a pair -- runs 21 times instead of 41.  A column's row of y moves on by one
+  // per pair of row numbers exactly as it does per row number, so the sums of the y-gradient travel as before; a row
+  // of the y-gradient now collects its terms with m > 0 first (parked when it leaves the last column) and those with
+  // m <= 0 afterwards (added at the end).
+  const int paired = a.paired;
+  auto is_last = [&](int m) __attribute__((always_inline)) { return paired ? m == 0 : m == lt; };
+  auto closes = [&](int m) __attribute__((always_inline)) { return !paired || m >= 0; };  // the sums are complete after m
   auto next_step = [&](Cursor &c) __attribute__((always_inline)) {
     if (--c.left > 0) {
       c.dlb += 2;
-    } else if (c.m < lt) {
-      start_m(c, c.m + 1);
+    } else if (!is_last(c.m)) {
+      start_m(c, paired ? (c.m < 0 ? c.m + 2 * l1 + 1 : c.m - 2 * l1) : c.m + 1);
     } else {
       c.dlb = nl;
       c.left = 1 << 30;
@@ -159,8 +172,11 @@ __global__ void __launch_bounds__(64) onepair_mfma_bwd_kernel(const OnePairMfmaA
 
   // the sums of one m are in D: both gradients, then every row of the y-gradient moves one lane up
   auto finish_m = [&](int m) __attribute__((always_inline)) {
-    // the lane's m2 = m - m1; outside [-l2, l2] (or m1 beyond l1) every coefficient was zero and so is Q
-    int m2 = m - (i - l1);
+    // the lane's m2 = m - m1; outside [-l2, l2] (or m1 beyond l1) every coefficient was zero and so is Q.  Paired: the
+    // columns up to m1 = mneg + l2 belong to the negative row number of the pair
+    const int mneg = m - 2 * l1 - 1;
+    const int mlane = (paired && m > 0 && (i - l1) <= mneg + l2) ? mneg : m;
+    int m2 = mlane - (i - l1);
     m2 = m2 < -l2 ? -l2 : (m2 > l2 ? l2 : m2);
     const float4 *yrow = reinterpret_cast<const float4 *>(ys + (m2 + l2) * 8);
     float2 yv[8];
@@ -187,7 +203,7 @@ __global__ void __launch_bounds__(64) onepair_mfma_bwd_kernel(const OnePairMfmaA
           S[j].y = fmaf(qi, xv[b].x, S[j].y);
           S[j].y = fmaf(-qr, xv[b].y, S[j].y);
         }
-    if (m < lt) {  // the row that leaves m1 = l1 is complete; after the last m the rows stay where they are
+    if (!is_last(m)) {  // the row that leaves m1 = l1 is complete (paired: its terms with m > 0 are); after the last m the rows stay where they are
 #pragma unroll
       for (int j = 0; j < 8; j++) {
         S[j].x = wave_shr1(S[j].x);
@@ -236,21 +252,25 @@ __global__ void __launch_bounds__(64) onepair_mfma_bwd_kernel(const OnePairMfmaA
         D[2] = __builtin_amdgcn_mfma_f32_32x32x2f32(g.z, c, D[2], 0, 0, 0);
         D[3] = __builtin_amdgcn_mfma_f32_32x32x2f32(g.w, c, D[3], 0, 0, 0);
       }
-      fresh = ck.left == 1;  // the next step starts a new m
+      fresh = ck.left == 1 && closes(ck.m);  // the next step starts new sums
       fetch(cf, G[k], C[k]);
       next_step(cf);
       __builtin_amdgcn_sched_barrier(0);
-      if (ck.left == 1) finish_m(ck.m);  // uniform; an idle step never ends an m
+      if (ck.left == 1 && closes(ck.m)) finish_m(ck.m);  // uniform; an idle step never ends an m
       next_step(ck);
     });
   }
-  // the rows that are still on their way are complete as well: column i holds m2 = lt - (i - l1)
+  // the rows that are still on their way are complete as well: column i holds m2 = (the last m) - (i - l1).  They are
+  // added to what is parked (zeros, or -- paired -- the row's terms with m > 0)
   {
-    const int m2 = lt - (i - l1);
+    const int m2 = (paired ? 0 : lt) - (i - l1);
     if (i < r1 && m2 >= -l2 && m2 <= l2) {
       float4 *dst = reinterpret_cast<float4 *>(accy[h] + (m2 + l2) * 8);
 #pragma unroll
-      for (int q = 0; q < 4; q++) dst[q] = make_float4(S[2 * q].x, S[2 * q].y, S[2 * q + 1].x, S[2 * q + 1].y);
+      for (int q = 0; q < 4; q++) {
+        const float4 o = dst[q];
+        dst[q] = make_float4(o.x + S[2 * q].x, o.y + S[2 * q].y, o.z + S[2 * q + 1].x, o.w + S[2 * q + 1].y);
+      }
     }
   }
   __syncthreads();
@@ -401,12 +421,12 @@ struct Tables {
 };
 std::mutex g_mutex;
 std::map<std::vector<int>, Tables> g_tables;  // (device, l1, l2, lmin, lt, nl, present...) -> device tables
-int g_enable = 1, g_enable_fwd = 1;
+int g_enable = 1, g_enable_fwd = 1, g_paired = 1;
 
-int device_tables(int l1, int l2, int lmin, int lt, int nl, const std::vector<int> &present, Tables *out) {
+int device_tables(int l1, int l2, int lmin, int lt, int nl, const std::vector<int> &present, bool paired, Tables *out) {
   int dev = 0;
   GELIB_HIP_TRY(hipGetDevice(&dev));
-  std::vector<int> key = {dev, l1, l2, lmin, lt, nl};
+  std::vector<int> key = {dev, l1, l2, lmin, lt, nl, paired ? 1 : 0};
   key.insert(key.end(), present.begin(), present.end());
   std::lock_guard<std::mutex> lock(g_mutex);
   auto it = g_tables.find(key);
@@ -419,7 +439,14 @@ int device_tables(int l1, int l2, int lmin, int lt, int nl, const std::vector<in
       }
     std::vector<float> coef;
     int step = 0;
-    for (int m = -lt; m <= lt; m++) {
+    std::vector<int> order;  // the row numbers in the order the backward kernel takes them
+    if (paired) {
+      for (int m = -lt; m < 0; m++) order.push_back(m), order.push_back(m + 2 * l1 + 1);
+      order.push_back(0);
+    } else {
+      for (int m = -lt; m <= lt; m++) order.push_back(m);
+    }
+    for (int m : order) {
       const int dl0 = std::max(std::abs(m), lmin) - lmin;   // the first l with a row m
       const int nks = (nl - dl0 + 1) / 2;
       for (int ks = 0; ks < nks; ks++, step++) {
@@ -510,8 +537,10 @@ int onepair_mfma_vec_bwd(const VecPlan &plan, const std::vector<const gelib_part
   if (ncells > 0x7fffffffLL) return GELIB_HIP_OK;
   Tables t;
   const int lt = std::min(l1 + l2, lmax);
-  int rc = device_tables(l1, l2, lmin, lt, nl, present, &t);
+  const bool paired = g_paired && l1 == l2 && lt == 2 * l1;
+  int rc = device_tables(l1, l2, lmin, lt, nl, present, paired, &t);
   if (rc) return rc;
+  a.paired = paired ? 1 : 0;
   a.coef = t.coef;
   a.nsteps = t.nsteps;
   a.ncells = ncells;
@@ -566,7 +595,7 @@ int onepair_mfma_vec_fwd(const VecPlan &plan, const std::vector<const gelib_part
   if (ncells > 0x7fffffffLL) return GELIB_HIP_OK;
   Tables t;
   const int lt = std::min(l1 + l2, lmax);
-  int rc = device_tables(l1, l2, lmin, lt, nl, present, &t);
+  int rc = device_tables(l1, l2, lmin, lt, nl, present, false, &t);
   if (rc) return rc;
   a.coef_fwd = t.coef_fwd;
   a.nsteps_fwd = t.nsteps_fwd;
@@ -601,6 +630,10 @@ int onepair_mfma_vec_fwd(const VecPlan &plan, const std::vector<const gelib_part
 int onepair_mfma_set_option(const char *name, int value) {
   if (!std::strcmp(name, "onepair_mfma_fwd")) {
     g_enable_fwd = value;
+    return GELIB_HIP_OK;
+  }
+  if (!std::strcmp(name, "onepair_mfma_paired")) {
+    g_paired = value;
     return GELIB_HIP_OK;
   }
   if (!std::strcmp(name, "onepair_mfma")) {

@@ -407,6 +407,97 @@ __global__ void __launch_bounds__(256) diag6_bwd_kernel(const Diag6Args a) {
   });
 }
 
+// The backward pass when every part of y up to l = 6 is there: the waves' sets of l2 are fixed at compile time, {6},
+// {5, 0}, {4, 1}, {3, 2} (13, 12, 12, 12 rows), so a wave keeps its rows of y in registers from the first pair to the
+// last and y is read once (the kernel above reads the rows of y[l2] again for every l1: 1.23 times the algorithmic
+// bytes on L = 6, 64 channels).  Everything else is as above -- the y-gradient of a pair is added into the wave's rows
+// of the image in LDS, the x-gradient partials meet in LDS after the last pair of an l1 -- so the sums are formed in
+// the same order and the results are the same bits.  The four waves run four instantiations of the loop over l1 and
+// meet at its two barriers per l1.
+template <int LCAP, bool PACKED, int LA, int LB>
+__device__ __forceinline__ void bwd_wave_set(const Diag6Args &a, float2 *yimg, float2 *xpart, const WavePos q, int wave,
+                                             int lane) {
+  constexpr int kXRows = 2 * kL6 + 1;
+  constexpr int RB = LB >= 0 ? 2 * LB + 1 : 1;
+  constexpr int LBX = LB >= 0 ? LB : 0;
+  const bool accumulate = a.accumulate != 0;
+  const bool wx = a.want_x != 0, wy = a.want_y != 0;
+  float2 ya[2 * LA + 1], yb[RB];
+#pragma unroll
+  for (int m = 0; m <= 2 * LA; m++) ya[m] = make_float2(0.f, 0.f);
+#pragma unroll
+  for (int m = 0; m < RB; m++) yb[m] = make_float2(0.f, 0.f);
+  if (wx) {
+    load_rows<LA, PACKED>(ya, a.y[LA], q);
+    if constexpr (LB >= 0) load_rows<LBX, PACKED>(yb, a.y[LBX], q);
+  }
+  static_for<kNP>([&](auto l1c) __attribute__((always_inline)) {
+    constexpr int L1 = decltype(l1c)::value;
+    if (a.x[L1].ptr != nullptr) {  // the same for the whole block
+      float2 xv[2 * L1 + 1], ax[2 * L1 + 1];
+      if (wy) {
+        load_rows<L1, PACKED>(xv, a.x[L1], q);
+      } else {
+#pragma unroll
+        for (int m1 = 0; m1 <= 2 * L1; m1++) xv[m1] = make_float2(0.f, 0.f);
+      }
+#pragma unroll
+      for (int m1 = 0; m1 <= 2 * L1; m1++) ax[m1] = make_float2(0.f, 0.f);
+      bwd_pair<L1, LA, LCAP, PACKED>(a, xv, ya, ax, yimg, q);
+      if constexpr (LB >= 0) bwd_pair<L1, LBX, LCAP, PACKED>(a, xv, yb, ax, yimg, q);
+      if (!wx) return;  // continues with the next l1; uniform for the block
+      float2 *mine = xpart + wave * kXRows * 64 + lane;
+#pragma unroll
+      for (int m1 = 0; m1 <= 2 * L1; m1++) mine[m1 * 64] = ax[m1];
+      __syncthreads();
+      const FastPart XG = a.xg[L1];
+      RowPtr row0 = cell_row0(XG, q.cell);
+      const long long step = row_step(XG);
+      const unsigned xlo = lane_offset<PACKED>(XG, q);
+      static_for<2 * L1 + 1>([&](auto rc) __attribute__((always_inline)) {
+        constexpr int r = decltype(rc)::value;
+        if ((r & 3) == wave && q.live) {
+          float2 t = xpart[(0 * kXRows + r) * 64 + lane];
+#pragma unroll
+          for (int k = 1; k < 4; k++) {
+            const float2 u = xpart[(k * kXRows + r) * 64 + lane];
+            t.x += u.x;
+            t.y += u.y;
+          }
+          row_store(row0 + r * step, xlo, t, accumulate);
+        }
+      });
+      __syncthreads();
+    }
+  });
+  if (wy) {
+    if (a.yg[LA].ptr != nullptr) store_rows<LA, PACKED>(yimg + (LA * LA) * 64 + lane, 64, a.yg[LA], q, accumulate);
+    if constexpr (LB >= 0)
+      if (a.yg[LBX].ptr != nullptr) store_rows<LBX, PACKED>(yimg + (LBX * LBX) * 64 + lane, 64, a.yg[LBX], q, accumulate);
+  }
+}
+
+template <int LCAP, bool PACKED>
+__global__ void __launch_bounds__(256) diag6_bwd_sets_kernel(const Diag6Args a) {
+  __shared__ float2 yimg[kImgRows * 64];
+  __shared__ float2 xpart[4 * (2 * kL6 + 1) * 64];  // [wave][row][lane]
+  const WavePos q = wave_pos(a, blockIdx.x);
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  for (int e = threadIdx.x; e < kImgRows * 64; e += 256) yimg[e] = make_float2(0.f, 0.f);
+  __syncthreads();
+  if (wave == 0) bwd_wave_set<LCAP, PACKED, 6, -1>(a, yimg, xpart, q, wave, lane);
+  else if (wave == 1) bwd_wave_set<LCAP, PACKED, 5, 0>(a, yimg, xpart, q, wave, lane);
+  else if (wave == 2) bwd_wave_set<LCAP, PACKED, 4, 1>(a, yimg, xpart, q, wave, lane);
+  else bwd_wave_set<LCAP, PACKED, 3, 2>(a, yimg, xpart, q, wave, lane);
+}
+
+template <int LCAP, bool PACKED>
+int launch_diag6_bwd_sets_variant(const Diag6Args &a, hipStream_t s) {
+  hipLaunchKernelGGL((diag6_bwd_sets_kernel<LCAP, PACKED>), dim3((unsigned)a.nwaves), dim3(256), 0, s, a);
+  GELIB_HIP_TRY(hipGetLastError());
+  return GELIB_HIP_OK;
+}
+
 template <int LCAP, bool PACKED>
 int launch_diag6_fwd_variant(const Diag6Args &a, hipStream_t s) {
   hipLaunchKernelGGL((diag6_fwd_kernel<LCAP, PACKED>), dim3((unsigned)a.nwaves), dim3(256), 0, s, a);

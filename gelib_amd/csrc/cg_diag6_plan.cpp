@@ -18,6 +18,7 @@ std::mutex g_mutex;
 std::map<int, float *> g_banks;                     // device -> coefficient table
 std::map<std::pair<int, std::vector<int>>, int *> g_offs;  // (device, offsets) -> device copy
 int g_enable = 1;
+int g_sets_enable = 1;  // backward: the kernel with the waves' sets of l2 fixed at compile time, where it applies
 
 int device_bank(const float **out) {
   int dev = 0;
@@ -181,7 +182,12 @@ int diag6_vec_bwd(const VecPlan &plan, const std::vector<const gelib_part_desc *
   a.accumulate = accumulate ? 1 : 0;
   a.want_x = xg.empty() ? 0 : 1;
   a.want_y = yg.empty() ? 0 : 1;
-  if ((rc = a.lg_npad < 6 ? launch_diag6_bwd_l6_packed(a, s) : launch_diag6_bwd_l6(a, s))) return rc;
+  bool all_y = true;
+  for (int l = 0; l < kNP; l++) all_y = all_y && a.y[l].ptr != nullptr;
+  if (a.lg_npad < 6) rc = launch_diag6_bwd_l6_packed(a, s);
+  else if (all_y && g_sets_enable) rc = launch_diag6_bwd_l6_sets(a, s);
+  else rc = launch_diag6_bwd_l6(a, s);
+  if (rc) return rc;
   *used = 1;
   return GELIB_HIP_OK;
 }
@@ -212,6 +218,10 @@ int diag6_part(int kind, const long long E[3], const gelib_part_desc *r, const g
 int diag6_set_option(const char *name, int value) {
   if (!std::strcmp(name, "diag6")) {
     g_enable = value;
+    return GELIB_HIP_OK;
+  }
+  if (!std::strcmp(name, "diag6_sets")) {
+    g_sets_enable = value;
     return GELIB_HIP_OK;
   }
   return GELIB_HIP_ERR_ARG;

@@ -135,3 +135,50 @@ def test_more_parts_than_the_fused_kernels_take(cabi, case):
     per pair of parts on the single-pair kernels (or again per triple) going backward."""
     fwd, bwd = run_vec(cabi, *case, False, seed=800, force_generic=False)
     assert fwd == 1 and bwd in (1, 5)
+
+
+def test_tuning_options_leave_the_results_alone(cabi):
+    """The launch-shape options (cells per tile and bytes per block of the forward pass, LDS per block of the backward
+    pass) and the switches between kernels that compute the same sums (the Diag backward kernel with fixed sets of l2,
+    the single-triple kernel, the paired row numbers of the matrix-core kernel) change timings only.  Options that keep
+    the order of every sum are held to the same bits, the others to the parity rules."""
+    cabi.set_option("force_generic", 0)
+
+    def product(tx, ty, maxl, diag, seed, B=37):
+        xs = [U.dev(U.seeded(seed + l, B, 2 * l + 1, n)) for l, n in sorted(tx.items())]
+        ys = [U.dev(U.seeded(seed + 40 + l, B, 2 * l + 1, n)) for l, n in sorted(ty.items())]
+        tau = cabi.so3type_product(tx, ty, maxl, diag)
+        rs = [torch.empty(B, 2 * l + 1, n, dtype=torch.complex64, device="cuda") for l, n in sorted(tau.items())]
+        cabi.so3vec_fwd(rs, xs, ys, accumulate=False, diag=diag)
+        xg, yg = [torch.empty_like(t) for t in xs], [torch.empty_like(t) for t in ys]
+        cabi.so3vec_bwd(xg, yg, rs, xs, ys, accumulate=False, diag=diag)
+        torch.cuda.synchronize()
+        return [U.host(t) for t in rs], [U.host(t) for t in xg + yg]
+
+    def same_bits(a, b):
+        return all(np.array_equal(p.view(np.float32), q.view(np.float32)) for p, q in zip(a, b))
+
+    def close(a, b):   # two float32 evaluations of the same sums in different orders
+        return all(np.max(np.abs(p - q)) <= 2e-5 * max(1.0, np.max(np.abs(p))) for p, q in zip(a, b))
+
+    L4 = {l: 4 for l in range(5)}
+    L6 = {l: 64 for l in range(7)}
+    cases = [
+        # option, default, other values, workload, forward bits kept, backward bits kept
+        ("fwd_cell_tile", -1, (0, 16, 4096), (L4, L4, 4, False), True, True),
+        ("fwd_block_bytes", 0, (32768, 262144), (L4, L4, -1, False), True, True),
+        ("bwd_lds_target", 40960, (16384, 65536), (L4, L4, 4, False), True, False),
+        ("diag6_sets", 1, (0,), (L6, L6, 6, True), True, True),
+        ("unrolled_bwd_one", 1, (0,), ({2: 8}, {3: 8}, 1, False), True, False),     # capped at l = 1: one triple
+        ("onepair_mfma_paired", 1, (0,), ({7: 8}, {7: 8}, -1, False), True, False),
+    ]
+    for name, default, others, (tx, ty, maxl, diag), fwd_bits, bwd_bits in cases:
+        r0, g0 = product(tx, ty, maxl, diag, seed=900)
+        try:
+            for v in others:
+                cabi.set_option(name, v)
+                r1, g1 = product(tx, ty, maxl, diag, seed=900)
+                assert same_bits(r0, r1) if fwd_bits else close(r0, r1), (name, v)
+                assert same_bits(g0, g1) if bwd_bits else close(g0, g1), (name, v)
+        finally:
+            cabi.set_option(name, default)

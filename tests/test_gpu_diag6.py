@@ -40,6 +40,8 @@ CASES = [
     (130, {0: 1, 3: 1}, {2: 1, 3: 1}, 6),                              # one channel: 64 cells per wave
     (9, {l: 24 for l in range(7)}, {l: 24 for l in range(7)}, 6),      # two cells per wave, 8 lanes of each idle
     (5, {1: 32, 6: 32}, {6: 32}, 5),                                   # exactly half a wave per cell
+    (3, {1: 64, 4: 64}, {l: 64 for l in range(7)}, 6),                 # every part of y, parts of x missing
+    (2, {l: 64 for l in range(7)}, {l: 64 for l in range(7)}, 3),      # every part of y, product capped low
 ]
 
 

@@ -60,6 +60,11 @@ struct Diag6Args {
 int launch_diag6_fwd_l6(const Diag6Args &a, hipStream_t s);  // product l up to 6
 int launch_diag6_bwd_l6(const Diag6Args &a, hipStream_t s);
 int launch_diag6_bwd_l6_sets(const Diag6Args &a, hipStream_t s);  // every part of y present: fixed sets of l2 per wave
+// operand parts up to l = 4, product up to l = 8
+int launch_diag6_fwd_l8(const Diag6Args &a, hipStream_t s);
+int launch_diag6_bwd_l8(const Diag6Args &a, hipStream_t s);
+int launch_diag6_fwd_l8_packed(const Diag6Args &a, hipStream_t s);
+int launch_diag6_bwd_l8_packed(const Diag6Args &a, hipStream_t s);
 int launch_diag6_fwd_l6_packed(const Diag6Args &a, hipStream_t s);  // several cells per wave (lg_npad < 6)
 int launch_diag6_bwd_l6_packed(const Diag6Args &a, hipStream_t s);
 

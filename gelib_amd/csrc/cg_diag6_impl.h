@@ -162,15 +162,16 @@ __device__ __forceinline__ void fwd_pair(const Diag6Args &a, const float2 (&xv)[
 // Copies the rows of all parts of one operand (the block's cell, or cells, and channel group) into LDS, row l*l + m of
 // the image holding row m of part l, one column per lane.  The rows are dealt to the four waves in turn; every wave
 // requests all of its rows before it writes the first one.
-template <bool PACKED>
+template <bool PACKED, int LOP>
 __device__ __forceinline__ void stage_operand(float2 *img, const FastPart (&parts)[kNP], const WavePos q, int wave, int lane) {
-  constexpr int kPer = (kImgRows + 3) / 4;
+  constexpr int kRows = (LOP + 1) * (LOP + 1);  // rows of the parts l = 0..LOP
+  constexpr int kPer = (kRows + 3) / 4;
   float2 v[kPer];
   static_for<kPer>([&](auto kc) __attribute__((always_inline)) {
     constexpr int k = decltype(kc)::value;
     const int r = 4 * k + wave;  // uniform for the wave
     v[k] = make_float2(0.f, 0.f);
-    static_for<kNP>([&](auto lc) __attribute__((always_inline)) {
+    static_for<LOP + 1>([&](auto lc) __attribute__((always_inline)) {
       constexpr int L = decltype(lc)::value;
       if (r >= L * L && r < (L + 1) * (L + 1) && parts[L].ptr != nullptr)
         v[k] = row_load(cell_row0(parts[L], q.cell) + (long long)(r - L * L) * row_step(parts[L]), lane_offset<PACKED>(parts[L], q));
@@ -179,7 +180,7 @@ __device__ __forceinline__ void stage_operand(float2 *img, const FastPart (&part
   static_for<kPer>([&](auto kc) __attribute__((always_inline)) {
     constexpr int k = decltype(kc)::value;
     const int r = 4 * k + wave;
-    if (r < kImgRows) img[r * 64 + lane] = v[k];
+    if (r < kRows) img[r * 64 + lane] = v[k];
   });
 }
 
@@ -196,20 +197,21 @@ __device__ __forceinline__ void read_rows(float2 (&v)[2 * L + 1], const float2 *
 // for the stores ahead of it.  x stays with the waves (every wave reads each part of it once): a second image would
 // leave room for three blocks per compute unit instead of five, and the store stream needs the waves (measured on
 // L = 6, 64 channels, 131072 cells: no image 18.2 - 20.2 ms, y alone 16.6 - 17.4 ms, both 29.7 ms).
-template <int LCAP, bool PACKED>
+// LOP: the largest l of an operand part the kernel has code for.
+template <int LCAP, bool PACKED, int LOP>
 __global__ void __launch_bounds__(256) diag6_fwd_kernel(const Diag6Args a) {
-  __shared__ float2 yimg[kImgRows * 64];
+  __shared__ float2 yimg[(LOP + 1) * (LOP + 1) * 64];
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const long long w = blockIdx.x;
   const WavePos q = wave_pos(a, w);
-  stage_operand<PACKED>(yimg, a.y, q, wave, lane);
+  stage_operand<PACKED, LOP>(yimg, a.y, q, wave, lane);
   __syncthreads();
-  static_for<kNP>([&](auto l1c) __attribute__((always_inline)) {
+  static_for<LOP + 1>([&](auto l1c) __attribute__((always_inline)) {
     constexpr int L1 = decltype(l1c)::value;
     if (a.x[L1].ptr != nullptr) {
       float2 xv[2 * L1 + 1];
       load_rows<L1, PACKED>(xv, a.x[L1], q);
-      static_for<kNP>([&](auto l2c) __attribute__((always_inline)) {
+      static_for<LOP + 1>([&](auto l2c) __attribute__((always_inline)) {
         constexpr int L2 = decltype(l2c)::value;
         if (((L1 * kNP + L2) & 3) == wave && a.y[L2].ptr != nullptr) {
           float2 yv[2 * L2 + 1];
@@ -335,19 +337,20 @@ __device__ __forceinline__ void store_rows(const float2 *v, int vstride, const F
 // Three waves per SIMD (168 registers) is what the LDS of a block lets a compute unit hold; both forms fit by
 // themselves (the packed one with a smaller row budget).  Forcing the limit with amdgpu_waves_per_eu instead changed the
 // schedule for the worse (twice as many waits).
-template <int LCAP, bool PACKED>
+template <int LCAP, bool PACKED, int LOP>
 __global__ void __launch_bounds__(256) diag6_bwd_kernel(const Diag6Args a) {
-  constexpr int kXRows = 2 * kL6 + 1;
-  __shared__ float2 yimg[kImgRows * 64];
+  constexpr int kXRows = 2 * LOP + 1;
+  constexpr int kYRows = (LOP + 1) * (LOP + 1);
+  __shared__ float2 yimg[kYRows * 64];
   __shared__ float2 xpart[4 * kXRows * 64];  // [wave][row][lane]
   const long long w = blockIdx.x;
   const WavePos q = wave_pos(a, w);
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const bool accumulate = a.accumulate != 0;
   const bool wx = a.want_x != 0, wy = a.want_y != 0;
-  for (int e = threadIdx.x; e < kImgRows * 64; e += 256) yimg[e] = make_float2(0.f, 0.f);
+  for (int e = threadIdx.x; e < kYRows * 64; e += 256) yimg[e] = make_float2(0.f, 0.f);
   __syncthreads();
-  static_for<kNP>([&](auto l1c) __attribute__((always_inline)) {
+  static_for<LOP + 1>([&](auto l1c) __attribute__((always_inline)) {
     constexpr int L1 = decltype(l1c)::value;
     if (a.x[L1].ptr != nullptr) {  // the same for the whole block
       // x is needed for the y-gradient only and y for the x-gradient only; an operand whose gradient is not wanted is
@@ -361,8 +364,8 @@ __global__ void __launch_bounds__(256) diag6_bwd_kernel(const Diag6Args a) {
       }
 #pragma unroll
       for (int m1 = 0; m1 <= 2 * L1; m1++) ax[m1] = make_float2(0.f, 0.f);
-      static_for<kNP>([&](auto l2c) __attribute__((always_inline)) {
-        constexpr int L2 = kL6 - decltype(l2c)::value;  // descending, so that neighbours in l2 run at the same time
+      static_for<LOP + 1>([&](auto l2c) __attribute__((always_inline)) {
+        constexpr int L2 = LOP - decltype(l2c)::value;  // descending, so that neighbours in l2 run at the same time
         if (a.owner[L2] == wave && a.y[L2].ptr != nullptr) {
           float2 yv[2 * L2 + 1];
           if (wx) {
@@ -399,7 +402,7 @@ __global__ void __launch_bounds__(256) diag6_bwd_kernel(const Diag6Args a) {
       __syncthreads();
     }
   });
-  static_for<kNP>([&](auto l2c) __attribute__((always_inline)) {
+  static_for<LOP + 1>([&](auto l2c) __attribute__((always_inline)) {
     constexpr int L2 = decltype(l2c)::value;
     const FastPart YG = a.yg[L2];
     if (wy && a.owner[L2] == wave && YG.ptr != nullptr)
@@ -498,16 +501,16 @@ int launch_diag6_bwd_sets_variant(const Diag6Args &a, hipStream_t s) {
   return GELIB_HIP_OK;
 }
 
-template <int LCAP, bool PACKED>
+template <int LCAP, bool PACKED, int LOP = kL6>
 int launch_diag6_fwd_variant(const Diag6Args &a, hipStream_t s) {
-  hipLaunchKernelGGL((diag6_fwd_kernel<LCAP, PACKED>), dim3((unsigned)a.nwaves), dim3(256), 0, s, a);
+  hipLaunchKernelGGL((diag6_fwd_kernel<LCAP, PACKED, LOP>), dim3((unsigned)a.nwaves), dim3(256), 0, s, a);
   GELIB_HIP_TRY(hipGetLastError());
   return GELIB_HIP_OK;
 }
 
-template <int LCAP, bool PACKED>
+template <int LCAP, bool PACKED, int LOP = kL6>
 int launch_diag6_bwd_variant(const Diag6Args &a, hipStream_t s) {
-  hipLaunchKernelGGL((diag6_bwd_kernel<LCAP, PACKED>), dim3((unsigned)a.nwaves), dim3(256), 0, s, a);
+  hipLaunchKernelGGL((diag6_bwd_kernel<LCAP, PACKED, LOP>), dim3((unsigned)a.nwaves), dim3(256), 0, s, a);
   GELIB_HIP_TRY(hipGetLastError());
   return GELIB_HIP_OK;
 }

@@ -18,6 +18,7 @@ std::mutex g_mutex;
 std::map<int, float *> g_banks;                     // device -> coefficient table
 std::map<std::pair<int, std::vector<int>>, int *> g_offs;  // (device, offsets) -> device copy
 int g_enable = 1;
+int g_l8_enable = 1;    // the kernels for products up to l = 8 of operands up to l = 4: 1 forward, 2 backward too
 int g_sets_enable = 1;  // backward: the kernel with the waves' sets of l2 fixed at compile time, where it applies
 
 int device_bank(const float **out) {
@@ -151,6 +152,15 @@ int make_args(const VecPlan &plan, const std::vector<const gelib_part_desc *> &r
 
 int cg_table_bank(const float **out) { return device_bank(out); }
 
+namespace {
+// no operand part (and no gradient of one) above l = lmax
+bool operands_up_to(const Diag6Args &a, int lmax) {
+  for (int l = lmax + 1; l < kNP; l++)
+    if (a.x[l].ptr || a.y[l].ptr || a.xg[l].ptr || a.yg[l].ptr) return false;
+  return true;
+}
+}  // namespace
+
 int diag6_vec_fwd(const VecPlan &plan, const std::vector<const gelib_part_desc *> &r,
                   const std::vector<const gelib_part_desc *> &x, const std::vector<const gelib_part_desc *> &y,
                   bool accumulate, hipStream_t s, int *used) {
@@ -160,9 +170,13 @@ int diag6_vec_fwd(const VecPlan &plan, const std::vector<const gelib_part_desc *
   bool ok = false;
   int rc = make_args(plan, r, x, y, nullptr, nullptr, true, &a, &lcap, &ok);
   if (rc || !ok) return rc;
-  if (lcap > kL6) return GELIB_HIP_OK;  // kernels are built for products capped at l = 6
+  // kernels are built for products capped at l = 6, and for products up to l = 8 of operands up to l = 4
+  const bool l8 = lcap > kL6;
+  if (l8 && !(lcap <= 8 && operands_up_to(a, 4) && g_l8_enable)) return GELIB_HIP_OK;
   a.accumulate = accumulate ? 1 : 0;
-  if ((rc = a.lg_npad < 6 ? launch_diag6_fwd_l6_packed(a, s) : launch_diag6_fwd_l6(a, s))) return rc;
+  if (l8) rc = a.lg_npad < 6 ? launch_diag6_fwd_l8_packed(a, s) : launch_diag6_fwd_l8(a, s);
+  else rc = a.lg_npad < 6 ? launch_diag6_fwd_l6_packed(a, s) : launch_diag6_fwd_l6(a, s);
+  if (rc) return rc;
   *used = 1;
   return GELIB_HIP_OK;
 }
@@ -178,13 +192,18 @@ int diag6_vec_bwd(const VecPlan &plan, const std::vector<const gelib_part_desc *
   bool ok = false;
   int rc = make_args(plan, g, x, y, xg.empty() ? nullptr : &xg, yg.empty() ? nullptr : &yg, false, &a, &lcap, &ok);
   if (rc || !ok) return rc;
-  if (lcap > kL6) return GELIB_HIP_OK;
+  // (backward, the one-launch kernel for products up to l = 8 is used on request only, diag6_l8 = 2: the wave that owns
+  // y[4] then has the terms of l = 5..8 on top of the largest share, and L=4, 64 channels, 131072 cells takes 16.4 ms
+  // against 14.4 ms for the split at l = 6)
+  const bool l8 = lcap > kL6;
+  if (l8 && !(lcap <= 8 && operands_up_to(a, 4) && g_l8_enable >= 2)) return GELIB_HIP_OK;
   a.accumulate = accumulate ? 1 : 0;
   a.want_x = xg.empty() ? 0 : 1;
   a.want_y = yg.empty() ? 0 : 1;
   bool all_y = true;
   for (int l = 0; l < kNP; l++) all_y = all_y && a.y[l].ptr != nullptr;
-  if (a.lg_npad < 6) rc = launch_diag6_bwd_l6_packed(a, s);
+  if (l8) rc = a.lg_npad < 6 ? launch_diag6_bwd_l8_packed(a, s) : launch_diag6_bwd_l8(a, s);
+  else if (a.lg_npad < 6) rc = launch_diag6_bwd_l6_packed(a, s);
   else if (all_y && g_sets_enable) rc = launch_diag6_bwd_l6_sets(a, s);
   else rc = launch_diag6_bwd_l6(a, s);
   if (rc) return rc;
@@ -218,6 +237,10 @@ int diag6_part(int kind, const long long E[3], const gelib_part_desc *r, const g
 int diag6_set_option(const char *name, int value) {
   if (!std::strcmp(name, "diag6")) {
     g_enable = value;
+    return GELIB_HIP_OK;
+  }
+  if (!std::strcmp(name, "diag6_l8")) {
+    g_l8_enable = value;
     return GELIB_HIP_OK;
   }
   if (!std::strcmp(name, "diag6_sets")) {

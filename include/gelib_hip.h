@@ -246,7 +246,11 @@ int gelib_hip_synchronize(void);
  * apply), "staged_bwd_atomic" (1/0: allow the single-pass backward kernels that add with LDS float atomics; off by
  * default, so that results do not depend on timing), "staged_bwd_pairs" (1/0: the pair-wise one of those),
  * "pairwise_bwd" (one launch of the single-pair kernels per pair of parts: 0 never, 1 for operand l above 7, 2 wherever
- * every pair qualifies), "onepair_mfma" (1/0: the matrix-core form of the single-pair kernel).  Unknown names return
+ * every pair qualifies), "onepair_mfma" (1/0: the matrix-core form of the single-pair kernel), "onepair_mfma_fwd" (1/0:
+ * its forward kernel), "onepair_mfma_paired" (1/0: row numbers taken in pairs when l1 = l2), "unrolled_bwd_one" (1/0: the
+ * backward kernel built for calls with one triple), "diag6_sets" (1/0: the Diag backward kernel with compile-time sets of
+ * l2 per wave), "diag6_l8" (0: Diag products above l = 6 are always split at l = 6; 1: operands up to l = 4 run forward in
+ * one launch of the kernels built for products up to l = 8; 2: backward too).  Unknown names return
  * GELIB_HIP_ERR_ARG.  Options are process-wide.
  * gelib_hip_last_path() tells which kernel family the last call of this thread used
  * (0 = none, 1 = generic, 2 = unrolled small-l kernels, 3 = staged any-l kernels, 4 = lane-per-channel Diag

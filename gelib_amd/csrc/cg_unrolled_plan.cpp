@@ -15,6 +15,7 @@ namespace {
 int g_fwd_block_bytes = 0;           // product bytes one forward block aims to write (0 = by the largest l of the product)
 int g_fwd_lds_bytes = 16 * 1024;     // LDS one forward block may use for its staged operands
 int g_fwd_cell_tile = -1;            // cells per tile of the forward launch (0 = all cells in one tile, -1 = by channels)
+int g_fwd_narrow_decline = 1;  // leave products with at most four channel pairs per block to the any-l forward kernel
 int g_fwd_ti = 0;                    // 0 = widest tile that divides every n1, else force 1 / 2 / 4
 int g_bwd_enable = 1;
 int g_bwd_one_enable = 1; // the backward kernel for calls with one triple
@@ -231,6 +232,15 @@ int run_fwd(bool diag, const std::vector<VecTriple> &triples, const std::vector<
             const std::vector<std::pair<int, int>> &ys, const std::vector<int> &rls, const FastLists &f,
             long long ncells, int offs_add, bool accumulate, hipStream_t s, int *used) {
   *used = 0;
+  // With at most four channel pairs per (l1,l2) block a store instruction of this kernel writes 32 bytes or less per
+  // cell; the any-l forward kernel, whose lanes own whole output rows of a cell, does better there (L=4, measured in
+  // one process: 2 channels 14.5 ms here, 9.3 ms there; 1 channel 23.3 / 12.2; from 4 channels on this kernel wins,
+  // 5.8 / 8.8 ms).
+  if (!diag && g_fwd_narrow_decline) {
+    long long widest = 0;
+    for (auto &t : triples) widest = std::max(widest, (long long)xs[t.xi].second * ys[t.yi].second);
+    if (widest <= 4 && triples.size() > 1) return GELIB_HIP_OK;
+  }
   // one cell's two operand parts must fit the LDS staging area
   for (auto &t : triples) {
     const long long op_bytes = 8LL * ((2 * t.l1 + 1) * (long long)xs[t.xi].second + (2 * t.l2 + 1) * (long long)ys[t.yi].second);
@@ -492,6 +502,10 @@ int unrolled_set_option(const char *name, int value) {
   if (!std::strcmp(name, "fwd_cell_tile")) {
     if (value < -1) return GELIB_HIP_ERR_ARG;
     g_fwd_cell_tile = value;
+    return GELIB_HIP_OK;
+  }
+  if (!std::strcmp(name, "fwd_narrow_decline")) {
+    g_fwd_narrow_decline = value;
     return GELIB_HIP_OK;
   }
   if (!std::strcmp(name, "fwd_tile")) {

@@ -250,7 +250,8 @@ int gelib_hip_synchronize(void);
  * its forward kernel), "onepair_mfma_paired" (1/0: row numbers taken in pairs when l1 = l2), "unrolled_bwd_one" (1/0: the
  * backward kernel built for calls with one triple), "diag6_sets" (1/0: the Diag backward kernel with compile-time sets of
  * l2 per wave), "diag6_l8" (0: Diag products above l = 6 are always split at l = 6; 1: operands up to l = 4 run forward in
- * one launch of the kernels built for products up to l = 8; 2: backward too).  Unknown names return
+ * one launch of the kernels built for products up to l = 8; 2: backward too), "fwd_narrow_decline" (1/0: products with
+ * at most four channel pairs per block go forward on the any-l kernels).  Unknown names return
  * GELIB_HIP_ERR_ARG.  Options are process-wide.
  * gelib_hip_last_path() tells which kernel family the last call of this thread used
  * (0 = none, 1 = generic, 2 = unrolled small-l kernels, 3 = staged any-l kernels, 4 = lane-per-channel Diag

@@ -250,8 +250,11 @@ __device__ __forceinline__ void pair_bwd(const GParts<LCAP> &gp, PairPtr pr, Coe
   for (int m2 = 0; m2 <= 2 * L2; m2++) asm volatile("" : "+v"(ay[m2].x), "+v"(ay[m2].y));
 
   if (WX) {
-    if (!DIAG) group_sum(ax, N2P);
-    if (q.live && valid && (DIAG || j == 0)) {
+    // more than 64 channels of y: a run holds 64 of the lanes that share i, the other runs of the same i add their
+    // sums into the image after it
+    const int N2G = N2P < kWave ? N2P : kWave;
+    if (!DIAG) group_sum(ax, N2G);
+    if (q.live && valid && (DIAG || (j & (N2G - 1)) == 0)) {
       float2 *xa = xacc + q.cell_local * xsize + p.xoff + i;
 #pragma unroll
       for (int m1 = 0; m1 <= 2 * L1; m1++) {

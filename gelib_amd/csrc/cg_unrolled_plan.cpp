@@ -338,7 +338,7 @@ int run_bwd(bool diag, const std::vector<VecTriple> &triples, const std::vector<
     const int n1 = xs[t.xi].second, n2 = ys[t.yi].second;
     if (n1 < 1 || n2 < 1) return GELIB_HIP_OK;
     const int lg1 = ilog2(n1), lg2 = ilog2(n2);
-    if (!diag && lg2 > 6) return GELIB_HIP_OK;
+    if (!diag && lg2 > 8) return GELIB_HIP_OK;
     const int lgu = diag ? lg1 : lg1 + lg2;
     if (lgu > 20) return GELIB_HIP_OK;
     u_min = std::min<int>(u_min, 1 << lgu);

@@ -29,6 +29,8 @@ CASES = [
     (5, {l: 8 for l in range(7)}, {l: 8 for l in range(7)}, 6),
     (6, {0: 2, 3: 4, 5: 8, 6: 2}, {1: 4, 4: 2, 6: 8}, 6),                # operands up to l = 6, mixed channel counts
     (3, {5: 16}, {6: 4}, 5),                                             # one pair with l1, l2 above 4, capped
+    (2, {1: 4}, {1: 128}, -1),                                           # more channels of y than a wave has lanes
+    (2, {0: 2, 1: 3}, {1: 128, 2: 96}, 2),                               # ... and counts that are not powers of two
 ]
 
 

@@ -20,6 +20,7 @@ int g_fwd_ti = 0;                    // 0 = widest tile that divides every n1, e
 int g_bwd_enable = 1;
 int g_bwd_one_enable = 1; // the backward kernel for calls with one triple
 int g_bwd_l6_enable = 1;  // the backward kernel for operands up to l = 6
+int g_bwd_min_runs = 128;           // runs of 64 slots a backward block should have at least, LDS allowing (0: no such rule)
 int g_bwd_lds_target = 40 * 1024;  // LDS bytes per block the backward kernel aims at when it picks the cells per block
 int g_fwd_enable = 1;
 
@@ -380,6 +381,12 @@ int run_bwd(bool diag, const std::vector<VecTriple> &triples, const std::vector<
     for (auto &p : plan->pairs) runs += (((long long)c << p.log2_u) + kWave - 1) / kWave;
     return runs;
   };
+  // few runs per cell (few pairs, few channels): more cells per block, so that the staging of the operands, the two
+  // barriers and the write-out of a block are shared by at least g_bwd_min_runs runs
+  // (as long as the launch keeps eight blocks per compute unit)
+  while (g_bwd_min_runs > 0 && runs_at(cpb) < g_bwd_min_runs && cpb < 64 && ncells / (2 * cpb) >= 2048 &&
+         unrolled_bwd_lds_bytes(a.bank_len, a.xsize, a.ysize, 2 * cpb) <= lds_target)
+    cpb <<= 1;
   while (cpb > 1) {
     const size_t need = unrolled_bwd_lds_bytes(a.bank_len, a.xsize, a.ysize, cpb);
     if (need <= lds_target) break;
@@ -514,6 +521,11 @@ int unrolled_set_option(const char *name, int value) {
   }
   if (!std::strcmp(name, "unrolled_fwd")) {
     g_fwd_enable = value;
+    return GELIB_HIP_OK;
+  }
+  if (!std::strcmp(name, "bwd_min_runs")) {
+    if (value < 0) return GELIB_HIP_ERR_ARG;
+    g_bwd_min_runs = value;
     return GELIB_HIP_OK;
   }
   if (!std::strcmp(name, "bwd_lds_target")) {

@@ -98,11 +98,17 @@ class SO3part_CGproductFn(torch.autograd.Function):
             vec = gb.SO3vec.view
             gb.SO3vec.setCGproduct_back(vec([xg]), vec([yg]), vec([g]), vec([x]), vec([y]))
             return xg, yg, None
-        xg = torch.zeros_like(x)
-        yg = torch.zeros_like(y)
-        _view(xg).add_CGproduct_back0(_view(g), _view(y))
-        _view(yg).add_CGproduct_back1(_view(g), _view(x))
-        return xg, yg, None
+        # a broadcast operand: one gradient per cell from the fused pass (the operand enters as a view with stride 0),
+        # summed over the cells it is shared by (the reference's two calls do that sum inside the kernel, where a
+        # destination of extent 1 is served one cell after the other)
+        gb = backend()
+        lead = g.shape[:-2]
+        vec = gb.SO3vec.view
+        xw, yw = x.expand(*lead, *x.shape[-2:]), y.expand(*lead, *y.shape[-2:])
+        xg = torch.empty(list(lead) + list(x.shape[-2:]), dtype=x.dtype, device=x.device)
+        yg = torch.empty(list(lead) + list(y.shape[-2:]), dtype=y.dtype, device=y.device)
+        gb.SO3vec.setCGproduct_back(vec([xg]), vec([yg]), vec([g]), vec([xw]), vec([yw]))
+        return xg.sum_to_size(x.shape), yg.sum_to_size(y.shape), None
 
 
 class SO3part_DiagCGproductFn(torch.autograd.Function):

@@ -137,12 +137,18 @@ def _product_fn(diag, part_cls=SO3part, prefix="SO3vec"):
             g = gb.SO3vec.view([t.contiguous() for t in gargs])
             xg = gb.SO3vec.view(grads[0:k1])
             yg = gb.SO3vec.view(grads[k1:k1 + k2])
-            if any(t.shape[:-2] != gargs[0].shape[:-2] for t in saved):
-                # a broadcast operand: its gradient is a sum over the broadcast cells, done by the accumulate path
-                for t in grads:
-                    t.zero_()
-                getattr(xg, "add%s_back0" % gb_type)(g, y)
-                getattr(yg, "add%s_back1" % gb_type)(g, x)
+            lead = gargs[0].shape[:-2]
+            if any(t.shape[:-2] != lead for t in saved):
+                # A broadcast operand (batch or grid extent 1 against the product's): its gradient is a sum over the
+                # cells it is shared by.  The fused backward writes one gradient per cell (the operand enters as a
+                # view with stride 0) and torch sums them; left to the part-level calls, that sum runs inside the
+                # shape-agnostic kernels, one cell after the other.
+                wide = [t.expand(*lead, *t.shape[-2:]) for t in saved]
+                full = [torch.empty(list(lead) + list(t.shape[-2:]), dtype=t.dtype, device=t.device) if t.shape[:-2] != lead
+                        else grads[i] for i, t in enumerate(saved)]
+                getattr(gb.SO3vec, "set%s_back" % gb_type)(gb.SO3vec.view(full[0:k1]), gb.SO3vec.view(full[k1:k1 + k2]), g,
+                                                           gb.SO3vec.view(wide[0:k1]), gb.SO3vec.view(wide[k1:k1 + k2]))
+                grads = [f if f is grads[i] else f.sum_to_size(saved[i].shape) for i, f in enumerate(full)]
             else:
                 getattr(gb.SO3vec, "set%s_back" % gb_type)(xg, yg, g, x, y)
             return tuple([None, None, None] + grads)

@@ -203,3 +203,37 @@ def test_linear_layer_runs_on_the_library_kernel_and_matches_matmul(G):
         (torch.view_as_real(ref) * torch.view_as_real(gl)).sum().backward()
         assert torch.allclose(x.parts[l].grad.as_subclass(torch.Tensor).to(torch.complex128), x64.grad, rtol=1e-4, atol=1e-3)
         assert torch.allclose(w.grad.to(torch.complex128), w64.grad, rtol=1e-4, atol=2e-3)
+
+
+@pytest.mark.parametrize("diag", [False, True])
+@pytest.mark.parametrize("shared", ["x", "y"])
+def test_vec_broadcast_operand_gradients(G, diag, shared):
+    """An operand with batch 1 against a batch of 7 (core/Gpart.hpp:168-185): its gradient is the sum over the batch of
+    the gradients the same product gives when the operand is repeated 7 times; the other operand's gradient is the
+    same in both."""
+    B = 7
+    tau = {0: 4, 1: 4, 2: 4} if diag else {0: 3, 1: 2, 2: 2}
+    fn = G.DiagCGproduct if diag else G.CGproduct
+    a1 = G.SO3vec.randn(1, tau, device="cuda")
+    bB = G.SO3vec.randn(B, tau, device="cuda")
+    aB = G.SO3vec()
+    for l, p in a1.parts.items():
+        aB.parts[l] = G.SO3part(p.repeat(B, 1, 1).contiguous())
+    for v in (a1, bB, aB):
+        for p in v.parts.values():
+            p.requires_grad_()
+    args = (lambda a, b: (a, b)) if shared == "x" else (lambda a, b: (b, a))
+    r1 = fn(*args(a1, bB), 3)
+    rB = fn(*args(aB, bB), 3)
+    ws = [torch.randn_like(torch.view_as_real(p)) for p in r1.parts.values()]
+    loss = lambda r: sum((torch.view_as_real(p) * w).sum() for p, w in zip(r.parts.values(), ws))
+    for p, q in zip(r1.parts.values(), rB.parts.values()):
+        assert torch.equal(torch.view_as_real(p), torch.view_as_real(q))
+    g_a1 = torch.autograd.grad(loss(r1), list(a1.parts.values()) + list(bB.parts.values()))
+    g_aB = torch.autograd.grad(loss(rB), list(aB.parts.values()) + list(bB.parts.values()))
+    k = len(a1.parts)
+    for got, rep in zip(g_a1[:k], g_aB[:k]):
+        assert got.shape[0] == 1
+        assert torch.allclose(got, rep.sum(0, keepdim=True), rtol=1e-4, atol=1e-4)
+    for got, rep in zip(g_a1[k:], g_aB[k:]):
+        assert torch.allclose(got, rep, rtol=1e-5, atol=1e-5)

@@ -90,7 +90,9 @@ __device__ __forceinline__ int pick_int(const int (&arr)[N], int i) {
 }
 
 // ti: channels of the first operand handled per thread (1, 2 or 4); must divide every n1.
-int launch_unrolled_fwd(const FwdArgs &a, bool diag, int ti, int lcap, int nblocks, size_t lds_bytes, hipStream_t s);
+// lop: largest l of an operand (above kLT: the kernel for l up to kLTMax -- unrolled_fwd_takes says when it exists)
+bool unrolled_fwd_takes(bool diag, int ti, int lcap, int lop);
+int launch_unrolled_fwd(const FwdArgs &a, bool diag, int ti, int lcap, int lop, int nblocks, size_t lds_bytes, hipStream_t s);
 // lcap: largest l present in the gradient; lop: largest l of an operand (above kLT: the kernel for l up to kLTMax, which
 // exists for CGproduct with power-of-two channel counts and lcap <= kLTMax only -- unrolled_bwd_takes says so)
 bool unrolled_bwd_takes(bool diag, bool padded, int lcap, int lop);

@@ -128,13 +128,14 @@ __device__ __forceinline__ void stage_part(float2 *dst, const FastPart P, int ro
   }
 }
 
-template <int LCAP, bool DIAG, int TI>
+// LT: largest operand l of the pairs the kernel has code for.
+template <int LCAP, bool DIAG, int TI, int LT>
 __global__ void __launch_bounds__(kBlock) unrolled_fwd_kernel(const FwdArgs a) {
   extern __shared__ float2 lds_ops[];
   int pidx = 0, first = 0;
   const int per_tile = a.blocks_per_tile;
   const int tile_idx = (int)blockIdx.x / per_tile, in_tile = (int)blockIdx.x - tile_idx * per_tile;
-  static_for<kMaxPairs>([&](auto k) __attribute__((always_inline)) {
+  static_for<(LT + 1) * (LT + 1)>([&](auto k) __attribute__((always_inline)) {
     if (k.value > 0 && k.value < a.npairs && in_tile >= a.first_block[k.value]) {
       pidx = k.value;
       first = a.first_block[k.value];
@@ -161,7 +162,7 @@ __global__ void __launch_bounds__(kBlock) unrolled_fwd_kernel(const FwdArgs a) {
   const int U = DIAG ? n1 : (n1 / TI) * n2;
   const int slots = ncell * U;
   const CoeffPtr C = (CoeffPtr)(a.bank + p->cg_base);
-  const int code = l1 * (kLT + 1) + l2;
+  const int code = l1 * (kLTMax + 1) + l2;
   for (int w0 = 0; w0 < slots; w0 += kBlock) {
     const int w = w0 + threadIdx.x;
     const bool live = w < slots;
@@ -170,10 +171,14 @@ __global__ void __launch_bounds__(kBlock) unrolled_fwd_kernel(const FwdArgs a) {
     const int u = wc - dc * U;
     const long long cell = cell0 + dc;
     switch (code) {
-#define GELIB_CASE(A, B) \
-  case A * (kLT + 1) + B: pair_fwd<A, B, LCAP, TI, DIAG>(rp_all, p, C, xs, ys, offs_add, accumulate, cell, dc, u, live); break;
-#define GELIB_ROW(A) GELIB_CASE(A, 0) GELIB_CASE(A, 1) GELIB_CASE(A, 2) GELIB_CASE(A, 3) GELIB_CASE(A, 4)
-      GELIB_ROW(0) GELIB_ROW(1) GELIB_ROW(2) GELIB_ROW(3) GELIB_ROW(4)
+#define GELIB_CASE(A, B)                                                                                      \
+  case A * (kLTMax + 1) + B:                                                                                  \
+    if constexpr (A <= LT && B <= LT)                                                                         \
+      pair_fwd<A, B, LCAP, TI, DIAG>(rp_all, p, C, xs, ys, offs_add, accumulate, cell, dc, u, live);          \
+    break;
+#define GELIB_ROW(A) \
+  GELIB_CASE(A, 0) GELIB_CASE(A, 1) GELIB_CASE(A, 2) GELIB_CASE(A, 3) GELIB_CASE(A, 4) GELIB_CASE(A, 5) GELIB_CASE(A, 6)
+      GELIB_ROW(0) GELIB_ROW(1) GELIB_ROW(2) GELIB_ROW(3) GELIB_ROW(4) GELIB_ROW(5) GELIB_ROW(6)
 #undef GELIB_ROW
 #undef GELIB_CASE
       default: break;
@@ -181,10 +186,10 @@ __global__ void __launch_bounds__(kBlock) unrolled_fwd_kernel(const FwdArgs a) {
   }
 }
 
-template <int LCAP, bool DIAG, int TI>
+template <int LCAP, bool DIAG, int TI, int LT = kLT>
 int launch_fwd_variant(const FwdArgs &a, int nblocks, size_t lds_bytes, hipStream_t s) {
-  static_assert(kLT == 4, "the case table above lists l1, l2 = 0..4");
-  hipLaunchKernelGGL((unrolled_fwd_kernel<LCAP, DIAG, TI>), dim3(nblocks), dim3(kBlock), lds_bytes, s, a);
+  static_assert(kLTMax == 6 && LT <= kLTMax, "the case table above lists l1, l2 = 0..6");
+  hipLaunchKernelGGL((unrolled_fwd_kernel<LCAP, DIAG, TI, LT>), dim3(nblocks), dim3(kBlock), lds_bytes, s, a);
   GELIB_HIP_TRY(hipGetLastError());
   return GELIB_HIP_OK;
 }

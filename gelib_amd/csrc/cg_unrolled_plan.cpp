@@ -23,6 +23,7 @@ int g_bwd_l6_enable = 1;  // the backward kernel for operands up to l = 6
 int g_bwd_min_runs = 128;           // runs of 64 slots a backward block should have at least, LDS allowing (0: no such rule)
 int g_bwd_lds_target = 40 * 1024;  // LDS bytes per block the backward kernel aims at when it picks the cells per block
 int g_fwd_enable = 1;
+int g_fwd_l6_enable = 1;  // the forward kernel for operands up to l = 6
 
 struct DevicePlan {
   std::vector<PairRec> pairs;
@@ -272,6 +273,10 @@ int run_fwd(bool diag, const std::vector<VecTriple> &triples, const std::vector<
     }
     if (g_fwd_ti == 1 || g_fwd_ti == 2 || g_fwd_ti == 4) ti = std::min(ti, g_fwd_ti);
   }
+  int lcap_all = 0, lop = 0;
+  for (auto &t : triples) lcap_all = std::max(lcap_all, t.l), lop = std::max(lop, std::max(t.l1, t.l2));
+  if (lop > kLT && ti == 4) ti = 2;  // the kernel for operands above kLT is built for two channels per thread
+  if (!unrolled_fwd_takes(diag, ti, lcap_all, lop) || (lop > kLT && !g_fwd_l6_enable)) return GELIB_HIP_OK;
   long long nblocks = 0;
   size_t lds_bytes = 0;
   int lcap = 0;
@@ -315,7 +320,7 @@ int run_fwd(bool diag, const std::vector<VecTriple> &triples, const std::vector<
   a.blocks_per_tile = (int)nblocks;
   nblocks *= (ncells + tile - 1) / tile;
   if (nblocks > 0x7fffffffLL) return GELIB_HIP_ERR_ARG;
-  rc = launch_unrolled_fwd(a, diag, ti, lcap, (int)nblocks, lds_bytes, s);
+  rc = launch_unrolled_fwd(a, diag, ti, lcap, lop, (int)nblocks, lds_bytes, s);
   if (rc) return rc;
   *used = 1;
   return GELIB_HIP_OK;
@@ -452,12 +457,12 @@ int unrolled_vec_fwd(const VecPlan &plan, const std::vector<const gelib_part_des
   *used = 0;
   if (!g_fwd_enable) return GELIB_HIP_OK;
   if (x.size() > (size_t)kFastIn || y.size() > (size_t)kFastIn || r.size() > (size_t)kFastOut) return GELIB_HIP_OK;
-  for (auto &t : plan.triples)
-    if (t.l1 > kLT || t.l2 > kLT) return GELIB_HIP_OK;
   for (auto *d : x)
-    if ((d->dims[3] - 1) / 2 > kLT) return GELIB_HIP_OK;
+    if ((d->dims[3] - 1) / 2 > kLTMax) return GELIB_HIP_OK;
   for (auto *d : y)
-    if ((d->dims[3] - 1) / 2 > kLT) return GELIB_HIP_OK;
+    if ((d->dims[3] - 1) / 2 > kLTMax) return GELIB_HIP_OK;
+  for (auto *d : r)
+    if ((d->dims[3] - 1) / 2 > 2 * kLTMax) return GELIB_HIP_OK;
   FastLists f;
   std::vector<std::pair<int, int>> xs, ys, rs;
   if (!lists_to_fast(x, plan.E, false, &f.x, &xs) || !lists_to_fast(y, plan.E, false, &f.y, &ys) ||
@@ -531,6 +536,10 @@ int unrolled_set_option(const char *name, int value) {
   if (!std::strcmp(name, "bwd_lds_target")) {
     if (value < 1024 || value > 150 * 1024) return GELIB_HIP_ERR_ARG;
     g_bwd_lds_target = value;
+    return GELIB_HIP_OK;
+  }
+  if (!std::strcmp(name, "unrolled_fwd_l6")) {
+    g_fwd_l6_enable = value;
     return GELIB_HIP_OK;
   }
   if (!std::strcmp(name, "unrolled_bwd_one")) {

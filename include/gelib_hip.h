@@ -240,7 +240,7 @@ int gelib_hip_synchronize(void);
  * "staged_fwd" / "staged_bwd" / "diag6" / "onepair" (1/0: use the family), "fwd_block_bytes", "fwd_lds_bytes", "fwd_tile",
  * "fwd_cell_tile" (cells per tile of the unrolled forward launch, 0 = one tile, -1 = chosen by the channel counts, the
  * default), "bwd_lds_target" (LDS bytes per block the unrolled backward kernels aim at when they choose their cells per
- * block), "bwd_min_runs" (runs of 64 lane slots such a block should have at least, 0 = no such rule), "unrolled_bwd_l6" (1/0: the backward kernel for operands up to l = 6),
+ * block), "bwd_min_runs" (runs of 64 lane slots such a block should have at least, 0 = no such rule), "unrolled_bwd_l6" / "unrolled_fwd_l6" (1/0: the backward / forward kernel for operands up to l = 6),
  * "staged_fwd_tile" (1, 2, 4), "staged_fwd_threads", "staged_fwd_coeffs_lds" (1/0), "staged_fwd_lds_target",
  * "staged_bwd_lds_target", "staged_bwd_threads" (256, 512, 1024), "staged_bwd_stripes" (0 never, otherwise wherever they
  * apply), "staged_bwd_atomic" (1/0: allow the single-pass backward kernels that add with LDS float atomics; off by

@@ -32,6 +32,7 @@ def cabi(request):
     c.set_option("onepair_mfma", 0)
     c.set_option("onepair_mfma_fwd", 0)
     c.set_option("unrolled_bwd_l6", 0)   # the unrolled backward kernel for operands up to l = 6 would take some too
+    c.set_option("unrolled_fwd_l6", 0)   # ... and so would the forward kernel for operands up to l = 6
     c.set_option("pairwise_bwd", 0)
     c.set_option("staged_bwd_stripes", 1 if request.param == "striped" else 0)
     c.set_option("staged_bwd_atomic", 1)   # the other two forms (and what the striped one leaves) add with LDS float atomics
@@ -42,6 +43,7 @@ def cabi(request):
     c.set_option("onepair_mfma", 1)
     c.set_option("onepair_mfma_fwd", 1)
     c.set_option("unrolled_bwd_l6", 1)
+    c.set_option("unrolled_fwd_l6", 1)
     c.set_option("pairwise_bwd", 1)
     c.set_option("staged_bwd_threads", 0)
     c.set_option("staged_bwd_stripes", 1)

@@ -416,7 +416,7 @@ int run_bwd(bool diag, const std::vector<VecTriple> &triples, const std::vector<
 
 int unrolled_part(int kind, const PartOp &op, bool accumulate, hipStream_t s, int *used) {
   *used = 0;
-  if (op.l1 > kLT || op.l2 > kLT) return GELIB_HIP_OK;
+  if (op.l1 > kLTMax || op.l2 > kLTMax) return GELIB_HIP_OK;  // (above kLT: run_fwd / run_bwd say what they take)
   if (kind == 0 && !g_fwd_enable) return GELIB_HIP_OK;
   if (kind != 0 && !g_bwd_enable) return GELIB_HIP_OK;
   FastLists f;

@@ -13,6 +13,7 @@ int launch_unrolled_bwd_cg8_pad(const BwdArgs &a, int nblocks, size_t lds_bytes,
 int launch_unrolled_bwd_diag4_pad(const BwdArgs &a, int nblocks, size_t lds_bytes, hipStream_t s);
 int launch_unrolled_bwd_diag8_pad(const BwdArgs &a, int nblocks, size_t lds_bytes, hipStream_t s);
 int launch_unrolled_bwd_cg6_l6(const BwdArgs &a, int nblocks, size_t lds_bytes, hipStream_t s);
+int launch_unrolled_bwd_cg6_l6_pad(const BwdArgs &a, int nblocks, size_t lds_bytes, hipStream_t s);
 int launch_unrolled_bwd_one(const BwdArgs &a, int nblocks, size_t lds_bytes, hipStream_t s);
 
 size_t unrolled_bwd_lds_bytes(int bank_len, int xsize, int ysize, int cells_per_block) {
@@ -22,11 +23,12 @@ size_t unrolled_bwd_lds_bytes(int bank_len, int xsize, int ysize, int cells_per_
 }
 
 // Operands up to l = 4: every product (l up to 8), Diag or not, any channel counts.  Operands up to l = 6: CGproduct
-// capped at l = 6 with power-of-two channel counts (one instantiation, five minutes of compile time; a kernel for the
-// uncapped product, l up to 12, is not built).
+// capped at l = 6 (two instantiations, power-of-two channel counts and others, five minutes of compile time each; a
+// kernel for the uncapped product, l up to 12, is not built).
 bool unrolled_bwd_takes(bool diag, bool padded, int lcap, int lop) {
+  (void)padded;
   if (lop <= kLT) return lcap <= 2 * kLT;
-  return lop <= kLTMax && !diag && !padded && lcap <= kLTMax;
+  return lop <= kLTMax && !diag && lcap <= kLTMax;
 }
 
 int unrolled_bwd_cap(int lcap, int lop) {
@@ -38,7 +40,9 @@ int unrolled_bwd_cap(int lcap, int lop) {
 // lcap: largest l present in the gradient; code for l above 4 is left out when the product is capped there
 int launch_unrolled_bwd(const BwdArgs &a, bool diag, int lcap, int lop, int nblocks, size_t lds_bytes, hipStream_t s) {
   if (nblocks <= 0) return GELIB_HIP_OK;
-  if (lop > kLT) return launch_unrolled_bwd_cg6_l6(a, nblocks, lds_bytes, s);
+  if (lop > kLT)
+    return a.padded ? launch_unrolled_bwd_cg6_l6_pad(a, nblocks, lds_bytes, s)
+                    : launch_unrolled_bwd_cg6_l6(a, nblocks, lds_bytes, s);
   if (a.only_dl >= 0 && !diag && !a.padded) return launch_unrolled_bwd_one(a, nblocks, lds_bytes, s);
   if (a.padded) {
     if (diag) return lcap <= kLT ? launch_unrolled_bwd_diag4_pad(a, nblocks, lds_bytes, s)

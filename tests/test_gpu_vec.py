@@ -127,6 +127,14 @@ def test_channel_counts_that_are_not_powers_of_two(cabi, case, diag):
         cabi.set_option("diag6", 1)
 
 
+def test_channel_counts_that_are_not_powers_of_two_above_l4(cabi):
+    """CGproduct of operands up to l = 6, capped at l = 6: forward on the unrolled kernel built for them (even channel
+    counts of the first operand), backward on its instantiation with padded lane slots."""
+    assert run_vec(cabi, 4, {2: 6, 5: 2}, {1: 12, 6: 5}, 6, False, seed=510, force_generic=False) == (2, 2)
+    assert run_vec(cabi, 3, {l: 6 for l in range(7)}, {l: 6 for l in range(7)}, 6, False, seed=511,
+                   force_generic=False) == (2, 2)
+
+
 @pytest.mark.parametrize("case", [
     (3, {l: 1 for l in range(17)}, {0: 2}, -1),      # 17 operand parts: more than the fused kernels' part lists hold
     (2, {32: 1}, {32: 1}, -1),                        # 65 product parts, l = 0..64

@@ -270,6 +270,9 @@ int run_fwd(bool diag, const std::vector<VecTriple> &triples, const std::vector<
       // four channels of x per thread leave n1/4 * n2 slots per cell: with few channels the pieces one store
       // instruction writes per cell get too short (8 channels: 4.77 -> 4.34 ms, 4 channels: 8.3 -> 6.9 ms with two)
       if (p.n1 < 16 && ti > 2) ti = 2;
+      // ... and so do few channels of the second operand (features x single-channel harmonics: 16 x 1 channels,
+      // L=4 x L=2, B=1M 9.85 -> 8.5 ms; 32 x 1 channels 8.6 -> 7.5 ms)
+      if (ti > 2 && (p.n1 / ti) * p.n2 < 16) ti = 2;
     }
     if (g_fwd_ti == 1 || g_fwd_ti == 2 || g_fwd_ti == 4) ti = std::min(ti, g_fwd_ti);
   }

@@ -91,6 +91,17 @@ class SO3vec:
     def CGproduct(self, y, maxl=-1):
         xparts = list(self.parts.values())
         yparts = list(y.parts.values())
+        one = _one_channel_side(xparts, yparts)
+        if one is not None:
+            # features times a one-channel vector (spherical harmonics of one direction per sample, say): block channel
+            # i*N2 + j has N2 = 1 (or N1 = 1), so the product is the DiagCGproduct with the one channel repeated, and the
+            # lane-per-channel kernels run it about twice as fast as the general ones run 16 x 1 channels.  The repeat is
+            # a torch op: its backward sums the gradient over the channels.
+            wide, narrow = (xparts, yparts) if one == "y" else (yparts, xparts)
+            n = wide[0].size(-1)
+            rep = [p.expand(*p.shape[:-1], n).contiguous() for p in narrow]
+            xs, ys = (wide, rep) if one == "y" else (rep, wide)
+            return SO3vec(*SO3vec_DiagCGproductFn.apply(len(xs), len(ys), maxl, *(xs + ys)))
         return SO3vec(*SO3vec_CGproductFn.apply(len(xparts), len(yparts), maxl, *(xparts + yparts)))
 
     def DiagCGproduct(self, y, maxl=-1):
@@ -100,6 +111,19 @@ class SO3vec:
 
     def __repr__(self):
         return "<SO3vec of type %s [b=%d]>" % (self.tau(), self.getb())
+
+
+def _one_channel_side(xparts, yparts):
+    """'y' if every part of y has one channel and the parts of x share one channel count above one (or 'x' the other
+    way round), else None."""
+    def side(wide, narrow):
+        n = wide[0].size(-1)
+        return n > 1 and all(p.size(-1) == n for p in wide) and all(p.size(-1) == 1 for p in narrow)
+    if side(xparts, yparts):
+        return "y"
+    if side(yparts, xparts):
+        return "x"
+    return None
 
 
 def _product_fn(diag, part_cls=SO3part, prefix="SO3vec"):

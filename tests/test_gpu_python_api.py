@@ -237,3 +237,31 @@ def test_vec_broadcast_operand_gradients(G, diag, shared):
         assert torch.allclose(got, rep.sum(0, keepdim=True), rtol=1e-4, atol=1e-4)
     for got, rep in zip(g_a1[k:], g_aB[k:]):
         assert torch.allclose(got, rep, rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize("narrow", ["x", "y"])
+def test_vec_product_with_a_one_channel_operand(G, narrow):
+    """CGproduct of features with a one-channel vector runs as the DiagCGproduct with the one channel repeated: the same
+    product (against the oracle's CGproduct loops) and the same gradients (against the general kernels, called through
+    the autograd function directly)."""
+    from gelib_amd.SO3vec import SO3vec_CGproductFn
+    B = 6
+    wide = G.SO3vec.randn(B, {0: 16, 1: 16, 2: 16, 3: 16}, device="cuda")
+    thin = G.SO3vec.randn(B, {0: 1, 1: 1, 2: 1}, device="cuda")
+    x, y = (thin, wide) if narrow == "x" else (wide, thin)
+    for p in list(x.parts.values()) + list(y.parts.values()):
+        p.requires_grad_()
+    r = G.CGproduct(x, y, 3)
+    xp, yp = list(x.parts.values()), list(y.parts.values())
+    want = ora.vec_fwd([U.host(p.detach()) for p in xp], [U.host(p.detach()) for p in yp], 3)
+    for a, b in zip(r.parts.values(), want):
+        assert a.shape == b.shape
+        assert U.gate_excess(U.host(a.detach()), b) <= 1.0
+    ref = SO3vec_CGproductFn.apply(len(xp), len(yp), 3, *(xp + yp))
+    ws = [torch.randn_like(torch.view_as_real(p)) for p in ref]
+    loss = lambda parts: sum((torch.view_as_real(p) * w).sum() for p, w in zip(parts, ws))
+    g1 = torch.autograd.grad(loss(list(r.parts.values())), xp + yp)
+    g2 = torch.autograd.grad(loss(list(ref)), xp + yp)
+    for a, b in zip(g1, g2):
+        assert a.shape == b.shape
+        assert torch.allclose(a, b, rtol=1e-4, atol=1e-4)

@@ -15,6 +15,9 @@ PKG = os.path.join(ROOT, "gelib_amd")
 ext = ce.CppExtension(
     name="gelib_amd.gelib_base",
     sources=[os.path.join(HERE, "gelib_base.cpp")],
+    # the class mirror is header-only: the module must be rebuilt when any of these changes
+    depends=[os.path.join(ROOT, "include", "gelib", "GElib.hpp"), os.path.join(ROOT, "include", "gelib", "cnine_min.hpp"),
+             os.path.join(ROOT, "include", "gelib_hip.h")],
     include_dirs=[os.path.join(ROOT, "include"), "/opt/rocm/include"],
     define_macros=[("__HIP_PLATFORM_AMD__", "1"), ("USE_ROCM", "1")],
     extra_compile_args=["-O2", "-g0", "-std=c++17", "-Wno-unused-function"],
@@ -24,6 +27,6 @@ ext = ce.CppExtension(
 )
 
 setup(name="gelib_amd_base", version="0.1", ext_modules=[ext], cmdclass={"build_ext": ce.BuildExtension.with_options(use_ninja=False)},
-      script_args=["build_ext", "--inplace", "--build-temp", os.path.join(PKG, "csrc", "build", "pybind"),
+      script_args=["build_ext", "--inplace", "--force", "--build-temp", os.path.join(PKG, "csrc", "build", "pybind"),
                    "--build-lib", os.path.join(PKG, "csrc", "build", "pybind_lib")],
       packages=[])

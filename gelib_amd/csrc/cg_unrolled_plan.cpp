@@ -146,6 +146,9 @@ int get_plan(bool diag, const std::vector<VecTriple> &triples, const std::vector
   for (auto &v : ys) key.push_back(v.first), key.push_back(v.second);
   for (int l : rls) key.push_back(l);
   for (auto &t : triples) key.push_back(t.ri), key.push_back(t.offs);
+  // a PairRec has room for kMaxDl values of l per pair; callers decline wider products before they come here
+  for (auto &t : triples)
+    if (t.l - std::abs(t.l1 - t.l2) < 0 || t.l - std::abs(t.l1 - t.l2) >= kMaxDl) return GELIB_HIP_ERR_UNSUPPORTED;
   std::lock_guard<std::mutex> lock(g_plan_mutex);
   auto it = g_plans.find(key);
   if (it != g_plans.end()) {
@@ -248,6 +251,27 @@ int run_fwd(bool diag, const std::vector<VecTriple> &triples, const std::vector<
     const long long op_bytes = 8LL * ((2 * t.l1 + 1) * (long long)xs[t.xi].second + (2 * t.l2 + 1) * (long long)ys[t.yi].second);
     if (op_bytes > g_fwd_lds_bytes) return GELIB_HIP_OK;
   }
+  // which kernel would run is decided from the type alone, before any table is built: a product this family declines
+  // (e.g. operands of l = 6 uncapped) must not cost a device allocation, and its l range does not fit a PairRec
+  int ti = 1;
+  if (!diag) {
+    ti = 4;
+    for (auto &t : triples) {
+      const int n1 = xs[t.xi].second, n2 = ys[t.yi].second;
+      while (ti > 1 && n1 % ti) ti >>= 1;
+      // four channels of x per thread leave n1/4 * n2 slots per cell: with few channels the pieces one store
+      // instruction writes per cell get too short (8 channels: 4.77 -> 4.34 ms, 4 channels: 8.3 -> 6.9 ms with two)
+      if (n1 < 16 && ti > 2) ti = 2;
+      // ... and so do few channels of the second operand (features x single-channel harmonics: 16 x 1 channels,
+      // L=4 x L=2, B=1M 9.85 -> 8.5 ms; 32 x 1 channels 8.6 -> 7.5 ms)
+      if (ti > 2 && (n1 / ti) * n2 < 16) ti = 2;
+    }
+    if (g_fwd_ti == 1 || g_fwd_ti == 2 || g_fwd_ti == 4) ti = std::min(ti, g_fwd_ti);
+  }
+  int lcap_all = 0, lop = 0;
+  for (auto &t : triples) lcap_all = std::max(lcap_all, t.l), lop = std::max(lop, std::max(t.l1, t.l2));
+  if (lop > kLT && ti == 4) ti = 2;  // the kernel for operands above kLT is built for two channels per thread
+  if (!unrolled_fwd_takes(diag, ti, lcap_all, lop) || (lop > kLT && !g_fwd_l6_enable)) return GELIB_HIP_OK;
   const DevicePlan *plan = nullptr;
   int rc = get_plan(diag, triples, xs, ys, rls, &plan);
   if (rc) return rc;
@@ -262,24 +286,6 @@ int run_fwd(bool diag, const std::vector<VecTriple> &triples, const std::vector<
   a.npairs = (int)plan->pairs.size();
   a.offs_add = offs_add;
   a.accumulate = accumulate ? 1 : 0;
-  int ti = 1;
-  if (!diag) {
-    ti = 4;
-    for (auto &p : plan->pairs) {
-      while (ti > 1 && p.n1 % ti) ti >>= 1;
-      // four channels of x per thread leave n1/4 * n2 slots per cell: with few channels the pieces one store
-      // instruction writes per cell get too short (8 channels: 4.77 -> 4.34 ms, 4 channels: 8.3 -> 6.9 ms with two)
-      if (p.n1 < 16 && ti > 2) ti = 2;
-      // ... and so do few channels of the second operand (features x single-channel harmonics: 16 x 1 channels,
-      // L=4 x L=2, B=1M 9.85 -> 8.5 ms; 32 x 1 channels 8.6 -> 7.5 ms)
-      if (ti > 2 && (p.n1 / ti) * p.n2 < 16) ti = 2;
-    }
-    if (g_fwd_ti == 1 || g_fwd_ti == 2 || g_fwd_ti == 4) ti = std::min(ti, g_fwd_ti);
-  }
-  int lcap_all = 0, lop = 0;
-  for (auto &t : triples) lcap_all = std::max(lcap_all, t.l), lop = std::max(lop, std::max(t.l1, t.l2));
-  if (lop > kLT && ti == 4) ti = 2;  // the kernel for operands above kLT is built for two channels per thread
-  if (!unrolled_fwd_takes(diag, ti, lcap_all, lop) || (lop > kLT && !g_fwd_l6_enable)) return GELIB_HIP_OK;
   long long nblocks = 0;
   size_t lds_bytes = 0;
   int lcap = 0;

@@ -89,26 +89,15 @@ class SO3part_CGproductFn(torch.autograd.Function):
     def backward(ctx, g):
         x, y = ctx.saved_tensors
         g = g.contiguous()
-        if x.shape[:-2] == g.shape[:-2] and y.shape[:-2] == g.shape[:-2]:
-            # no broadcast operand: both gradients from ONE pass over g (the vector-level backward on one-part
-            # vectors); the reference makes the two calls below, each of which reads g
-            gb = backend()
-            xg = torch.empty_like(x)
-            yg = torch.empty_like(y)
-            vec = gb.SO3vec.view
-            gb.SO3vec.setCGproduct_back(vec([xg]), vec([yg]), vec([g]), vec([x]), vec([y]))
-            return xg, yg, None
-        # a broadcast operand: one gradient per cell from the fused pass (the operand enters as a view with stride 0),
-        # summed over the cells it is shared by (the reference's two calls do that sum inside the kernel, where a
-        # destination of extent 1 is served one cell after the other)
+        # both gradients from ONE pass over g (the vector-level backward on one-part vectors); the reference makes two
+        # calls, each of which reads g.  An operand shared by the batch (extent 1) gets the sum over the batch, formed
+        # inside the library in a fixed order.
         gb = backend()
-        lead = g.shape[:-2]
+        xg = torch.empty_like(x, memory_format=torch.contiguous_format)
+        yg = torch.empty_like(y, memory_format=torch.contiguous_format)
         vec = gb.SO3vec.view
-        xw, yw = x.expand(*lead, *x.shape[-2:]), y.expand(*lead, *y.shape[-2:])
-        xg = torch.empty(list(lead) + list(x.shape[-2:]), dtype=x.dtype, device=x.device)
-        yg = torch.empty(list(lead) + list(y.shape[-2:]), dtype=y.dtype, device=y.device)
-        gb.SO3vec.setCGproduct_back(vec([xg]), vec([yg]), vec([g]), vec([xw]), vec([yw]))
-        return xg.sum_to_size(x.shape), yg.sum_to_size(y.shape), None
+        gb.SO3vec.setCGproduct_back(vec([xg]), vec([yg]), vec([g]), vec([x]), vec([y]))
+        return xg, yg, None
 
 
 class SO3part_DiagCGproductFn(torch.autograd.Function):

@@ -155,18 +155,17 @@ def _product_fn(diag, part_cls=SO3part, prefix="SO3vec"):
             gb = backend()
             k1, k2 = ctx.k1, ctx.k2
             saved = ctx.saved_tensors
-            grads = [torch.empty_like(t) for t in saved]
+            grads = [torch.empty_like(t, memory_format=torch.contiguous_format) for t in saved]
             x = gb.SO3vec.view(list(saved[0:k1]))
             y = gb.SO3vec.view(list(saved[k1:k1 + k2]))
             g = gb.SO3vec.view([t.contiguous() for t in gargs])
             xg = gb.SO3vec.view(grads[0:k1])
             yg = gb.SO3vec.view(grads[k1:k1 + k2])
             lead = gargs[0].shape[:-2]
-            if any(t.shape[:-2] != lead for t in saved):
-                # A broadcast operand (batch or grid extent 1 against the product's): its gradient is a sum over the
-                # cells it is shared by.  The fused backward writes one gradient per cell (the operand enters as a
-                # view with stride 0) and torch sums them; left to the part-level calls, that sum runs inside the
-                # shape-agnostic kernels, one cell after the other.
+            if any(t.shape[:-2] != lead for t in saved) and (len(lead) > 3 or any(t.dim() not in (3, len(lead) + 2) for t in saved)):
+                # Broadcast operands among more than two grid dimensions: the library sees those fused into one, which
+                # an extent of 1 inside them prevents.  The operand enters as a view with stride 0, the fused backward
+                # writes one gradient per cell and torch sums them over the cells the operand is shared by.
                 wide = [t.expand(*lead, *t.shape[-2:]) for t in saved]
                 full = [torch.empty(list(lead) + list(t.shape[-2:]), dtype=t.dtype, device=t.device) if t.shape[:-2] != lead
                         else grads[i] for i, t in enumerate(saved)]
@@ -174,6 +173,8 @@ def _product_fn(diag, part_cls=SO3part, prefix="SO3vec"):
                                                            gb.SO3vec.view(wide[0:k1]), gb.SO3vec.view(wide[k1:k1 + k2]))
                 grads = [f if f is grads[i] else f.sum_to_size(saved[i].shape) for i, f in enumerate(full)]
             else:
+                # a gradient shaped like an operand that is shared by the batch or the grid (extent 1 there) is summed
+                # over the cells inside the library, in a fixed order
                 getattr(gb.SO3vec, "set%s_back" % gb_type)(xg, yg, g, x, y)
             return tuple([None, None, None] + grads)
 

@@ -6,6 +6,8 @@
 #include <algorithm>
 #include <cstdio>
 #include <cstring>
+#include <functional>
+#include <map>
 #include <mutex>
 #include <string>
 #include <vector>
@@ -74,6 +76,16 @@ bool known_range(const char *p, const char *end, int dev) {
   for (int i = 0; i < g_known_count; i++)
     if (g_known[i].device == dev && p >= g_known[i].base && end <= g_known[i].base + g_known[i].size) return true;
   return false;
+}
+
+// base == nullptr: forget everything; otherwise the entries that start at base (the allocation is being freed)
+void forget_ranges(const void *base) {
+  std::lock_guard<std::mutex> lock(g_known_mutex);
+  int k = 0;
+  for (int i = 0; i < g_known_count; i++)
+    if (base && g_known[i].base != (const char *)base) g_known[k++] = g_known[i];
+  g_known_count = k;
+  g_known_next = k % kKnownRanges;
 }
 
 void remember_range(const char *base, size_t size, int dev) {
@@ -190,6 +202,117 @@ int make_part_op(const gelib_part_desc *r, const gelib_part_desc *x, const gelib
   return GELIB_HIP_OK;
 }
 
+
+// ---- gradient destinations that broadcast ---------------------------------------------------------------------
+// A gradient whose destination has extent 1 where the operation has extent E (the operand is shared by the batch or by
+// the grid, core/Gpart.hpp:168-185) is a sum over that dimension.  The product kernels then write one gradient per
+// cell into a packed temporary and bcast_reduce.hip adds those up in a fixed order; the batch is taken in chunks so
+// that the temporary stays within "bcast_scratch_kb" KiB (64 MiB unless set) (it is 1 % of the bytes of g at the headline type).  The
+// temporary belongs to the library: one buffer per (device, stream), allocated by the first such call and grown when a
+// later one needs more.
+struct ScratchBuf {
+  char *ptr = nullptr;
+  size_t bytes = 0;
+};
+std::mutex g_bcast_mutex;
+std::map<std::pair<int, hipStream_t>, ScratchBuf> g_bcast_scratch;
+int g_bcast_scratch_kb = 64 * 1024;
+int g_bcast_reduce = 1;
+
+bool dest_broadcasts(const gelib_part_desc *d, const long long E[3]) {
+  for (int k = 0; k < 3; k++)
+    if (d->dims[k] == 1 && E[k] > 1) return true;
+  return false;
+}
+
+// descs: the descriptors of the call (copies the caller's `inner` reads); dests: indices of the destinations among
+// them; inner(accumulate) runs the operation on descs as they stand.
+int with_bcast_dests(std::vector<gelib_part_desc> &descs, const std::vector<int> &dests, const long long E[3],
+                     int accumulate, hipStream_t s, const std::function<int(int)> &inner) {
+  const std::vector<gelib_part_desc> orig = descs;
+  std::vector<int> bidx;
+  bool all_bcast = true;
+  for (int i : dests) {
+    if (dest_broadcasts(&orig[i], E)) bidx.push_back(i);
+    else all_bcast = false;
+  }
+  const long long G = E[1] * E[2];
+  long long per_cell = 0;
+  for (int i : bidx) per_cell += orig[i].dims[3] * orig[i].dims[4] * (long long)sizeof(float2);
+  if (per_cell == 0 || E[0] * G == 0) return inner(accumulate);
+  const long long cap = (long long)std::max(1, g_bcast_scratch_kb) << 10;
+  const long long cb = std::max<long long>(1, std::min<long long>(E[0], cap / std::max<long long>(1, per_cell * G)));
+  if (cb * G > 0x7fffffffLL) return GELIB_HIP_ERR_ARG;
+  const long long Ec[3] = {cb, E[1], E[2]};
+  size_t partial = 0;
+  for (int i : bidx) {
+    const long long D[3] = {orig[i].dims[0] == 1 ? 1 : cb, orig[i].dims[1] == 1 ? 1 : E[1], orig[i].dims[2] == 1 ? 1 : E[2]};
+    partial = std::max(partial, bcast_partial_bytes(Ec, D, (int)orig[i].dims[3], (int)orig[i].dims[4]));
+  }
+  const size_t tmp_bytes = ((size_t)(cb * G * per_cell) + 255) & ~(size_t)255;
+  const size_t need = tmp_bytes + partial;
+  int dev = 0;
+  GELIB_HIP_TRY(hipGetDevice(&dev));
+  // held while the kernels of this call are put on the stream: another thread using the same stream's buffer must
+  // come entirely before or entirely after them
+  std::lock_guard<std::mutex> lock(g_bcast_mutex);
+  ScratchBuf &buf = g_bcast_scratch[{dev, s}];
+  if (buf.bytes < need) {
+    if (buf.ptr) {
+      forget_ranges(buf.ptr);
+      GELIB_HIP_TRY(hipFree(buf.ptr));  // waits for the kernels that still use it
+    }
+    buf.ptr = nullptr;
+    buf.bytes = 0;
+    GELIB_HIP_TRY(hipMalloc((void **)&buf.ptr, need));
+    buf.bytes = need;
+  }
+  int rc;
+  for (long long b0 = 0; b0 < E[0]; b0 += cb) {
+    const long long cbn = std::min(cb, E[0] - b0);
+    const long long En[3] = {cbn, E[1], E[2]};
+    for (size_t i = 0; i < descs.size(); i++) {
+      descs[i] = orig[i];
+      if (orig[i].dims[0] == E[0] && E[0] > 1) {
+        descs[i].ptr = (char *)orig[i].ptr + b0 * orig[i].strides[0] * (long long)sizeof(float2);
+        descs[i].dims[0] = cbn;
+      }
+    }
+    size_t off = 0;
+    for (int i : bidx) {
+      gelib_part_desc &d = descs[i];
+      const long long rows = orig[i].dims[3], n = orig[i].dims[4];
+      d.ptr = buf.ptr + off;
+      d.dims[0] = cbn, d.dims[1] = E[1], d.dims[2] = E[2];
+      d.strides[4] = 1, d.strides[3] = n, d.strides[2] = rows * n, d.strides[1] = E[2] * rows * n;
+      d.strides[0] = G * rows * n;
+      off += (size_t)(cb * G * rows * n) * sizeof(float2);
+    }
+    const int inner_acc = (accumulate && !all_bcast) ? 1 : 0;
+    if (inner_acc)
+      for (int i : bidx) {
+        long long own[3];
+        PartDev pd = to_dev(&descs[i], En, own);
+        if ((rc = launch_zero_fill(pd, own, (int)descs[i].dims[3], (int)descs[i].dims[4], s))) return rc;
+      }
+    if ((rc = inner(inner_acc))) return rc;
+    for (int i : bidx) {
+      gelib_part_desc d = orig[i];
+      if (orig[i].dims[0] == E[0] && E[0] > 1) {
+        d.ptr = (char *)orig[i].ptr + b0 * orig[i].strides[0] * (long long)sizeof(float2);
+        d.dims[0] = cbn;
+      }
+      long long own[3];
+      PartDev pd = to_dev(&d, En, own);
+      const bool summed_over_batch = orig[i].dims[0] == 1 && E[0] > 1;
+      rc = launch_bcast_reduce((const float2 *)descs[i].ptr, (float2 *)(buf.ptr + tmp_bytes), pd, En, own,
+                               (int)d.dims[3], (int)d.dims[4], accumulate != 0 || (summed_over_batch && b0 > 0), s);
+      if (rc) return rc;
+    }
+  }
+  return GELIB_HIP_OK;
+}
+
 enum Kind { kFwd, kBack0, kBack1 };
 
 int part_entry(Kind kind, bool diag, const gelib_part_desc *r, const gelib_part_desc *x, const gelib_part_desc *y,
@@ -202,6 +325,12 @@ int part_entry(Kind kind, bool diag, const gelib_part_desc *r, const gelib_part_
   if ((rc = check_pointer(r)) || (rc = check_pointer(x)) || (rc = check_pointer(y))) return rc;
   if (op.E[0] * op.E[1] * op.E[2] == 0 || op.nout == 0) return GELIB_HIP_OK;
   hipStream_t s = (hipStream_t)stream;
+  if (!g_force_generic && g_bcast_reduce && kind != kFwd && dest_broadcasts(kind == kBack0 ? x : y, op.E)) {
+    std::vector<gelib_part_desc> d = {*r, *x, *y};
+    return with_bcast_dests(d, {kind == kBack0 ? 1 : 2}, op.E, accumulate, s, [&](int acc) {
+      return part_entry(kind, diag, &d[0], &d[1], &d[2], offs, acc, stream);
+    });
+  }
   if (!g_force_generic) {
     int used = 0;
     if (diag && kind == kFwd) {
@@ -590,6 +719,28 @@ int vec_bwd_entry(bool diag, const gelib_part_desc *xg, const gelib_part_desc *y
       if ((rc = check_pointer(v.d))) return rc;
   if (plan.E[0] * plan.E[1] * plan.E[2] == 0) return GELIB_HIP_OK;
   hipStream_t s = (hipStream_t)stream;
+  if (!g_force_generic && g_bcast_reduce) {
+    bool bcast = false;
+    for (auto *L : {&XG, &YG})
+      for (auto &v : *L) bcast = bcast || dest_broadcasts(v.d, plan.E);
+    if (bcast) {
+      // descriptors in the caller's order: g, x, y, xg, yg
+      std::vector<gelib_part_desc> d;
+      d.insert(d.end(), g, g + ng);
+      d.insert(d.end(), x, x + nx);
+      d.insert(d.end(), y, y + ny);
+      const int ixg = (int)d.size();
+      if (xg) d.insert(d.end(), xg, xg + nx);
+      const int iyg = (int)d.size();
+      if (yg) d.insert(d.end(), yg, yg + ny);
+      std::vector<int> dests;
+      for (int i = ixg; i < (int)d.size(); i++) dests.push_back(i);
+      return with_bcast_dests(d, dests, plan.E, accumulate, s, [&](int acc) {
+        return vec_bwd_entry(diag, xg ? &d[ixg] : nullptr, yg ? &d[iyg] : nullptr, ng, &d[0], nx, &d[ng], ny, &d[ng + nx],
+                             acc, stream);
+      });
+    }
+  }
   if (!g_force_generic) {
     VecPlan A, B;
     std::vector<View> GA, GB;
@@ -1001,6 +1152,7 @@ int gelib_hip_malloc(void **ptr, uint64_t bytes) {
   return GELIB_HIP_OK;
 }
 int gelib_hip_free(void *ptr) {
+  if (ptr) forget_ranges(ptr);  // the pointer check must not pass views into memory that is gone
   if (ptr) GELIB_HIP_TRY(hipFree(ptr));
   return GELIB_HIP_OK;
 }
@@ -1035,6 +1187,15 @@ int gelib_hip_set_option(const char *name, int value) {
   }
   if (!std::strcmp(name, "check_pointers")) {
     g_check_pointers = value;
+    forget_ranges(nullptr);
+    return GELIB_HIP_OK;
+  }
+  if (!std::strcmp(name, "bcast_scratch_kb")) {  // KiB the temporary of a broadcast gradient destination may take
+    g_bcast_scratch_kb = value > 0 ? value : 64 * 1024;
+    return GELIB_HIP_OK;
+  }
+  if (!std::strcmp(name, "bcast_reduce")) {  // 0: sum a broadcast destination inside the shape-agnostic kernels
+    g_bcast_reduce = value;
     return GELIB_HIP_OK;
   }
   if (!std::strncmp(name, "staged_", 7)) return staged_set_option(name, value);

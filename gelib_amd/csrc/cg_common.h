@@ -51,6 +51,12 @@ int launch_generic_back0(const PartOp &op, bool accumulate, hipStream_t s);  // 
 int launch_generic_back1(const PartOp &op, bool accumulate, hipStream_t s);  // destination = op.y
 int launch_zero_fill(const PartDev &d, const long long D[3], int M, int n, hipStream_t s);
 
+// ---- sums over broadcast dimensions of a gradient destination (bcast_reduce.hip) ----
+// tmp: per-cell gradients packed (E0, E1, E2, rows, n); d: the destination, whose own extents D are E[k] or 1
+size_t bcast_partial_bytes(const long long E[3], const long long D[3], int rows, int n);
+int launch_bcast_reduce(const float2 *tmp, float2 *partial, const PartDev &d, const long long E[3], const long long D[3],
+                        int rows, int n, bool accumulate, hipStream_t s);
+
 // ---- spherical harmonics (spharm.hip): xs = strides of x in floats over (batch, grid0, grid1, xyz, channel) ----
 int launch_spharm(const PartDev &r, const float *x, const long long xs[5], const long long D[3], int L, int n,
                   bool accumulate, hipStream_t s);

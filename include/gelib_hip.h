@@ -12,8 +12,18 @@
  * one of the gelib_hip_status codes without printing or throwing.  Device memory: the first call for a
  * new coefficient table or a new SO3vec type signature on a device computes its tables and uploads them
  * (one allocation and one synchronous copy, kept for the life of the process); gelib_hip_gather_map_create
- * allocates the map it returns; gelib_hip_malloc allocates what it is asked for.  No other call allocates,
- * frees or synchronises: the channel-mixing entry points take their workspace from the caller.
+ * allocates the map it returns; gelib_hip_malloc allocates what it is asked for; a backward call whose gradient
+ * destination broadcasts (see below) takes a temporary that the library keeps per (device, stream).  No other call
+ * allocates, frees or synchronises: the channel-mixing entry points take their workspace from the caller.
+ *
+ * Gradient destinations that broadcast: xg (or yg) with extent 1 along a leading dimension where the other tensors of
+ * the call have extent E > 1 is the gradient of an operand shared along that dimension (core/Gpart.hpp:168-185) and
+ * receives the SUM over it.  The library forms one gradient per cell with the same kernels as without the broadcast,
+ * in a packed temporary of its own (at most "bcast_scratch_kb" KiB, 64 MiB unless set; larger batches are taken in
+ * chunks), and adds those up with a two-stage reduction whose order of additions is fixed: same bits every run, no
+ * atomics.  The temporary is allocated by the first such call on a (device, stream) pair -- make that call outside
+ * stream capture -- grown when a later call needs more, and kept until the process ends; calls on one stream share it
+ * in stream order.
  */
 #ifndef GELIB_HIP_H
 #define GELIB_HIP_H
@@ -234,8 +244,13 @@ int gelib_hip_synchronize(void);
 /*
  * Tuning / introspection (no counterpart in the reference).
  * gelib_hip_set_option("force_generic", 1) routes every call through the shape-agnostic kernels;
- * "check_pointers" (default 1) switches the device-pointer validation of every call off or on (an allocation
- * that has passed once is remembered, so repeated calls on the same buffers make no driver calls for it).
+ * "check_pointers" (default 1) switches the device-pointer validation of every call off (0) or on: with 1 an
+ * allocation that has passed once is remembered (the last 64 of them), so repeated calls on the same buffers make no
+ * driver calls; a buffer that was freed behind the library's back and handed out again smaller at the same address
+ * still passes until its entry is pushed out -- gelib_hip_free forgets the entry, setting the option (to any value)
+ * forgets all of them, and 2 asks the driver on every call (about 30 us per call instead of 3).
+ * "bcast_scratch_kb": KiB the temporary of a broadcast gradient destination may take (0 restores 64 MiB);
+ * "bcast_reduce" (1/0): 0 sums such a destination inside the shape-agnostic kernels, one cell after the other.
  * Tuning knobs of the fast families (0 restores the built-in choice unless noted): "unrolled_fwd" / "unrolled_bwd" /
  * "staged_fwd" / "staged_bwd" / "diag6" / "onepair" (1/0: use the family), "fwd_block_bytes", "fwd_lds_bytes", "fwd_tile",
  * "fwd_cell_tile" (cells per tile of the unrolled forward launch, 0 = one tile, -1 = chosen by the channel counts, the
@@ -255,7 +270,7 @@ int gelib_hip_synchronize(void);
  * GELIB_HIP_ERR_ARG.  Options are process-wide.
  * gelib_hip_last_path() tells which kernel family the last call of this thread used
  * (0 = none, 1 = generic, 2 = unrolled small-l kernels, 3 = staged any-l kernels, 4 = lane-per-channel Diag
- * kernels for operand l up to 6, 5 = single-pair backward kernel for large l).
+ * kernels for operand l up to 6, 5 = single-pair kernels for large l, 6 = the product fused with the weight matrices).
  */
 int gelib_hip_set_option(const char *name, int value);
 int gelib_hip_last_path(void);

@@ -237,6 +237,14 @@ def test_vec_broadcast_operand_gradients(G, diag, shared):
         assert torch.allclose(got, rep.sum(0, keepdim=True), rtol=1e-4, atol=1e-4)
     for got, rep in zip(g_a1[k:], g_aB[k:]):
         assert torch.allclose(got, rep, rtol=1e-5, atol=1e-5)
+    # ... and against the oracle's serial sum over the batch under the parity rules (term sums over the batch too)
+    ha = [U.host(p.detach()) for p in a1.parts.values()]
+    hb = [U.host(p.detach()) for p in bB.parts.values()]
+    hx, hy = args(ha, hb)
+    O = U.VecOracle(hx, hy, 3, diag, gs=[U.host(torch.view_as_complex(w.contiguous())) for w in ws])
+    got_a, got_b = [U.host(t) for t in g_a1[:k]], [U.host(t) for t in g_a1[k:]]
+    got_x, got_y = args(got_a, got_b)
+    O.check_bwd(got_x, got_y, "shared %s diag %d" % (shared, diag))
 
 
 @pytest.mark.parametrize("narrow", ["x", "y"])

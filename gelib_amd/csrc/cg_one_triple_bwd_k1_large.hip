@@ -1,0 +1,11 @@
+// One instantiation of the single-triple backward kernel (cg_one_triple_bwd_impl.h): second operand of 16 channels,
+// the triples whose code does not fit four waves per SIMD.
+#include "cg_one_triple_bwd_impl.h"
+
+namespace gelib_hip {
+
+int launch_one_triple_bwd_k1_large(const BwdArgs &a, int nblocks, size_t lds_bytes, hipStream_t s) {
+  return launch_one_triple_k<1, false>(a, nblocks, lds_bytes, s);
+}
+
+}  // namespace gelib_hip

@@ -100,5 +100,8 @@ bool unrolled_bwd_takes(bool diag, bool padded, int lcap, int lop);
 // or -1 when no backward kernel takes the vector
 int unrolled_bwd_cap(int lcap, int lop);
 int launch_unrolled_bwd(const BwdArgs &a, bool diag, int lcap, int lop, int nblocks, size_t lds_bytes, hipStream_t s);
+// one triple (a.only_dl >= 0), second operand of 16 k channels (k = 1, 2), first operand a power of two >= 16
+size_t one_triple_bwd_lds_bytes(int xsize, int ysize);
+int launch_one_triple_bwd(const BwdArgs &a, int k, int l1, int l2, int l, int nblocks, size_t lds_bytes, hipStream_t s);
 
 }  // namespace gelib_hip

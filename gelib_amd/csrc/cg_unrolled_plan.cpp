@@ -19,6 +19,8 @@ int g_fwd_narrow_decline = 1;  // leave products with at most four channel pairs
 int g_fwd_ti = 0;                    // 0 = widest tile that divides every n1, else force 1 / 2 / 4
 int g_bwd_enable = 1;
 int g_bwd_one_enable = 1; // the backward kernel for calls with one triple
+int g_bwd_one_wide = 1;   // ... and the one for a second operand of 16 or 32 channels (0 off, else cells per wave and block)
+long long g_bwd_one_wide_cells = 4096;  // ... in launches with at least this many cells (a wave takes whole cells)
 int g_bwd_l6_enable = 1;  // the backward kernel for operands up to l = 6
 int g_bwd_min_runs = 128;           // runs of 64 slots a backward block should have at least, LDS allowing (0: no such rule)
 int g_bwd_lds_target = 40 * 1024;  // LDS bytes per block the backward kernel aims at when it picks the cells per block
@@ -413,6 +415,21 @@ int run_bwd(bool diag, const std::vector<VecTriple> &triples, const std::vector<
   a.only_dl = -1;
   if (triples.size() == 1 && !diag && !plan->padded && lop <= kLT && g_bwd_one_enable)
     a.only_dl = triples[0].l - std::abs(triples[0].l1 - triples[0].l2);
+  if (a.only_dl >= 0 && g_bwd_one_wide > 0) {
+    const int n1 = xs[triples[0].xi].second, n2 = ys[triples[0].yi].second;
+    // every wave of that kernel takes whole cells: it needs launches with cells enough to fill the GPU that way
+    if ((n2 == 16 || n2 == 32) && n1 >= 16 && is_pow2(n1) && ncells >= g_bwd_one_wide_cells) {
+      const int cpb1 = 4 * std::max(1, g_bwd_one_wide);
+      a.cells_per_block = cpb1;
+      const long long nb = (ncells + cpb1 - 1) / cpb1;
+      if (nb > 0x7fffffffLL) return GELIB_HIP_ERR_ARG;
+      rc = launch_one_triple_bwd(a, n2 / 16, triples[0].l1, triples[0].l2, triples[0].l, (int)nb,
+                                 one_triple_bwd_lds_bytes(a.xsize, a.ysize), s);
+      if (rc) return rc;
+      *used = 1;
+      return GELIB_HIP_OK;
+    }
+  }
   const long long nblocks = (ncells + cpb - 1) / cpb;
   if (nblocks > 0x7fffffffLL) return GELIB_HIP_ERR_ARG;
   rc = launch_unrolled_bwd(a, diag, lcap, lop, (int)nblocks, lds, s);
@@ -549,6 +566,14 @@ int unrolled_set_option(const char *name, int value) {
   }
   if (!std::strcmp(name, "unrolled_fwd_l6")) {
     g_fwd_l6_enable = value;
+    return GELIB_HIP_OK;
+  }
+  if (!std::strcmp(name, "unrolled_bwd_one_wide_cells")) {
+    g_bwd_one_wide_cells = value;
+    return GELIB_HIP_OK;
+  }
+  if (!std::strcmp(name, "unrolled_bwd_one_wide")) {  // 0 off, otherwise the cells per wave of a block of that kernel
+    g_bwd_one_wide = value;
     return GELIB_HIP_OK;
   }
   if (!std::strcmp(name, "unrolled_bwd_one")) {

@@ -39,6 +39,12 @@ SHAPES = [
     (9, 0, 3, 3, 16, 4),
     (2, 6, 6, 6, 2, 4),          # operands above l = 4, product l up to 6
     (2, 5, 6, 1, 8, 2),
+    (5, 2, 3, 4, 32, 32),        # configuration 2's triple: the single-triple backward kernel, 32 channels of y
+    (3, 3, 2, 1, 16, 64),        # ... 64
+    (3, 4, 4, 8, 64, 16),        # ... 16
+    (2, 0, 4, 4, 16, 32),
+    (2, 4, 0, 4, 128, 32),
+    (6, 1, 1, 0, 32, 16),
 ]
 
 

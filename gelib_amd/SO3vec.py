@@ -92,11 +92,12 @@ class SO3vec:
         xparts = list(self.parts.values())
         yparts = list(y.parts.values())
         one = _one_channel_side(xparts, yparts)
-        if one is not None:
+        if one is not None and (xparts if one == "y" else yparts)[0].size(-1) > 64:
             # features times a one-channel vector (spherical harmonics of one direction per sample, say): block channel
-            # i*N2 + j has N2 = 1 (or N1 = 1), so the product is the DiagCGproduct with the one channel repeated, and the
-            # lane-per-channel kernels run it about twice as fast as the general ones run 16 x 1 channels.  The repeat is
-            # a torch op: its backward sums the gradient over the channels.
+            # i*N2 + j has N2 = 1 (or N1 = 1), so the product is the DiagCGproduct with the one channel repeated.  Up to
+            # 64 channels the library runs it that way by itself, forward and backward (every lane reads the one
+            # channel, no copy); with more channels its backward pass would fall to the general kernels, so here the
+            # channel is repeated by a torch op, whose backward sums the gradient over the channels.
             wide, narrow = (xparts, yparts) if one == "y" else (yparts, xparts)
             n = wide[0].size(-1)
             rep = [p.expand(*p.shape[:-1], n).contiguous() for p in narrow]

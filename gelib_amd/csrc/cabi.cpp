@@ -438,16 +438,24 @@ PartOp triple_op(const VecPlan &plan, const VecTriple &t, const std::vector<View
 
 // A Diag product that reaches above l = 6: the lane-per-channel kernels (built for products up to l = 6) take the
 // triples up to there, the other families the rest.  R is sorted by l, so A keeps a prefix of it and B the remainder.
-bool split_diag(const VecPlan &plan, const std::vector<View> &R, VecPlan &A, VecPlan &B, std::vector<View> &RA,
-                std::vector<View> &RB) {
+// (A CGproduct with a one-channel operand is such a Diag product with the channel repeated, and is split the same way.)
+bool split_diag(const VecPlan &plan, const std::vector<View> &R, const std::vector<View> &X, const std::vector<View> &Y,
+                VecPlan &A, VecPlan &B, std::vector<View> &RA, std::vector<View> &RB) {
   constexpr int kSplit = 6;
-  if (!plan.diag) return false;
+  if (!plan.diag) {
+    auto all_one = [](const std::vector<View> &v) {
+      for (auto &p : v)
+        if (p.n != 1) return false;
+      return true;
+    };
+    if (!all_one(X) && !all_one(Y)) return false;
+  }
   bool lo = false, hi = false;
   for (auto &t : plan.triples) (t.l <= kSplit ? lo : hi) = true;
   if (!lo || !hi) return false;
   size_t k0 = 0;
   while (k0 < R.size() && R[k0].l <= kSplit) k0++;
-  A.diag = B.diag = true;
+  A.diag = B.diag = plan.diag;
   for (int k = 0; k < 3; k++) A.E[k] = B.E[k] = plan.E[k];
   for (auto t : plan.triples) {
     if (t.l <= kSplit) {
@@ -530,7 +538,7 @@ int vec_fwd_entry(bool diag, int nr, const gelib_part_desc *r, int nx, const gel
   if (!g_force_generic) {
     VecPlan A, B;
     std::vector<View> RA, RB;
-    if (split_diag(plan, R, A, B, RA, RB)) {
+    if (split_diag(plan, R, X, Y, A, B, RA, RB)) {
       std::vector<const gelib_part_desc *> rd, xd, yd;
       for (auto &v : RA) rd.push_back(v.d);
       for (auto &v : X) xd.push_back(v.d);
@@ -744,7 +752,7 @@ int vec_bwd_entry(bool diag, const gelib_part_desc *xg, const gelib_part_desc *y
   if (!g_force_generic) {
     VecPlan A, B;
     std::vector<View> GA, GB;
-    if (split_diag(plan, G, A, B, GA, GB)) {
+    if (split_diag(plan, G, X, Y, A, B, GA, GB)) {
       std::vector<const gelib_part_desc *> gd, xd, yd, xgd, ygd;
       for (auto &v : GA) gd.push_back(v.d);
       for (auto &v : X) xd.push_back(v.d);

@@ -50,7 +50,8 @@ struct Diag6Args {
   long long ncells;
   int groups;         // 64-channel groups per cell (more than 32 channels)
   int lg_npad;        // log2 of the channel count rounded up to a power of two, at most 6
-  int n;              // channels of every part
+  int n;              // channels of every part (of every part of the wider operand when xbc or ybc is set)
+  int xbc, ybc;       // CGproduct with a one-channel first / second operand: every lane reads that channel
   int offs_add;
   int accumulate;
   int want_x, want_y;  // backward: which gradients are stored (the operand of an unwanted one is never read)

@@ -15,6 +15,7 @@
 #pragma once
 
 #include "cg_diag6.h"
+#include "cg_lane_sums.h"
 #include "cg_unrolled_dev.h"
 
 namespace gelib_hip {
@@ -82,10 +83,13 @@ __device__ __forceinline__ WavePos wave_pos(const Diag6Args &a, long long w) {
 
 // Byte offset of the lane's element from row 0 of the wave's first cell; 32 bits (the host checks the range).
 // PACKED: several cells per wave, so the offset depends on the part's cell stride; otherwise it is the channel alone.
+// bc: the part has ONE channel, which every lane reads (a CGproduct with a one-channel operand is the Diag product with
+// that channel repeated); its gradient is then a sum over the lanes of a cell.
 template <bool PACKED>
-__device__ __forceinline__ unsigned lane_offset(const FastPart P, const WavePos q) {
-  if constexpr (PACKED) return ((unsigned)q.cell_local * (unsigned)P.sb + (unsigned)q.ch) * 8u;
-  else return (unsigned)q.ch * 8u;
+__device__ __forceinline__ unsigned lane_offset(const FastPart P, const WavePos q, bool bc = false) {
+  const unsigned ch = bc ? 0u : (unsigned)q.ch;
+  if constexpr (PACKED) return ((unsigned)q.cell_local * (unsigned)P.sb + ch) * 8u;
+  else return ch * 8u;
 }
 
 // Row 0 of a part in the wave's cell, and the distance between its rows in bytes.
@@ -93,10 +97,10 @@ __device__ __forceinline__ RowPtr cell_row0(const FastPart P, long long cell) { 
 __device__ __forceinline__ long long row_step(const FastPart P) { return (long long)P.sm * 8; }
 
 template <int L, bool PACKED>
-__device__ __forceinline__ void load_rows(float2 (&v)[2 * L + 1], const FastPart P, const WavePos q) {
+__device__ __forceinline__ void load_rows(float2 (&v)[2 * L + 1], const FastPart P, const WavePos q, bool bc) {
   RowPtr row = cell_row0(P, q.cell);
   const long long step = row_step(P);
-  const unsigned lo = lane_offset<PACKED>(P, q);
+  const unsigned lo = lane_offset<PACKED>(P, q, bc);
 #pragma unroll
   for (int m = 0; m <= 2 * L; m++) {
     v[m] = row_load(row, lo);
@@ -163,7 +167,8 @@ __device__ __forceinline__ void fwd_pair(const Diag6Args &a, const float2 (&xv)[
 // the image holding row m of part l, one column per lane.  The rows are dealt to the four waves in turn; every wave
 // requests all of its rows before it writes the first one.
 template <bool PACKED, int LOP>
-__device__ __forceinline__ void stage_operand(float2 *img, const FastPart (&parts)[kNP], const WavePos q, int wave, int lane) {
+__device__ __forceinline__ void stage_operand(float2 *img, const FastPart (&parts)[kNP], const WavePos q, int wave, int lane,
+                                              bool bc) {
   constexpr int kRows = (LOP + 1) * (LOP + 1);  // rows of the parts l = 0..LOP
   constexpr int kPer = (kRows + 3) / 4;
   float2 v[kPer];
@@ -174,7 +179,7 @@ __device__ __forceinline__ void stage_operand(float2 *img, const FastPart (&part
     static_for<LOP + 1>([&](auto lc) __attribute__((always_inline)) {
       constexpr int L = decltype(lc)::value;
       if (r >= L * L && r < (L + 1) * (L + 1) && parts[L].ptr != nullptr)
-        v[k] = row_load(cell_row0(parts[L], q.cell) + (long long)(r - L * L) * row_step(parts[L]), lane_offset<PACKED>(parts[L], q));
+        v[k] = row_load(cell_row0(parts[L], q.cell) + (long long)(r - L * L) * row_step(parts[L]), lane_offset<PACKED>(parts[L], q, bc));
     });
   });
   static_for<kPer>([&](auto kc) __attribute__((always_inline)) {
@@ -204,13 +209,13 @@ __global__ void __launch_bounds__(256) diag6_fwd_kernel(const Diag6Args a) {
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const long long w = blockIdx.x;
   const WavePos q = wave_pos(a, w);
-  stage_operand<PACKED, LOP>(yimg, a.y, q, wave, lane);
+  stage_operand<PACKED, LOP>(yimg, a.y, q, wave, lane, a.ybc != 0);
   __syncthreads();
   static_for<LOP + 1>([&](auto l1c) __attribute__((always_inline)) {
     constexpr int L1 = decltype(l1c)::value;
     if (a.x[L1].ptr != nullptr) {
       float2 xv[2 * L1 + 1];
-      load_rows<L1, PACKED>(xv, a.x[L1], q);
+      load_rows<L1, PACKED>(xv, a.x[L1], q, a.xbc != 0);
       static_for<LOP + 1>([&](auto l2c) __attribute__((always_inline)) {
         constexpr int L2 = decltype(l2c)::value;
         if (((L1 * kNP + L2) & 3) == wave && a.y[L2].ptr != nullptr) {
@@ -315,12 +320,29 @@ __device__ __forceinline__ void bwd_pair(const Diag6Args &a, const float2 (&xv)[
   }
 }
 
+// bc: the part has one channel: the lanes' values are added over the lanes of a cell (2^lg_n of them, a fixed order of
+// additions) and the cell's first lane stores the total.
 template <int L, bool PACKED>
-__device__ __forceinline__ void store_rows(const float2 *v, int vstride, const FastPart P, const WavePos q, bool accumulate) {
-  if (!q.live) return;
+__device__ __forceinline__ void store_rows(const float2 *v, int vstride, const FastPart P, const WavePos q, bool accumulate,
+                                           bool bc, int lg_n) {
   RowPtr row = cell_row0(P, q.cell);
   const long long step = row_step(P);
-  const unsigned lo = lane_offset<PACKED>(P, q);
+  const unsigned lo = lane_offset<PACKED>(P, q, bc);
+  if (bc) {
+    float2 t[2 * L + 1];
+#pragma unroll
+    for (int m = 0; m <= 2 * L; m++) t[m] = q.live ? v[m * vstride] : make_float2(0.f, 0.f);
+    group_sum(t, 1 << lg_n);
+    if (q.live && q.ch == 0) {
+#pragma unroll
+      for (int m = 0; m <= 2 * L; m++) {
+        row_store(row, lo, t[m], accumulate);
+        row += step;
+      }
+    }
+    return;
+  }
+  if (!q.live) return;
 #pragma unroll
   for (int m = 0; m <= 2 * L; m++) {
     row_store(row, lo, v[m * vstride], accumulate);
@@ -357,7 +379,7 @@ __global__ void __launch_bounds__(256) diag6_bwd_kernel(const Diag6Args a) {
       // never read (a part-level call for one gradient does not even have it) and enters as zeros
       float2 xv[2 * L1 + 1], ax[2 * L1 + 1];
       if (wy) {
-        load_rows<L1, PACKED>(xv, a.x[L1], q);
+        load_rows<L1, PACKED>(xv, a.x[L1], q, a.xbc != 0);
       } else {
 #pragma unroll
         for (int m1 = 0; m1 <= 2 * L1; m1++) xv[m1] = make_float2(0.f, 0.f);
@@ -369,7 +391,7 @@ __global__ void __launch_bounds__(256) diag6_bwd_kernel(const Diag6Args a) {
         if (a.owner[L2] == wave && a.y[L2].ptr != nullptr) {
           float2 yv[2 * L2 + 1];
           if (wx) {
-            load_rows<L2, PACKED>(yv, a.y[L2], q);
+            load_rows<L2, PACKED>(yv, a.y[L2], q, a.ybc != 0);
           } else {
 #pragma unroll
             for (int m2 = 0; m2 <= 2 * L2; m2++) yv[m2] = make_float2(0.f, 0.f);
@@ -385,18 +407,26 @@ __global__ void __launch_bounds__(256) diag6_bwd_kernel(const Diag6Args a) {
       const FastPart XG = a.xg[L1];
       RowPtr row0 = cell_row0(XG, q.cell);
       const long long step = row_step(XG);
-      const unsigned xlo = lane_offset<PACKED>(XG, q);
+      const bool xbc = a.xbc != 0;
+      const unsigned xlo = lane_offset<PACKED>(XG, q, xbc);
       static_for<2 * L1 + 1>([&](auto rc) __attribute__((always_inline)) {
         constexpr int r = decltype(rc)::value;
-        if ((r & 3) == wave && q.live) {
-          float2 t = xpart[(0 * kXRows + r) * 64 + lane];
+        if ((r & 3) == wave) {  // uniform
+          float2 t[1];
+          t[0] = xpart[(0 * kXRows + r) * 64 + lane];
 #pragma unroll
           for (int k = 1; k < 4; k++) {
             const float2 u = xpart[(k * kXRows + r) * 64 + lane];
-            t.x += u.x;
-            t.y += u.y;
+            t[0].x += u.x;
+            t[0].y += u.y;
           }
-          row_store(row0 + r * step, xlo, t, accumulate);
+          if (xbc) {  // one channel of x: its gradient is the sum over the lanes of the cell
+            if (!q.live) t[0] = make_float2(0.f, 0.f);
+            group_sum(t, 1 << a.lg_npad);
+            if (q.live && q.ch == 0) row_store(row0 + r * step, xlo, t[0], accumulate);
+          } else if (q.live) {
+            row_store(row0 + r * step, xlo, t[0], accumulate);
+          }
         }
       });
       __syncthreads();
@@ -406,7 +436,7 @@ __global__ void __launch_bounds__(256) diag6_bwd_kernel(const Diag6Args a) {
     constexpr int L2 = decltype(l2c)::value;
     const FastPart YG = a.yg[L2];
     if (wy && a.owner[L2] == wave && YG.ptr != nullptr)
-      store_rows<L2, PACKED>(yimg + (L2 * L2) * 64 + lane, 64, YG, q, accumulate);
+      store_rows<L2, PACKED>(yimg + (L2 * L2) * 64 + lane, 64, YG, q, accumulate, a.ybc != 0, a.lg_npad);
   });
 }
 
@@ -431,15 +461,15 @@ __device__ __forceinline__ void bwd_wave_set(const Diag6Args &a, float2 *yimg, f
 #pragma unroll
   for (int m = 0; m < RB; m++) yb[m] = make_float2(0.f, 0.f);
   if (wx) {
-    load_rows<LA, PACKED>(ya, a.y[LA], q);
-    if constexpr (LB >= 0) load_rows<LBX, PACKED>(yb, a.y[LBX], q);
+    load_rows<LA, PACKED>(ya, a.y[LA], q, a.ybc != 0);
+    if constexpr (LB >= 0) load_rows<LBX, PACKED>(yb, a.y[LBX], q, a.ybc != 0);
   }
   static_for<kNP>([&](auto l1c) __attribute__((always_inline)) {
     constexpr int L1 = decltype(l1c)::value;
     if (a.x[L1].ptr != nullptr) {  // the same for the whole block
       float2 xv[2 * L1 + 1], ax[2 * L1 + 1];
       if (wy) {
-        load_rows<L1, PACKED>(xv, a.x[L1], q);
+        load_rows<L1, PACKED>(xv, a.x[L1], q, a.xbc != 0);
       } else {
 #pragma unroll
         for (int m1 = 0; m1 <= 2 * L1; m1++) xv[m1] = make_float2(0.f, 0.f);
@@ -456,27 +486,37 @@ __device__ __forceinline__ void bwd_wave_set(const Diag6Args &a, float2 *yimg, f
       const FastPart XG = a.xg[L1];
       RowPtr row0 = cell_row0(XG, q.cell);
       const long long step = row_step(XG);
-      const unsigned xlo = lane_offset<PACKED>(XG, q);
+      const bool xbc = a.xbc != 0;
+      const unsigned xlo = lane_offset<PACKED>(XG, q, xbc);
       static_for<2 * L1 + 1>([&](auto rc) __attribute__((always_inline)) {
         constexpr int r = decltype(rc)::value;
-        if ((r & 3) == wave && q.live) {
-          float2 t = xpart[(0 * kXRows + r) * 64 + lane];
+        if ((r & 3) == wave) {  // uniform
+          float2 t[1];
+          t[0] = xpart[(0 * kXRows + r) * 64 + lane];
 #pragma unroll
           for (int k = 1; k < 4; k++) {
             const float2 u = xpart[(k * kXRows + r) * 64 + lane];
-            t.x += u.x;
-            t.y += u.y;
+            t[0].x += u.x;
+            t[0].y += u.y;
           }
-          row_store(row0 + r * step, xlo, t, accumulate);
+          if (xbc) {  // one channel of x: its gradient is the sum over the lanes of the cell
+            if (!q.live) t[0] = make_float2(0.f, 0.f);
+            group_sum(t, 1 << a.lg_npad);
+            if (q.live && q.ch == 0) row_store(row0 + r * step, xlo, t[0], accumulate);
+          } else if (q.live) {
+            row_store(row0 + r * step, xlo, t[0], accumulate);
+          }
         }
       });
       __syncthreads();
     }
   });
   if (wy) {
-    if (a.yg[LA].ptr != nullptr) store_rows<LA, PACKED>(yimg + (LA * LA) * 64 + lane, 64, a.yg[LA], q, accumulate);
+    if (a.yg[LA].ptr != nullptr)
+      store_rows<LA, PACKED>(yimg + (LA * LA) * 64 + lane, 64, a.yg[LA], q, accumulate, a.ybc != 0, a.lg_npad);
     if constexpr (LB >= 0)
-      if (a.yg[LBX].ptr != nullptr) store_rows<LBX, PACKED>(yimg + (LBX * LBX) * 64 + lane, 64, a.yg[LBX], q, accumulate);
+      if (a.yg[LBX].ptr != nullptr)
+        store_rows<LBX, PACKED>(yimg + (LBX * LBX) * 64 + lane, 64, a.yg[LBX], q, accumulate, a.ybc != 0, a.lg_npad);
   }
 }
 

@@ -20,6 +20,7 @@ std::map<std::pair<int, std::vector<int>>, int *> g_offs;  // (device, offsets) 
 int g_enable = 1;
 int g_l8_enable = 1;    // the kernels for products up to l = 8 of operands up to l = 4: 1 forward, 2 backward too
 int g_sets_enable = 1;  // backward: the kernel with the waves' sets of l2 fixed at compile time, where it applies
+int g_one_channel = 1;  // CGproduct with a one-channel operand runs here as the Diag product with the channel repeated
 
 int device_bank(const float **out) {
   int dev = 0;
@@ -62,7 +63,7 @@ int make_args(const VecPlan &plan, const std::vector<const gelib_part_desc *> &r
               const std::vector<const gelib_part_desc *> *xg, const std::vector<const gelib_part_desc *> *yg,
               bool r_is_dest, Diag6Args *a, int *lcap, bool *ok) {
   *ok = false;
-  if (!g_enable || !plan.diag) return GELIB_HIP_OK;
+  if (!g_enable) return GELIB_HIP_OK;
   std::vector<FastPart> fx, fy, fr, fxg, fyg;
   std::vector<std::pair<int, int>> lx, ly, lr;
   if (!lists_to_fast(x, plan.E, false, &fx, &lx) || !lists_to_fast(y, plan.E, false, &fy, &ly) ||
@@ -70,12 +71,29 @@ int make_args(const VecPlan &plan, const std::vector<const gelib_part_desc *> &r
     return GELIB_HIP_OK;
   if (xg && !lists_to_fast(*xg, plan.E, true, &fxg, nullptr)) return GELIB_HIP_OK;
   if (yg && !lists_to_fast(*yg, plan.E, true, &fyg, nullptr)) return GELIB_HIP_OK;
-  const int n = lx[0].second;
+  // A CGproduct in which every part of one operand has ONE channel is the Diag product with that channel repeated:
+  // block channel i * 1 + 0 (resp. 0 * n + j) is the wide operand's own channel, and the blocks follow each other n
+  // apart either way (core/Gvec.hpp:311-321 against :358-367).  Lanes then all read the one channel, and its gradient
+  // is a sum over the lanes of a cell (one block per cell: up to 64 channels).
+  bool xbc = false, ybc = false;
+  if (!plan.diag) {
+    if (!g_one_channel) return GELIB_HIP_OK;
+    auto all_one = [](const std::vector<std::pair<int, int>> &v) {
+      for (auto &p : v)
+        if (p.second != 1) return false;
+      return true;
+    };
+    ybc = all_one(ly);
+    xbc = !ybc && all_one(lx);
+    if (!xbc && !ybc) return GELIB_HIP_OK;
+  }
+  const int n = (xbc ? ly : lx)[0].second;
   if (n < 1 || n > kMaxChannels) return GELIB_HIP_OK;
+  if ((xbc && xg && n > 64) || (ybc && yg && n > 64)) return GELIB_HIP_OK;
   for (auto &p : lx)
-    if (p.first > kL6 || p.second != n) return GELIB_HIP_OK;
+    if (p.first > kL6 || p.second != (xbc ? 1 : n)) return GELIB_HIP_OK;
   for (auto &p : ly)
-    if (p.first > kL6 || p.second != n) return GELIB_HIP_OK;
+    if (p.first > kL6 || p.second != (ybc ? 1 : n)) return GELIB_HIP_OK;
   for (auto &p : lr)
     if (p.first > 2 * kL6) return GELIB_HIP_OK;
   std::memset(a, 0, sizeof(*a));
@@ -125,6 +143,8 @@ int make_args(const VecPlan &plan, const std::vector<const gelib_part_desc *> &r
   const long long ncells = plan.E[0] * plan.E[1] * plan.E[2];
   a->ncells = ncells;
   a->n = n;
+  a->xbc = xbc ? 1 : 0;
+  a->ybc = ybc ? 1 : 0;
   int lg = 0;
   while ((1 << lg) < n && lg < 6) lg++;
   a->lg_npad = lg;
@@ -241,6 +261,10 @@ int diag6_set_option(const char *name, int value) {
   }
   if (!std::strcmp(name, "diag6_l8")) {
     g_l8_enable = value;
+    return GELIB_HIP_OK;
+  }
+  if (!std::strcmp(name, "diag6_one_channel")) {
+    g_one_channel = value;
     return GELIB_HIP_OK;
   }
   if (!std::strcmp(name, "diag6_sets")) {

@@ -87,7 +87,8 @@ def test_diag6_vec(cabi, B, tx, ty, maxl):
 
 
 def test_diag6_declines_what_it_cannot_do(cabi):
-    # a product above l = 6 is shared with the other families; a broadcast operand whose gradient is wanted is theirs
+    # a product above l = 6 is shared with the other families; the gradient of an operand shared by the batch is formed
+    # per cell by these kernels and summed over the batch by the library
     x = [U.dev(U.seeded(1, 1, 13, 64))]
     y = [U.dev(U.seeded(2, 4, 13, 64))]
     r = [torch.zeros(4, 2 * l + 1, 64, dtype=torch.complex64, device="cuda") for l in range(13)]
@@ -103,7 +104,10 @@ def test_diag6_declines_what_it_cannot_do(cabi):
         assert U.gate_excess(U.host(a), b) <= 1.0
     xg, yg = [torch.zeros_like(x[0])], [torch.zeros_like(y[0])]
     cabi.so3vec_bwd(xg, yg, r6, x, y, accumulate=False, diag=True)
-    assert cabi.last_path() != DIAG6          # its gradient needs a sum over the batch
+    assert cabi.last_path() == DIAG6          # one gradient per cell from these kernels, then the sum over the batch
+    torch.cuda.synchronize()
+    O = U.VecOracle([U.host(x[0])], [U.host(y[0])], 6, True, gs=[U.host(a) for a in r6])
+    O.check_bwd([U.host(xg[0])], [U.host(yg[0])], "x shared by the batch")
     # a broadcast operand with several cells per wave
     x8 = [U.dev(U.seeded(3, 1, 11, 8))]
     y8 = [U.dev(U.seeded(4, 21, 11, 8))]
@@ -157,3 +161,81 @@ def _above_l6(cabi, B, tau, maxl):
         else:
             O.check_fwd(hr, "split Diag product")
             O.check_bwd(hxg, hyg, "split Diag gradients")
+
+
+ONE_CHANNEL = [
+    # (B, channels of the wide operand, l of the wide parts, l of the one-channel parts, maxl, narrow side)
+    (37, 16, range(5), range(3), 4, "y"),        # features x single-channel harmonics, four cells per wave
+    (37, 16, range(5), range(3), -1, "y"),       # uncapped: l up to 6
+    (9, 64, range(4), range(4), 6, "y"),         # one cell per wave
+    (11, 40, [0, 2, 5], [1, 6], 6, "x"),         # the first operand is the narrow one; 24 lanes idle
+    (70, 5, [3, 4], [2], 6, "x"),                # eight cells per wave, three lanes of each idle
+    (5, 64, range(7), range(7), 6, "y"),         # every part of y: the kernel with fixed sets of l2 per wave
+    (3, 16, range(5), range(5), -1, "y"),        # product up to l = 8: split at l = 6 (or the l <= 8 kernels forward)
+]
+
+
+@pytest.mark.parametrize("B,n,lw,ln,maxl,narrow", ONE_CHANNEL)
+def test_cgproduct_with_a_one_channel_operand(cabi, B, n, lw, ln, maxl, narrow):
+    """CGproduct in which every part of one operand has ONE channel (features times single-channel spherical harmonics,
+    the usual use of add_spharm's output): the lane-per-channel kernels take it as the Diag product with that channel
+    repeated -- every lane reads the one channel, its gradient is summed over the lanes of a cell.  Against the oracle's
+    CGproduct loops."""
+    seed = 4000 + B
+    wide = [U.seeded(seed + l, B, 2 * l + 1, n) for l in lw]
+    thin = [U.seeded(seed + 50 + l, B, 2 * l + 1, 1) for l in ln]
+    xs, ys = (thin, wide) if narrow == "x" else (wide, thin)
+    O = U.VecOracle(xs, ys, maxl, False, gseed=seed + 100)
+    dxs, dys, dgs = [U.dev(a) for a in xs], [U.dev(a) for a in ys], [U.dev(a) for a in O.gs]
+    drs = [torch.full(p.shape, 7.0 + 1j, dtype=torch.complex64, device="cuda") for p in O.r32]
+    cabi.so3vec_fwd(drs, dxs, dys, accumulate=False)
+    assert cabi.last_path() == DIAG6
+    dxg = [torch.full(a.shape, 3.0 - 2j, dtype=torch.complex64, device="cuda") for a in xs]
+    dyg = [torch.full(a.shape, 3.0 - 2j, dtype=torch.complex64, device="cuda") for a in ys]
+    cabi.so3vec_bwd(dxg, dyg, dgs, dxs, dys, accumulate=False)
+    assert cabi.last_path() == DIAG6
+    torch.cuda.synchronize()
+    tag = "B%d n%d %s x %s maxl %d narrow %s" % (B, n, list(lw), list(ln), maxl, narrow)
+    O.check_fwd([U.host(a) for a in drs], tag)
+    O.check_bwd([U.host(a) for a in dxg], [U.host(a) for a in dyg], tag)
+    # accumulate mode, and one gradient per call (bit for bit the same sums)
+    dxg2, dyg2 = [a.clone() for a in dxg], [a.clone() for a in dyg]
+    cabi.so3vec_bwd(dxg2, dyg2, dgs, dxs, dys, accumulate=True)
+    torch.cuda.synchronize()
+    O.check_bwd_onto([U.host(a) for a in dxg2], [U.host(a) for a in dyg2], [U.host(a) for a in dxg],
+                     [U.host(a) for a in dyg], tag + " accumulated")
+    dxg3, dyg3 = [torch.full_like(a, 9.0) for a in dxg], [torch.full_like(a, 9.0) for a in dyg]
+    cabi.so3vec_bwd(dxg3, None, dgs, dxs, dys, accumulate=False)
+    cabi.so3vec_bwd(None, dyg3, dgs, dxs, dys, accumulate=False)
+    if maxl <= 6 and max(list(lw)) + max(list(ln)) <= 6 or maxl in range(0, 7):
+        for a, b in zip(dxg3 + dyg3, dxg + dyg):
+            assert torch.equal(torch.view_as_real(a), torch.view_as_real(b))
+    # the general kernels give the same to rounding
+    cabi.set_option("diag6_one_channel", 0)
+    try:
+        cabi.so3vec_bwd(dxg3, dyg3, dgs, dxs, dys, accumulate=False)
+        assert cabi.last_path() != DIAG6
+        torch.cuda.synchronize()
+        O.check_bwd([U.host(a) for a in dxg3], [U.host(a) for a in dyg3], tag + " general kernels")
+    finally:
+        cabi.set_option("diag6_one_channel", 1)
+
+
+def test_one_channel_operand_with_many_channels_on_the_other_side(cabi):
+    # more than 64 channels: forward here (any count), the gradient of the one-channel operand on the other families
+    B, n = 4, 96
+    xs = [U.seeded(10 + l, B, 2 * l + 1, n) for l in range(3)]
+    ys = [U.seeded(20 + l, B, 2 * l + 1, 1) for l in range(3)]
+    O = U.VecOracle(xs, ys, 4, False, gseed=77)
+    dxs, dys, dgs = [U.dev(a) for a in xs], [U.dev(a) for a in ys], [U.dev(a) for a in O.gs]
+    drs = [torch.empty(p.shape, dtype=torch.complex64, device="cuda") for p in O.r32]
+    cabi.so3vec_fwd(drs, dxs, dys, accumulate=False)
+    assert cabi.last_path() == DIAG6
+    dxg, dyg = [torch.empty_like(a) for a in dxs], [torch.empty_like(a) for a in dys]
+    cabi.so3vec_bwd(dxg, dyg, dgs, dxs, dys, accumulate=False)
+    assert cabi.last_path() != DIAG6
+    cabi.so3vec_bwd(dxg, None, dgs, dxs, dys, accumulate=False)
+    assert cabi.last_path() == DIAG6      # the wide operand's gradient alone needs no sum over lanes
+    torch.cuda.synchronize()
+    O.check_fwd([U.host(a) for a in drs], "n 96")
+    O.check_bwd([U.host(a) for a in dxg], [U.host(a) for a in dyg], "n 96")

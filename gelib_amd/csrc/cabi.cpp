@@ -35,6 +35,43 @@ int record_hip_error(hipError_t e, const char *what) {
 }
 
 namespace {
+void forget_ranges(const void *base);
+struct ScratchBuf {
+  char *ptr = nullptr;
+  size_t bytes = 0;
+};
+constexpr int kScratchKinds = 2;
+std::mutex g_scratch_mutex[kScratchKinds];
+std::map<std::pair<int, hipStream_t>, ScratchBuf> g_scratch[kScratchKinds];
+}  // namespace
+
+std::mutex &stream_scratch_mutex(int kind) { return g_scratch_mutex[kind]; }
+
+int stream_scratch(int kind, hipStream_t s, size_t bytes, void **out) {
+  // A call that is being recorded into a graph gets none (*out = nullptr) and takes its scratch-free route: the graph
+  // would keep the buffer's address, and a later call that needs a larger buffer frees it.
+  *out = nullptr;
+  hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(s, &cap) != hipSuccess) (void)hipGetLastError();
+  if (cap != hipStreamCaptureStatusNone) return GELIB_HIP_OK;
+  int dev = 0;
+  GELIB_HIP_TRY(hipGetDevice(&dev));
+  ScratchBuf &buf = g_scratch[kind][{dev, s}];
+  if (buf.bytes < bytes) {
+    if (buf.ptr) {
+      forget_ranges(buf.ptr);
+      GELIB_HIP_TRY(hipFree(buf.ptr));  // waits for the kernels that still use it
+    }
+    buf.ptr = nullptr;
+    buf.bytes = 0;
+    GELIB_HIP_TRY(hipMalloc((void **)&buf.ptr, bytes));
+    buf.bytes = bytes;
+  }
+  *out = buf.ptr;
+  return GELIB_HIP_OK;
+}
+
+namespace {
 
 struct View {  // one validated descriptor
   const gelib_part_desc *d;
@@ -210,12 +247,6 @@ int make_part_op(const gelib_part_desc *r, const gelib_part_desc *x, const gelib
 // that the temporary stays within "bcast_scratch_kb" KiB (64 MiB unless set) (it is 1 % of the bytes of g at the headline type).  The
 // temporary belongs to the library: one buffer per (device, stream), allocated by the first such call and grown when a
 // later one needs more.
-struct ScratchBuf {
-  char *ptr = nullptr;
-  size_t bytes = 0;
-};
-std::mutex g_bcast_mutex;
-std::map<std::pair<int, hipStream_t>, ScratchBuf> g_bcast_scratch;
 int g_bcast_scratch_kb = 64 * 1024;
 int g_bcast_reduce = 1;
 
@@ -251,23 +282,15 @@ int with_bcast_dests(std::vector<gelib_part_desc> &descs, const std::vector<int>
   }
   const size_t tmp_bytes = ((size_t)(cb * G * per_cell) + 255) & ~(size_t)255;
   const size_t need = tmp_bytes + partial;
-  int dev = 0;
-  GELIB_HIP_TRY(hipGetDevice(&dev));
   // held while the kernels of this call are put on the stream: another thread using the same stream's buffer must
   // come entirely before or entirely after them
-  std::lock_guard<std::mutex> lock(g_bcast_mutex);
-  ScratchBuf &buf = g_bcast_scratch[{dev, s}];
-  if (buf.bytes < need) {
-    if (buf.ptr) {
-      forget_ranges(buf.ptr);
-      GELIB_HIP_TRY(hipFree(buf.ptr));  // waits for the kernels that still use it
-    }
-    buf.ptr = nullptr;
-    buf.bytes = 0;
-    GELIB_HIP_TRY(hipMalloc((void **)&buf.ptr, need));
-    buf.bytes = need;
-  }
-  int rc;
+  std::lock_guard<std::mutex> lock(stream_scratch_mutex(0));
+  struct {
+    char *ptr;
+  } buf;
+  int rc = stream_scratch(0, s, need, (void **)&buf.ptr);
+  if (rc) return rc;
+  if (!buf.ptr) return GELIB_HIP_ERR_UNSUPPORTED;  // under stream capture: the caller sums inside the shape-agnostic kernels
   for (long long b0 = 0; b0 < E[0]; b0 += cb) {
     const long long cbn = std::min(cb, E[0] - b0);
     const long long En[3] = {cbn, E[1], E[2]};
@@ -327,9 +350,12 @@ int part_entry(Kind kind, bool diag, const gelib_part_desc *r, const gelib_part_
   hipStream_t s = (hipStream_t)stream;
   if (!g_force_generic && g_bcast_reduce && kind != kFwd && dest_broadcasts(kind == kBack0 ? x : y, op.E)) {
     std::vector<gelib_part_desc> d = {*r, *x, *y};
-    return with_bcast_dests(d, {kind == kBack0 ? 1 : 2}, op.E, accumulate, s, [&](int acc) {
+    rc = with_bcast_dests(d, {kind == kBack0 ? 1 : 2}, op.E, accumulate, s, [&](int acc) {
       return part_entry(kind, diag, &d[0], &d[1], &d[2], offs, acc, stream);
     });
+    if (rc != GELIB_HIP_ERR_UNSUPPORTED) return rc;
+    t_last_path = kPathGeneric;   // no scratch (the call is being recorded into a graph): the serial sum
+    return kind == kBack0 ? launch_generic_back0(op, accumulate != 0, s) : launch_generic_back1(op, accumulate != 0, s);
   }
   if (!g_force_generic) {
     int used = 0;
@@ -743,10 +769,13 @@ int vec_bwd_entry(bool diag, const gelib_part_desc *xg, const gelib_part_desc *y
       if (yg) d.insert(d.end(), yg, yg + ny);
       std::vector<int> dests;
       for (int i = ixg; i < (int)d.size(); i++) dests.push_back(i);
-      return with_bcast_dests(d, dests, plan.E, accumulate, s, [&](int acc) {
+      rc = with_bcast_dests(d, dests, plan.E, accumulate, s, [&](int acc) {
         return vec_bwd_entry(diag, xg ? &d[ixg] : nullptr, yg ? &d[iyg] : nullptr, ng, &d[0], nx, &d[ng], ny, &d[ng + nx],
                              acc, stream);
       });
+      if (rc != GELIB_HIP_ERR_UNSUPPORTED) return rc;
+      // no scratch (the call is being recorded into a graph): the families below decline a destination that
+      // broadcasts, and the shape-agnostic kernels sum it serially
     }
   }
   if (!g_force_generic) {

@@ -4,6 +4,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <mutex>
+
 #include "gelib_hip.h"
 
 namespace gelib_hip {
@@ -50,6 +52,14 @@ int launch_generic_fwd(const PartOp &op, bool accumulate, hipStream_t s);
 int launch_generic_back0(const PartOp &op, bool accumulate, hipStream_t s);  // destination = op.x
 int launch_generic_back1(const PartOp &op, bool accumulate, hipStream_t s);  // destination = op.y
 int launch_zero_fill(const PartDev &d, const long long D[3], int M, int n, hipStream_t s);
+
+// ---- scratch memory that belongs to the library (cabi.cpp): one buffer per (kind, device, stream), allocated on first
+// use, grown when more is asked for, kept until the process ends.  The caller holds stream_scratch_mutex(kind) from
+// the call until the last kernel that uses the buffer is on the stream (kernels of one stream run in order, so the
+// next user of the buffer comes after them).  kind 0: per-cell gradients of a broadcast destination; 1: partial sums of
+// backward launches that deal the pairs of a cell to several blocks.
+int stream_scratch(int kind, hipStream_t s, size_t bytes, void **out);
+std::mutex &stream_scratch_mutex(int kind);
 
 // ---- sums over broadcast dimensions of a gradient destination (bcast_reduce.hip) ----
 // tmp: per-cell gradients packed (E0, E1, E2, rows, n); d: the destination, whose own extents D are E[k] or 1

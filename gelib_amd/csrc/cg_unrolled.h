@@ -53,6 +53,8 @@ struct PairRec {
                      // to powers of two; -1 when that exceeds 2^20
   int lg_n2p;        // log2 of n2p
   int rec_off;       // offset (floats) in the bank of the pair's step records (kernel for operands up to l = kLTMax), or -1
+  int cost_rank;     // position of the pair when the pairs are sorted by falling cost (backward launches that deal the
+                     // pairs of a cell to several blocks take every S-th of that order)
 };
 
 // Helpers shared by the kernel families that need contiguous channels and one cell index (cg_unrolled_plan.cpp).

@@ -368,7 +368,9 @@ unrolled_bwd_kernel(const BwdArgs a) {
   float2 *xacc_all = ys + cpb * ysize;                 // [wave][cell][xsize]
   float2 *yacc_all = xacc_all + kWaves * cpb * xsize;  // [wave][cell][ysize]
 
-  const long long cell0 = (long long)blockIdx.x * cpb;
+  const int nsplit = a.pair_split;  // > 1: this block takes every nsplit-th pair (by cost rank) of its cells
+  const int split = nsplit > 1 ? (int)(blockIdx.x % nsplit) : 0;
+  const long long cell0 = (long long)(nsplit > 1 ? blockIdx.x / nsplit : blockIdx.x) * cpb;
   const long long left = a.ncells - cell0;
   const int ncell = left < cpb ? (int)left : cpb;
   // readfirstlane tells the compiler the wave index is uniform, so everything derived from it (which pair, which
@@ -399,6 +401,7 @@ unrolled_bwd_kernel(const BwdArgs a) {
                   // than waves (few channels, few cells per block) do not leave the same waves idle every time
   for (int pidx = 0; pidx < npairs; pidx++) {
     const PairPtr p = pairs + pidx;
+    if (nsplit > 1 && p->cost_rank % nsplit != split) continue;
     const int nruns = runs_of(pidx);
     CoeffPtr C = (CoeffPtr)(a.bank + p->cg_base);
     const int first = (wave - dealt) & (kWaves - 1);
@@ -428,6 +431,25 @@ unrolled_bwd_kernel(const BwdArgs a) {
   }
 
   __syncthreads();
+  if (nsplit > 1) {
+    // the sums of this block's pairs (the four wave images added in their order) go to the block's slice of the
+    // partial images; unrolled_bwd_sum_splits_kernel adds the slices of a cell and writes the gradients
+    auto park = [&](float2 *part, const float2 *acc, int size) {
+      float2 *dst = part + ((long long)split * a.ncells + cell0) * size;
+      for (int e = threadIdx.x; e < ncell * size; e += kBlock) {
+        float2 v = acc[e];
+        for (int w = 1; w < kWaves; w++) {
+          const float2 t = acc[w * cpb * size + e];
+          v.x += t.x;
+          v.y += t.y;
+        }
+        dst[e] = v;
+      }
+    };
+    if (WX) park(a.part_x, xacc_all, xsize);
+    if (WY) park(a.part_y, yacc_all, ysize);
+    return;
+  }
   if (WX) copy_image<false>(a.xg, a.xrows, a.nx, xacc_all, xsize, cell0, ncell, kWaves, cpb * xsize, a.accumulate != 0);
   if (WY) copy_image<false>(a.yg, a.yrows, a.ny, yacc_all, ysize, cell0, ncell, kWaves, cpb * ysize, a.accumulate != 0);
 }

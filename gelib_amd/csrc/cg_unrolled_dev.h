@@ -45,6 +45,11 @@ struct BwdArgs {
   int xrows[kFastIn], yrows[kFastIn];  // 2l+1 of each x / y part
   int cells_per_block;
   int only_dl;      // -1, or: the call has one triple, l = |l1 - l2| + only_dl (the kernel built for that case)
+  // Launches with few cells: the pairs of a cell are dealt to pair_split blocks (by PairRec::cost_rank), each of which
+  // writes the sums of its pairs into part_x / part_y, [split][cell][packed image of the parts]; a second small kernel
+  // adds the pair_split images of a cell in their order and writes the gradients.  1: one block takes all pairs.
+  int pair_split;
+  float2 *part_x, *part_y;
 };
 
 size_t unrolled_bwd_lds_bytes(int bank_len, int xsize, int ysize, int cells_per_block);
@@ -100,6 +105,8 @@ bool unrolled_bwd_takes(bool diag, bool padded, int lcap, int lop);
 // or -1 when no backward kernel takes the vector
 int unrolled_bwd_cap(int lcap, int lop);
 int launch_unrolled_bwd(const BwdArgs &a, bool diag, int lcap, int lop, int nblocks, size_t lds_bytes, hipStream_t s);
+// adds the pair_split partial images of every cell and writes xg / yg (nblocks = blocks of a.cells_per_block cells)
+int launch_unrolled_bwd_sum_splits(const BwdArgs &a, int nblocks, hipStream_t s);
 // one triple (a.only_dl >= 0), second operand of 16 k channels (k = 1, 2), first operand a power of two >= 16
 size_t one_triple_bwd_lds_bytes(int xsize, int ysize);
 int launch_one_triple_bwd(const BwdArgs &a, int k, int l1, int l2, int l, int nblocks, size_t lds_bytes, hipStream_t s);

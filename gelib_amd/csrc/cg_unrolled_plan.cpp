@@ -19,6 +19,9 @@ int g_fwd_narrow_decline = 1;  // leave products with at most four channel pairs
 int g_fwd_ti = 0;                    // 0 = widest tile that divides every n1, else force 1 / 2 / 4
 int g_bwd_enable = 1;
 int g_bwd_one_enable = 1; // the backward kernel for calls with one triple
+int g_bwd_split = 1;        // backward launches with few cells deal the pairs of a cell to several blocks
+int g_bwd_split_below = 1024;  // ... when the launch would have fewer blocks than this (four per compute unit)
+int g_bwd_split_max = 16;   // ... to at most this many blocks per cell (headline type, 64 cells: 115 us with one block per cell, 43 with 8, 37 with 16, 51 with 25)
 int g_bwd_one_wide = 1;   // ... and the one for a second operand of 16 or 32 channels (0 off, else cells per wave and block)
 long long g_bwd_one_wide_cells = 4096;  // ... in launches with at least this many cells (a wave takes whole cells)
 int g_bwd_l6_enable = 1;  // the backward kernel for operands up to l = 6
@@ -204,6 +207,22 @@ int get_plan(bool diag, const std::vector<VecTriple> &triples, const std::vector
     bank.resize(bank.size() + n);
     cg_matrix_host(t.l1, t.l2, t.l, bank.data() + bank.size() - n);
     p->cg_len = (int)bank.size() - p->cg_base;
+  }
+  {
+    // rank of every pair by falling cost (terms of its triples times lane slots): launches that deal the pairs of a
+    // cell to S blocks give block s the pairs of rank s, s + S, ...
+    std::vector<long long> cost(plan.pairs.size(), 0);
+    for (auto &t : triples) {
+      size_t k = 0;
+      while (k < plan.pairs.size() && !(plan.pairs[k].xi == t.xi && plan.pairs[k].yi == t.yi)) k++;
+      long long terms = 0;
+      for (int m = -t.l; m <= t.l; m++) terms += std::min(t.l1, m + t.l2) - std::max(-t.l1, m - t.l2) + 1;
+      cost[k] += terms * (diag ? plan.pairs[k].n1 : (long long)plan.pairs[k].n1 * plan.pairs[k].n2);
+    }
+    std::vector<int> order(plan.pairs.size());
+    for (size_t k = 0; k < order.size(); k++) order[k] = (int)k;
+    std::stable_sort(order.begin(), order.end(), [&](int a, int b) { return cost[a] > cost[b]; });
+    for (size_t r = 0; r < order.size(); r++) plan.pairs[order[r]].cost_rank = (int)r;
   }
   if (bank.size() % 2) bank.push_back(0.f);
   plan.zero_off = (int)bank.size();
@@ -432,6 +451,30 @@ int run_bwd(bool diag, const std::vector<VecTriple> &triples, const std::vector<
   }
   const long long nblocks = (ncells + cpb - 1) / cpb;
   if (nblocks > 0x7fffffffLL) return GELIB_HIP_ERR_ARG;
+  a.pair_split = 1;
+  // Few cells: a block would walk through all pairs of its cells while most of the GPU idles (L=4, 16 channels, 64
+  // cells: 64 blocks of 25 pairs each, 111 us).  The pairs of a cell are then dealt to several blocks, whose partial
+  // sums a second small kernel adds in a fixed order.
+  if (g_bwd_split && a.only_dl < 0 && a.npairs > 1 && nblocks < g_bwd_split_below) {
+    long long S = std::min<long long>({(long long)g_bwd_split_max, 32LL /* most blocks per cell the summing kernel adds */, (long long)a.npairs,
+                                      (g_bwd_split_below + nblocks - 1) / nblocks});
+    if (S >= 2) {
+      const size_t xbytes = want_x ? sizeof(float2) * (size_t)S * ncells * a.xsize : 0;
+      const size_t ybytes = want_y ? sizeof(float2) * (size_t)S * ncells * a.ysize : 0;
+      std::lock_guard<std::mutex> lock(stream_scratch_mutex(1));
+      void *buf = nullptr;
+      if ((rc = stream_scratch(1, s, xbytes + ybytes, &buf))) return rc;
+      if (buf) {  // none while the call is recorded into a graph: one block per cell then
+        a.pair_split = (int)S;
+        a.part_x = (float2 *)buf;
+        a.part_y = (float2 *)((char *)buf + xbytes);
+        if ((rc = launch_unrolled_bwd(a, diag, lcap, lop, (int)(nblocks * S), lds, s))) return rc;
+        if ((rc = launch_unrolled_bwd_sum_splits(a, (int)nblocks, s))) return rc;
+        *used = 1;
+        return GELIB_HIP_OK;
+      }
+    }
+  }
   rc = launch_unrolled_bwd(a, diag, lcap, lop, (int)nblocks, lds, s);
   if (rc) return rc;
   *used = 1;
@@ -566,6 +609,18 @@ int unrolled_set_option(const char *name, int value) {
   }
   if (!std::strcmp(name, "unrolled_fwd_l6")) {
     g_fwd_l6_enable = value;
+    return GELIB_HIP_OK;
+  }
+  if (!std::strcmp(name, "unrolled_bwd_split")) {
+    g_bwd_split = value;
+    return GELIB_HIP_OK;
+  }
+  if (!std::strcmp(name, "unrolled_bwd_split_below")) {
+    g_bwd_split_below = value > 0 ? value : 1024;
+    return GELIB_HIP_OK;
+  }
+  if (!std::strcmp(name, "unrolled_bwd_split_max")) {
+    g_bwd_split_max = value > 1 ? value : 16;
     return GELIB_HIP_OK;
   }
   if (!std::strcmp(name, "unrolled_bwd_one_wide_cells")) {

@@ -83,6 +83,47 @@ def test_vec_default_path(cabi, case, diag):
     run_vec(cabi, *case, diag, seed=400, force_generic=False)
 
 
+@pytest.mark.parametrize("case", CASES)
+@pytest.mark.parametrize("diag", [False, True])
+def test_vec_without_pair_split(cabi, case, diag):
+    """Launches with few cells (every case here) deal the pairs of a cell to several blocks of the unrolled backward
+    kernels and add their partial sums in a second kernel; with that switched off one block takes all pairs of its
+    cells, as in launches with many cells.  Both ways to the same parity rules; the fixed order of additions makes
+    each of them reproducible bit for bit."""
+    cabi.set_option("unrolled_bwd_split", 0)
+    try:
+        run_vec(cabi, *case, diag, seed=400, force_generic=False)
+    finally:
+        cabi.set_option("unrolled_bwd_split", 1)
+
+
+def test_pair_split_is_reproducible_and_respects_accumulate(cabi):
+    cabi.set_option("force_generic", 0)
+    B, tau = 40, {l: 16 for l in range(5)}
+    xs = [U.seeded(1 + l, B, 2 * l + 1, n) for l, n in tau.items()]
+    ys = [U.seeded(11 + l, B, 2 * l + 1, n) for l, n in tau.items()]
+    O = U.VecOracle(xs, ys, 4, False, gseed=21)
+    dxs, dys, dgs = [U.dev(a) for a in xs], [U.dev(a) for a in ys], [U.dev(a) for a in O.gs]
+    outs = []
+    for smax in (16, 16, 3):
+        cabi.set_option("unrolled_bwd_split_max", smax)
+        dxg = [torch.full(a.shape, 3.0 - 2j, dtype=torch.complex64, device="cuda") for a in xs]
+        dyg = [torch.full(a.shape, 3.0 - 2j, dtype=torch.complex64, device="cuda") for a in ys]
+        cabi.so3vec_bwd(dxg, dyg, dgs, dxs, dys, accumulate=False)
+        assert cabi.last_path() == 2
+        torch.cuda.synchronize()
+        outs.append([U.host(a) for a in dxg + dyg])
+        O.check_bwd(outs[-1][:5], outs[-1][5:], "pair split, at most %d blocks per cell" % smax)
+    cabi.set_option("unrolled_bwd_split_max", 16)
+    assert all(np.array_equal(a, b) for a, b in zip(outs[0], outs[1]))
+    sx = [U.seeded(31 + i, *a.shape) for i, a in enumerate(xs)]
+    sy = [U.seeded(41 + i, *a.shape) for i, a in enumerate(ys)]
+    dxg, dyg = [U.dev(a) for a in sx], [U.dev(a) for a in sy]
+    cabi.so3vec_bwd(dxg, dyg, dgs, dxs, dys, accumulate=True)
+    torch.cuda.synchronize()
+    O.check_bwd_onto([U.host(a) for a in dxg], [U.host(a) for a in dyg], sx, sy, "pair split, accumulate")
+
+
 def test_absent_output_part_keeps_offsets(cabi):
     # a product part that is missing is skipped; the blocks of the other parts stay where they are
     cabi.set_option("force_generic", 0)

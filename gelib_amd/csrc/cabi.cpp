@@ -474,7 +474,7 @@ bool split_diag(const VecPlan &plan, const std::vector<View> &R, const std::vect
         if (p.n != 1) return false;
       return true;
     };
-    if (!all_one(X) && !all_one(Y)) return false;
+    if (all_one(X) == all_one(Y)) return false;   // exactly one narrow side
   }
   bool lo = false, hi = false;
   for (auto &t : plan.triples) (t.l <= kSplit ? lo : hi) = true;

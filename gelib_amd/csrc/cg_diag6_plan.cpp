@@ -84,8 +84,8 @@ int make_args(const VecPlan &plan, const std::vector<const gelib_part_desc *> &r
       return true;
     };
     ybc = all_one(ly);
-    xbc = !ybc && all_one(lx);
-    if (!xbc && !ybc) return GELIB_HIP_OK;
+    xbc = all_one(lx);
+    if (xbc == ybc) return GELIB_HIP_OK;   // exactly one narrow side (one channel on both sides stays where it was)
   }
   const int n = (xbc ? ly : lx)[0].second;
   if (n < 1 || n > kMaxChannels) return GELIB_HIP_OK;

@@ -66,6 +66,7 @@ WORKLOADS = {
     "so3vec_diagcg_L4_n64_B131072": ("vec", 131072, {l: 64 for l in range(5)}, {l: 64 for l in range(5)}, 4, True),
     "so3vec_diagcg_L4_n16_B524288": ("vec", 524288, {l: 16 for l in range(5)}, {l: 16 for l in range(5)}, 4, True),
     "so3vec_cg_L6_tau8_B16384_maxl6": ("vec", 16384, {l: 8 for l in range(7)}, {l: 8 for l in range(7)}, 6, False),
+    "so3vec_cg_L6_tau8_B16384_uncapped": ("vec", 16384, {l: 8 for l in range(7)}, {l: 8 for l in range(7)}, -1, False),
     "so3vec_cg_L4_tau4_B524288_maxl4": ("vec", 524288, {l: 4 for l in range(5)}, {l: 4 for l in range(5)}, 4, False),
     "so3vec_cg_L2_tau64_B8192_maxl2": ("vec", 8192, {l: 64 for l in range(3)}, {l: 64 for l in range(3)}, 2, False),
     "so3vec_diagcg_L4_n64_B131072_uncapped": ("vec", 131072, {l: 64 for l in range(5)}, {l: 64 for l in range(5)}, -1, True),
@@ -80,7 +81,7 @@ OTHER_CONFIGS = [("so3part_cg_1x1to1_n16_B1024", 1024), ("so3part_cg_2x3to4_n32_
 ALIASES = {"cg23": "so3vec_cg_l2_x_l3_n32_B65536_maxl4", "cfg1": "so3part_cg_1x1to1_n16_B1024", "cfg4": "so3vec_cg_L4_tau16_B32768_maxl4", "cfg4u": "so3vec_cg_L4_tau16_B32768_uncapped",
            "cfg2": "so3part_cg_2x3to4_n32_B65536", "cfg3": "so3vec_diagcg_L6_n64_B131072",
            "cfg5": "so3part_cg_10x10_all_l_n8_B16384", "diag4": "so3vec_diagcg_L4_n64_B131072",
-           "diag4n16": "so3vec_diagcg_L4_n16_B524288", "cg6": "so3vec_cg_L6_tau8_B16384_maxl6",
+           "diag4n16": "so3vec_diagcg_L4_n16_B524288", "cg6": "so3vec_cg_L6_tau8_B16384_maxl6", "cg6u": "so3vec_cg_L6_tau8_B16384_uncapped",
            "diag4u": "so3vec_diagcg_L4_n64_B131072_uncapped", "cg2n64": "so3vec_cg_L2_tau64_B8192_maxl2",
            "cg4n4": "so3vec_cg_L4_tau4_B524288_maxl4", "cg10m": "so3vec_cg_l8l10_x_l9l10_tau4_B32768_maxl12"}
 

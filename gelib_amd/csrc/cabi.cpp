@@ -465,9 +465,10 @@ PartOp triple_op(const VecPlan &plan, const VecTriple &t, const std::vector<View
 // A Diag product that reaches above l = 6: the lane-per-channel kernels (built for products up to l = 6) take the
 // triples up to there, the other families the rest.  R is sorted by l, so A keeps a prefix of it and B the remainder.
 // (A CGproduct with a one-channel operand is such a Diag product with the channel repeated, and is split the same way.)
+bool split_at_l6(const VecPlan &plan, const std::vector<View> &R, VecPlan &A, VecPlan &B, std::vector<View> &RA,
+                 std::vector<View> &RB);
 bool split_diag(const VecPlan &plan, const std::vector<View> &R, const std::vector<View> &X, const std::vector<View> &Y,
                 VecPlan &A, VecPlan &B, std::vector<View> &RA, std::vector<View> &RB) {
-  constexpr int kSplit = 6;
   if (!plan.diag) {
     auto all_one = [](const std::vector<View> &v) {
       for (auto &p : v)
@@ -476,6 +477,13 @@ bool split_diag(const VecPlan &plan, const std::vector<View> &R, const std::vect
     };
     if (all_one(X) == all_one(Y)) return false;   // exactly one narrow side
   }
+  return split_at_l6(plan, R, A, B, RA, RB);
+}
+
+// The triples of a plan up to l = 6 (A, with the parts RA) and above (B, RB); false when one of the two is empty.
+bool split_at_l6(const VecPlan &plan, const std::vector<View> &R, VecPlan &A, VecPlan &B, std::vector<View> &RA,
+                 std::vector<View> &RB) {
+  constexpr int kSplit = 6;
   bool lo = false, hi = false;
   for (auto &t : plan.triples) (t.l <= kSplit ? lo : hi) = true;
   if (!lo || !hi) return false;
@@ -518,6 +526,26 @@ int fwd_dispatch(const VecPlan &plan, const std::vector<View> &R, const std::vec
     if (used) {
       t_last_path = kPathUnrolled;
       return GELIB_HIP_OK;
+    }
+    {
+      // A CGproduct of operands above l = 4 that reaches above l = 6 (the API default is uncapped): the unrolled kernel
+      // built for such operands takes the triples up to l = 6, the any-l kernels the rest (different product parts).
+      int lop = 0;
+      for (auto &v : X) lop = std::max(lop, v.l);
+      for (auto &v : Y) lop = std::max(lop, v.l);
+      VecPlan A, B;
+      std::vector<View> RA, RB;
+      if (!plan.diag && lop > 4 && lop <= 6 && split_at_l6(plan, R, A, B, RA, RB)) {
+        std::vector<const gelib_part_desc *> ra;
+        for (auto &v : RA) ra.push_back(v.d);
+        rc = unrolled_vec_fwd(A, ra, xd, yd, accumulate != 0, s, &used);
+        if (rc) return rc;
+        if (used) {
+          rc = fwd_dispatch(B, RB, X, Y, accumulate, s);
+          t_last_path = kPathUnrolled;
+          return rc;
+        }
+      }
     }
     rc = onepair_mfma_vec_fwd(plan, rd, xd, yd, accumulate != 0, s, &used);
     if (rc) return rc;

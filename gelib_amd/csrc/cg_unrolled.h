@@ -16,7 +16,7 @@ namespace gelib_hip {
 
 constexpr int kLT = 4;                // largest operand l handled by the unrolled kernels
 constexpr int kLTMax = 6;             // ... and by the one backward kernel built for operands up to l = 6 (product l <= 6)
-constexpr int kMaxDl = 2 * kLT + 1;   // most l values one (l1,l2) pair can produce
+constexpr int kMaxDl = 2 * kLTMax + 1;  // most l values one (l1,l2) pair can produce
 constexpr int kMaxPairs = (kLTMax + 1) * (kLTMax + 1);  // most (x part, y part) pairs of one launch
 
 struct VecTriple {

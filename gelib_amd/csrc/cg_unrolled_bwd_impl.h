@@ -101,11 +101,14 @@ __device__ __forceinline__ LanePos lane_pos(int run, int lane, int log2_u, int n
 // the code for the other l of the pair is left out.  (The branch-free form reads rows of zeros and multiplies by
 // tables of zeros for the l that are absent: for (2, 3) -> 4 with 32 x 32 channels that is 510 multiply-adds per lane
 // and run where 350 are needed, and 24 row loads where 9 are.)
-template <int L1, int L2, int LCAP, bool DIAG, bool WX, bool WY, bool PAD, bool REC, int ONLY = -1>
+// LLO: the launch takes only the l from LLO up (a product that reaches above l = 6 with operands above l = 4 is taken
+// in two launches, l <= 6 and l >= 7, each reading its own parts of g; the second adds onto the first).
+template <int L1, int L2, int LCAP, bool DIAG, bool WX, bool WY, bool PAD, bool REC, int ONLY = -1, int LLO = 0>
 __device__ __forceinline__ void pair_bwd(const GParts<LCAP> &gp, PairPtr pr, CoeffPtr Cs, CoeffPtr Zc, GlobalRows zrows,
                                          const float2 *xs, const float2 *ys, float2 *xacc, float2 *yacc, int xsize,
                                          int ysize, long long cell0, int offs_add, const LanePos q) {
-  constexpr int DL0 = ONLY >= 0 ? ONLY : 0;  // the pair's tables are indexed by dl = l - |L1 - L2|; the first one used
+  // the pair's tables are indexed by dl = l - |L1 - L2|; the first one used
+  constexpr int DL0 = ONLY >= 0 ? ONLY : (LLO > cabs_(L1 - L2) ? LLO - cabs_(L1 - L2) : 0);
   constexpr int LMIN = cabs_(L1 - L2) + DL0;
   constexpr int LTOP = ONLY >= 0 ? LMIN : cmin_(L1 + L2, LCAP);
   if constexpr (LMIN > LCAP || LMIN > L1 + L2) return;  // no l of this pair can be present
@@ -181,7 +184,7 @@ __device__ __forceinline__ void pair_bwd(const GParts<LCAP> &gp, PairPtr pr, Coe
   // the memory latency), otherwise as many m as fit the budget.  The kernels for l up to 8 hold more sums and are
   // near the register limit of three waves per SIMD already, so their budget is smaller.
   constexpr int kRowBudget =
-      (LCAP <= 4 || ONLY >= 0) ? 32 : LCAP == kLTMax ? ((L1 > kLT || L2 > kLT) ? 16 : 32) : 14;
+      (LCAP <= 4 || ONLY >= 0) ? 32 : (LCAP == kLTMax || LLO > 0) ? ((L1 > kLT || L2 > kLT) ? 16 : 32) : 14;
   constexpr int ROWS = (LTOP + 1) * (LTOP + 1) - LMIN * LMIN;  // sum of 2l+1 over the l of the pair
   constexpr int PF = ROWS <= kRowBudget ? 2 * LTOP + 1 : (kRowBudget / NLP > 1 ? kRowBudget / NLP : 1);
   float2 gq[PF][NLP];
@@ -357,7 +360,7 @@ __device__ __forceinline__ void pair_bwd_one(int only_dl, const GParts<LCAP> &gp
   });
 }
 
-template <int LCAP, bool DIAG, bool WX, bool WY, bool PAD, int LT, bool ONE>
+template <int LCAP, bool DIAG, bool WX, bool WY, bool PAD, int LT, bool ONE, int LLO = 0>
 __global__ void __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(LT > kLT ? 3 : 1)))
 unrolled_bwd_kernel(const BwdArgs a) {
   constexpr int KR = 2 * LCAP + 1;
@@ -411,13 +414,13 @@ unrolled_bwd_kernel(const BwdArgs a) {
       switch (p->l1 * (kLTMax + 1) + p->l2) {
 #define GELIB_CASE(A, B)                                                                                      \
   case A * (kLTMax + 1) + B:                                                                                  \
-    if constexpr (A <= LT && B <= LT) {                                                                       \
+    if constexpr (A <= LT && B <= LT && A + B >= LLO) { /* the pair has an l the launch takes */              \
       if constexpr (ONE)                                                                                      \
         pair_bwd_one<A, B, LCAP, DIAG, WX, WY, PAD>(only_dl, gp, p, C, Zc, zrows, xs, ys, xacc, yacc, xsize, ysize,   \
                                                     cell0, offs_add, q);                                      \
       else                                                                                                    \
-        pair_bwd<A, B, LCAP, DIAG, WX, WY, PAD, (LT > kLT)>(gp, p, C, Zc, zrows, xs, ys, xacc, yacc, xsize, ysize,    \
-                                                              cell0, offs_add, q);                            \
+        pair_bwd<A, B, LCAP, DIAG, WX, WY, PAD, (LT > kLT), -1, LLO>(gp, p, C, Zc, zrows, xs, ys, xacc, yacc, xsize,  \
+                                                                       ysize, cell0, offs_add, q);            \
     }                                                                                                         \
     break;
 #define GELIB_ROW(A) \
@@ -454,9 +457,9 @@ unrolled_bwd_kernel(const BwdArgs a) {
   if (WY) copy_image<false>(a.yg, a.yrows, a.ny, yacc_all, ysize, cell0, ncell, kWaves, cpb * ysize, a.accumulate != 0);
 }
 
-template <int LCAP, bool DIAG, bool WX, bool WY, bool PAD, int LT, bool ONE>
+template <int LCAP, bool DIAG, bool WX, bool WY, bool PAD, int LT, bool ONE, int LLO>
 int launch_variant(const BwdArgs &a, int nblocks, size_t lds, hipStream_t s) {
-  auto kern = unrolled_bwd_kernel<LCAP, DIAG, WX, WY, PAD, LT, ONE>;
+  auto kern = unrolled_bwd_kernel<LCAP, DIAG, WX, WY, PAD, LT, ONE, LLO>;
   static bool attr_set = false;  // benign race: setting the attribute twice is harmless
   if (!attr_set) {
     GELIB_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -469,13 +472,13 @@ int launch_variant(const BwdArgs &a, int nblocks, size_t lds, hipStream_t s) {
 }
 
 // want_x / want_y select which gradients are computed
-template <int LCAP, bool DIAG, bool PAD, int LT = kLT, bool ONE = false>
+template <int LCAP, bool DIAG, bool PAD, int LT = kLT, bool ONE = false, int LLO = 0>
 int launch_bwd_variants(const BwdArgs &a, int nblocks, size_t lds_bytes, hipStream_t s) {
   static_assert(kLTMax == 6 && LT <= kLTMax, "the case table above lists l1, l2 = 0..6");
   const bool wx = a.want_x != 0, wy = a.want_y != 0;
-  if (wx && wy) return launch_variant<LCAP, DIAG, true, true, PAD, LT, ONE>(a, nblocks, lds_bytes, s);
-  if (wx) return launch_variant<LCAP, DIAG, true, false, PAD, LT, ONE>(a, nblocks, lds_bytes, s);
-  return launch_variant<LCAP, DIAG, false, true, PAD, LT, ONE>(a, nblocks, lds_bytes, s);
+  if (wx && wy) return launch_variant<LCAP, DIAG, true, true, PAD, LT, ONE, LLO>(a, nblocks, lds_bytes, s);
+  if (wx) return launch_variant<LCAP, DIAG, true, false, PAD, LT, ONE, LLO>(a, nblocks, lds_bytes, s);
+  return launch_variant<LCAP, DIAG, false, true, PAD, LT, ONE, LLO>(a, nblocks, lds_bytes, s);
 }
 
 }  // namespace

@@ -100,10 +100,11 @@ bool unrolled_fwd_takes(bool diag, int ti, int lcap, int lop);
 int launch_unrolled_fwd(const FwdArgs &a, bool diag, int ti, int lcap, int lop, int nblocks, size_t lds_bytes, hipStream_t s);
 // lcap: largest l present in the gradient; lop: largest l of an operand (above kLT: the kernel for l up to kLTMax, which
 // exists for CGproduct with power-of-two channel counts and lcap <= kLTMax only -- unrolled_bwd_takes says so)
-bool unrolled_bwd_takes(bool diag, bool padded, int lcap, int lop);
+bool unrolled_bwd_takes(bool diag, bool padded, int lcap, int lop, int llo);
 // largest l the backward kernel that launch_unrolled_bwd picks has code for (its step records are laid out for it),
 // or -1 when no backward kernel takes the vector
-int unrolled_bwd_cap(int lcap, int lop);
+int unrolled_bwd_cap(int lcap, int lop, int llo);
+int unrolled_bwd_lo(int lcap, int lop, int llo);   // ... and the smallest (llo: smallest l present in the gradient)
 int launch_unrolled_bwd(const BwdArgs &a, bool diag, int lcap, int lop, int nblocks, size_t lds_bytes, hipStream_t s);
 // adds the pair_split partial images of every cell and writes xg / yg (nblocks = blocks of a.cells_per_block cells)
 int launch_unrolled_bwd_sum_splits(const BwdArgs &a, int nblocks, hipStream_t s);

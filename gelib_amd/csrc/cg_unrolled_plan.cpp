@@ -19,6 +19,7 @@ int g_fwd_narrow_decline = 1;  // leave products with at most four channel pairs
 int g_fwd_ti = 0;                    // 0 = widest tile that divides every n1, else force 1 / 2 / 4
 int g_bwd_enable = 1;
 int g_bwd_one_enable = 1; // the backward kernel for calls with one triple
+int g_bwd_l6_split = 1;     // operands above l = 4, product above l = 6: two launches of the unrolled kernels (l <= 6, l >= 7)
 int g_bwd_split = 1;        // backward launches with few cells deal the pairs of a cell to several blocks
 int g_bwd_split_below = 1024;  // ... when the launch would have fewer blocks than this (four per compute unit)
 int g_bwd_split_max = 16;   // ... to at most this many blocks per cell (headline type, 64 cells: 115 us with one block per cell, 43 with 8, 37 with 16, 51 with 25)
@@ -112,16 +113,17 @@ namespace {
 
 // Step records for the backward kernels: for every pair, one record per (m1,m2) step in the order the kernel runs
 // them (row number m = m1 + m2 rising from -ltop, m1 rising inside a row), holding C_l[m1,m2] for
-// l = |l1-l2| .. ltop = min(l1+l2, cap) -- zero where the part is absent or l < |m| -- padded to a power of two floats.
+// l = max(|l1-l2|, lo) .. ltop = min(l1+l2, cap) -- zero where the part is absent or l < |m| -- padded to a power of two floats.
 // cap is the largest l the kernel that will run has code for (unrolled_bwd_cap).  A pair's records start on a 64-byte
 // boundary of the device allocation and are padded to whole 64-byte groups, the unit the kernel loads.
-void append_step_records(bool diag, int cap, size_t pair_bytes, std::vector<PairRec> *pairs, std::vector<float> *bank) {
+void append_step_records(bool diag, int cap, int lo, size_t pair_bytes, std::vector<PairRec> *pairs, std::vector<float> *bank) {
   (void)diag;
   for (auto &p : *pairs) p.rec_off = -1;
   if (cap < 0) return;
   while ((pair_bytes + bank->size() * sizeof(float)) % 64) bank->push_back(0.f);
   for (auto &p : *pairs) {
-    const int lmin = std::abs(p.l1 - p.l2), ltop = std::min(p.l1 + p.l2, cap);
+    const int lmin = std::max(std::abs(p.l1 - p.l2), lo), ltop = std::min(p.l1 + p.l2, cap);
+    const int dl0 = lmin - std::abs(p.l1 - p.l2);   // the pair's tables are indexed from |l1 - l2|
     if (lmin > ltop) continue;
     const int nl = ltop - lmin + 1, w2 = 2 * p.l2 + 1;
     int recw = 1;
@@ -132,8 +134,8 @@ void append_step_records(bool diag, int cap, size_t pair_bytes, std::vector<Pair
         const int m2 = m - m1;
         for (int dl = 0; dl < recw; dl++) {
           float c = 0.f;
-          if (dl < nl && dl < kMaxDl && p.ri[dl] >= 0 && lmin + dl >= std::abs(m))
-            c = (*bank)[p.cg_base + p.cg[dl] + (m1 + p.l1) * w2 + (m2 + p.l2)];
+          if (dl < nl && dl0 + dl < kMaxDl && p.ri[dl0 + dl] >= 0 && lmin + dl >= std::abs(m))
+            c = (*bank)[p.cg_base + p.cg[dl0 + dl] + (m1 + p.l1) * w2 + (m2 + p.l2)];
           bank->push_back(c);
         }
       }
@@ -229,9 +231,9 @@ int get_plan(bool diag, const std::vector<VecTriple> &triples, const std::vector
   bank.resize(bank.size() + (2 * kLTMax + 1) * (2 * kLTMax + 1) + 1, 0.f);
   const size_t pair_bytes = plan.pairs.size() * sizeof(PairRec);
   {
-    int lcap = 0, lop = 0;
-    for (auto &t : triples) lcap = std::max(lcap, t.l), lop = std::max(lop, std::max(t.l1, t.l2));
-    append_step_records(diag, unrolled_bwd_cap(lcap, lop), pair_bytes, &plan.pairs, &bank);
+    int lcap = 0, lop = 0, llo = 1 << 30;
+    for (auto &t : triples) lcap = std::max(lcap, t.l), lop = std::max(lop, std::max(t.l1, t.l2)), llo = std::min(llo, t.l);
+    append_step_records(diag, unrolled_bwd_cap(lcap, lop, llo), unrolled_bwd_lo(lcap, lop, llo), pair_bytes, &plan.pairs, &bank);
   }
   plan.bank_len = (int)bank.size();
   const size_t bank_bytes = bank.size() * sizeof(float);
@@ -360,14 +362,15 @@ int run_bwd(bool diag, const std::vector<VecTriple> &triples, const std::vector<
             const std::vector<std::pair<int, int>> &ys, const std::vector<int> &rls, const FastLists &f,
             long long ncells, int offs_add, bool accumulate, bool want_x, bool want_y, hipStream_t s, int *used) {
   *used = 0;
-  int lcap = 0, lop = 0;
+  int lcap = 0, lop = 0, llo = 1 << 30;
   bool padded = false;
   for (auto &t : triples) {
     lcap = std::max(lcap, t.l);
+    llo = std::min(llo, t.l);
     lop = std::max(lop, std::max(t.l1, t.l2));
     padded = padded || !is_pow2(xs[t.xi].second) || (!diag && !is_pow2(ys[t.yi].second));
   }
-  if (!unrolled_bwd_takes(diag, padded, lcap, lop) || (lop > kLT && !g_bwd_l6_enable)) return GELIB_HIP_OK;
+  if (!unrolled_bwd_takes(diag, padded, lcap, lop, llo) || (lop > kLT && !g_bwd_l6_enable)) return GELIB_HIP_OK;
   // lane slots are the channel counts rounded up to powers of two; the reduced operand must fit a wave
   int u_min = 1 << 30;
   for (auto &t : triples) {
@@ -566,6 +569,39 @@ int unrolled_vec_bwd(const VecPlan &plan, const std::vector<const gelib_part_des
   std::vector<int> rls;
   for (auto &v : rs) rls.push_back(v.first);
   const long long ncells = plan.E[0] * plan.E[1] * plan.E[2];
+  // A CGproduct of operands above l = 4 that reaches above l = 6 (the API default is uncapped): the triples up to l = 6
+  // run on the kernel built for them, the rest on the one built for l = 7..12, which adds onto what the first wrote.
+  // Each launch reads its own parts of g, so g is still read once.
+  {
+    int lcap = 0, lop = 0, llo = 1 << 30;
+    bool padded = false;
+    for (auto &t : plan.triples) {
+      lcap = std::max(lcap, t.l), llo = std::min(llo, t.l), lop = std::max(lop, std::max(t.l1, t.l2));
+      padded = padded || !is_pow2(xs[t.xi].second) || !is_pow2(ys[t.yi].second);
+    }
+    if (!plan.diag && !padded && g_bwd_l6_enable && g_bwd_l6_split && lop > kLT && lop <= kLTMax && llo <= kLTMax &&
+        lcap > kLTMax && lcap <= 2 * kLTMax) {
+      std::vector<VecTriple> ta, tb;
+      std::vector<int> rla, rlb, map_a(rls.size(), -1), map_b(rls.size(), -1);
+      FastLists fa = f, fb = f;
+      fa.r.clear();
+      fb.r.clear();
+      for (size_t k = 0; k < rls.size(); k++) {
+        if (rls[k] <= kLTMax) map_a[k] = (int)rla.size(), rla.push_back(rls[k]), fa.r.push_back(f.r[k]);
+        else map_b[k] = (int)rlb.size(), rlb.push_back(rls[k]), fb.r.push_back(f.r[k]);
+      }
+      for (auto t : plan.triples) {
+        if (t.l <= kLTMax) t.ri = map_a[t.ri], ta.push_back(t);
+        else t.ri = map_b[t.ri], tb.push_back(t);
+      }
+      int rc = run_bwd(false, ta, xs, ys, rla, fa, ncells, 0, accumulate, !xg.empty(), !yg.empty(), s, used);
+      if (rc || !*used) return rc;
+      int used_b = 0;
+      rc = run_bwd(false, tb, xs, ys, rlb, fb, ncells, 0, true, !xg.empty(), !yg.empty(), s, &used_b);
+      if (rc) return rc;
+      return used_b ? GELIB_HIP_OK : GELIB_HIP_ERR_ARG;   // the same operands and cells: what took the first part takes the second
+    }
+  }
   return run_bwd(plan.diag, plan.triples, xs, ys, rls, f, ncells, 0, accumulate, !xg.empty(), !yg.empty(), s, used);
 }
 
@@ -609,6 +645,10 @@ int unrolled_set_option(const char *name, int value) {
   }
   if (!std::strcmp(name, "unrolled_fwd_l6")) {
     g_fwd_l6_enable = value;
+    return GELIB_HIP_OK;
+  }
+  if (!std::strcmp(name, "unrolled_bwd_l6_split")) {
+    g_bwd_l6_split = value;
     return GELIB_HIP_OK;
   }
   if (!std::strcmp(name, "unrolled_bwd_split")) {

@@ -124,6 +124,24 @@ def test_pair_split_is_reproducible_and_respects_accumulate(cabi):
     O.check_bwd_onto([U.host(a) for a in dxg], [U.host(a) for a in dyg], sx, sy, "pair split, accumulate")
 
 
+@pytest.mark.parametrize("case", [
+    (3, {l: 8 for l in range(7)}, {l: 8 for l in range(7)}, -1),       # L = 6 uncapped: product l up to 12
+    (4, {2: 4, 5: 8, 6: 2}, {3: 4, 6: 4}, 9),                          # parts missing, capped between 6 and 12
+    (2, {6: 16}, {6: 4}, -1),                                          # one pair, l = 0..12
+    (5, {0: 2, 5: 2}, {1: 4, 6: 1}, 11),
+])
+def test_operands_above_l4_product_above_l6(cabi, case):
+    """CGproduct of operands up to l = 6 that reaches above l = 6: the triples up to l = 6 on the unrolled kernels built
+    for them, the rest forward on the any-l kernels and backward on the unrolled instantiation for l = 7..12, which adds
+    onto the first launch's gradients; g is read once."""
+    assert run_vec(cabi, *case, False, seed=520, force_generic=False) == (2, 2)
+    cabi.set_option("unrolled_bwd_l6_split", 0)
+    try:
+        assert run_vec(cabi, *case, False, seed=520, force_generic=False)[1] != 2     # the striped any-l kernels
+    finally:
+        cabi.set_option("unrolled_bwd_l6_split", 1)
+
+
 def test_absent_output_part_keeps_offsets(cabi):
     # a product part that is missing is skipped; the blocks of the other parts stay where they are
     cabi.set_option("force_generic", 0)

@@ -338,6 +338,25 @@ def fused_linear_bench(torch, args):
 
     fused_ms, fused_wall = timed(fused)
     two_ms, _ = timed(two_step)
+    # backward: the bounded-memory entry point (the product and its gradient exist for one chunk of the batch at a time,
+    # in an 8 GiB workspace) beside the four separate calls on full-size buffers
+    gouts = seeded_parts(torch, 404, B, {l: n_out for l in tr}, dev)
+    xg, yg = [torch.empty_like(t) for t in xs], [torch.empty_like(t) for t in ys]
+    wg = [torch.empty_like(w) for w in ws]
+
+    def chunked_bwd():
+        assert cabi.so3vec_cg_linear_bwd(xg, yg, wg, gouts, xs, ys, ws, accumulate=False, workspace_bytes=8 << 30)
+
+    def four_calls_bwd():
+        cabi.so3vec_fwd(prod, xs, ys, accumulate=False)
+        for w_g, p, g in zip(wg, prod, gouts):
+            cabi.part_mix_channels_wgrad(w_g, p, g)
+        for p, g, w in zip(prod, gouts, ws):
+            cabi.part_mix_channels(p, g, w, adjoint=True)
+        cabi.so3vec_bwd(xg, yg, prod, xs, ys, accumulate=False)
+
+    bwd_ms, _ = timed(chunked_bwd)
+    bwd4_ms, _ = timed(four_calls_bwd)
     # terms (m1, m2) of one channel of every (l1, l2, l) block
     terms = sum(1 for l1 in tx for l2 in tx for l in range(abs(l1 - l2), min(l1 + l2, 4) + 1)
                 for m in range(-l, l + 1) for m1 in range(-l1, l1 + 1) if abs(m - m1) <= l2)
@@ -351,6 +370,8 @@ def fused_linear_bench(torch, args):
            "dtype": "f32", "data": "synthetic",
            "config": {"workload": FUSED_WORKLOAD, "batch": B, "tau_x": tx, "tau_y": tx, "maxl": 4, "tau_product": tr,
                       "n_out": n_out, "fused_fwd_ms": fused_ms, "two_step_fwd_ms": two_ms,
+                      "bwd_bounded_memory_ms": bwd_ms, "bwd_four_calls_full_size_ms": bwd4_ms,
+                      "bwd_workspace_bytes": 8 << 30, "fwd_bwd_ms": fused_ms + bwd_ms,
                       "speedup_over_two_step": two_ms / fused_ms,
                       "product_bytes_never_stored": product_bytes,
                       "flops": {"product": flops_product, "mixing": flops_mix}},

@@ -95,8 +95,11 @@ class SO3linear(torch.nn.Module):
 
 class CGproductLinearFn(torch.autograd.Function):
     """CGproduct(x, y, maxl) * W with the product formed and consumed inside one kernel (forward).  The backward pass
-    forms the product again, through the unfused functions, and differentiates those: nothing of the product's size is
+    forms the product again, a chunk of the batch at a time (gelib_hip_so3vec_cg_linear_bwd): the product and its gradient
+    exist only for the chunk at hand, in a workspace of at most BWD_WORKSPACE_BYTES, and nothing of the product's size is
     kept between the two passes."""
+
+    BWD_WORKSPACE_BYTES = 8 << 30   # headline type, 32768 cells: 34.6 ms with 1 GiB, 24.5 with 4, 22.0 with 8, 19.5 with 28 (one chunk)
 
     @staticmethod
     def forward(ctx, k1, k2, maxl, *args):
@@ -113,9 +116,21 @@ class CGproductLinearFn(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, *gargs):
+        from gelib_amd import cabi
         from gelib_amd.SO3vec import SO3vec
         k1, k2 = ctx.k1, ctx.k2
-        leaves = [t.detach().requires_grad_() for t in ctx.saved_tensors]
+        saved = ctx.saved_tensors
+        xs, ys, ws = list(saved[0:k1]), list(saved[k1:k1 + k2]), list(saved[k1 + k2:])
+        need = ctx.needs_input_grad[3:]
+        gs = [g.contiguous() for g in gargs]
+        xg = [torch.empty_like(t, memory_format=torch.contiguous_format) for t in xs] if any(need[0:k1]) else None
+        yg = [torch.empty_like(t, memory_format=torch.contiguous_format) for t in ys] if any(need[k1:k1 + k2]) else None
+        wg = [torch.empty_like(t, memory_format=torch.contiguous_format) for t in ws] if any(need[k1 + k2:]) else None
+        if cabi.so3vec_cg_linear_bwd(xg, yg, wg, gs, xs, ys, ws, accumulate=False,
+                                     workspace_bytes=CGproductLinearFn.BWD_WORKSPACE_BYTES):
+            grads = (xg or [None] * k1) + (yg or [None] * k2) + (wg or [None] * len(ws))
+            return tuple([None, None, None] + [g if n else None for g, n in zip(grads, need)])
+        leaves = [t.detach().requires_grad_() for t in saved]
         with torch.enable_grad():
             x, y = SO3vec(*leaves[0:k1]), SO3vec(*leaves[k1:k1 + k2])
             out = x.CGproduct(y, ctx.maxl) * SO3weights(*leaves[k1 + k2:])

@@ -20,6 +20,7 @@ SYMBOLS = [
     "gelib_hip_gather_map_destroy", "gelib_hip_part_gather", "gelib_hip_part_mix_channels",
     "gelib_hip_part_mix_channels_static", "gelib_hip_part_mix_channels_wgrad", "gelib_hip_part_mix_workspace_bytes",
     "gelib_hip_so3vec_cg_linear_fwd", "gelib_hip_so3vec_cg_linear_workspace_bytes",
+    "gelib_hip_so3vec_cg_linear_bwd", "gelib_hip_so3vec_cg_linear_bwd_workspace_bytes",
     "gelib_hip_set_option",
     "gelib_hip_last_path",
     "gelib_hip_malloc", "gelib_hip_free", "gelib_hip_memcpy", "gelib_hip_memset", "gelib_hip_synchronize",
@@ -85,6 +86,12 @@ def lib():
         L.gelib_hip_so3vec_cg_linear_fwd.argtypes = [ctypes.c_int, P, ctypes.c_int, P, ctypes.c_int, P,
                                                      ctypes.POINTER(ctypes.c_void_p), ctypes.c_int, ctypes.c_void_p,
                                                      ctypes.c_uint64, ctypes.c_void_p]
+        L.gelib_hip_so3vec_cg_linear_bwd.argtypes = [P, P, ctypes.c_void_p, ctypes.c_int, P, ctypes.c_int, P, ctypes.c_int, P,
+                                                     ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p, ctypes.c_uint64,
+                                                     ctypes.c_void_p]
+        L.gelib_hip_so3vec_cg_linear_bwd_workspace_bytes.restype = ctypes.c_uint64
+        L.gelib_hip_so3vec_cg_linear_bwd_workspace_bytes.argtypes = [ctypes.c_int, P, ctypes.c_int, P, ctypes.c_int, P,
+                                                                     ctypes.c_int64]
         L.gelib_hip_so3vec_cg_linear_workspace_bytes.restype = ctypes.c_uint64
         L.gelib_hip_so3vec_cg_linear_workspace_bytes.argtypes = [ctypes.c_int, P, ctypes.c_int, P, ctypes.c_int, P]
         L.gelib_hip_part_mix_workspace_bytes.restype = ctypes.c_uint64
@@ -212,6 +219,33 @@ def so3vec_cg_linear_fwd(rparts, xparts, yparts, wparts, accumulate=False):
     wp = (ctypes.c_void_p * len(wparts))(*[w.data_ptr() for w in wparts])
     rc = L.gelib_hip_so3vec_cg_linear_fwd(len(rparts), ra, len(xparts), xa, len(yparts), ya, wp, int(accumulate),
                                           ctypes.c_void_p(ws.data_ptr()), nbytes, _stream(rparts[0]))
+    if rc == UNSUPPORTED:
+        return False
+    check(rc)
+    return True
+
+
+def so3vec_cg_linear_bwd(xgparts, ygparts, wgparts, gparts, xparts, yparts, wparts, accumulate=False,
+                         workspace_bytes=1 << 30):
+    """Gradients of CGproduct(x, y) @ W with respect to x, y and the matrices (any of the three lists may be None), given
+    the gradient gparts of the result, in the memory of one chunk of the batch: the product and its gradient exist only
+    for the chunk at hand, in a workspace of at most workspace_bytes (more when one batch entry needs more).  False
+    (nothing launched) when the shapes are not ones the call takes."""
+    import torch
+    L = lib()
+    ga, xa, ya = _arr(gparts), _arr(xparts), _arr(yparts)
+    args = (len(gparts), ga, len(xparts), xa, len(yparts), ya)
+    whole = int(L.gelib_hip_so3vec_cg_linear_bwd_workspace_bytes(*args, 0))
+    if whole == 0:
+        return False
+    one = int(L.gelib_hip_so3vec_cg_linear_bwd_workspace_bytes(*args, 1))
+    nbytes = whole if whole <= workspace_bytes else max(one, workspace_bytes)
+    ws = torch.empty(nbytes + 256, dtype=torch.uint8, device=gparts[0].device)
+    base = (ws.data_ptr() + 255) & ~255
+    wp = (ctypes.c_void_p * len(wparts))(*[w.data_ptr() for w in wparts])
+    wgp = (ctypes.c_void_p * len(wgparts))(*[w.data_ptr() for w in wgparts]) if wgparts is not None else None
+    rc = L.gelib_hip_so3vec_cg_linear_bwd(_arr(xgparts), _arr(ygparts), wgp, len(gparts), ga, len(xparts), xa, len(yparts),
+                                          ya, wp, int(accumulate), ctypes.c_void_p(base), nbytes, _stream(gparts[0]))
     if rc == UNSUPPORTED:
         return False
     check(rc)

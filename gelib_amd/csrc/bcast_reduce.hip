@@ -95,7 +95,28 @@ int choose_ranges(long long dcells, int elems, int Rn) {
   return (int)std::max<long long>(1, P);
 }
 
+// dst[i] (+)= src[i]
+__global__ void __launch_bounds__(256) add_into_kernel(float2 *dst, const float2 *src, long long n, int accumulate) {
+  for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long long)gridDim.x * blockDim.x) {
+    float2 v = src[i];
+    if (accumulate) {
+      const float2 o = dst[i];
+      v.x += o.x;
+      v.y += o.y;
+    }
+    dst[i] = v;
+  }
+}
+
 }  // namespace
+
+int launch_add_into(float2 *dst, const float2 *src, long long n, bool accumulate, hipStream_t s) {
+  if (n <= 0) return GELIB_HIP_OK;
+  hipLaunchKernelGGL(add_into_kernel, dim3((unsigned)std::min<long long>((n + 255) / 256, 1 << 16)), dim3(256), 0, s, dst, src,
+                     n, accumulate ? 1 : 0);
+  GELIB_HIP_TRY(hipGetLastError());
+  return GELIB_HIP_OK;
+}
 
 size_t bcast_partial_bytes(const long long E[3], const long long D[3], int rows, int n) {
   long long dcells = D[0] * D[1] * D[2], Rn = 1;

@@ -21,6 +21,8 @@ using namespace gelib_hip;
 
 namespace gelib_hip {
 
+int launch_add_into(float2 *dst, const float2 *src, long long n, bool accumulate, hipStream_t s);  // bcast_reduce.hip
+
 namespace {
 thread_local std::string t_last_error;
 thread_local int t_last_path = kPathNone;
@@ -885,6 +887,177 @@ int linear_fwd_entry(int nr, const gelib_part_desc *r, int nx, const gelib_part_
   return GELIB_HIP_OK;
 }
 
+
+// ---- backward of CGproduct followed by the weight matrices, in bounded memory ------------------------------------
+// out_l = P_l W_l with P = CGproduct(x, y):  xg, yg = the product's backward pass on gP_l = gout_l W_l^H, and
+// wg_l = sum over the rows of P_l^H gout_l.  Neither P nor gP is ever held at full size: the batch is taken in chunks
+// whose product fits the caller's workspace; a chunk's product is formed by the forward kernels, read by the
+// matrix-gradient kernel, overwritten in place by gP and read once more by the backward kernels.
+struct LinBwdShape {
+  std::vector<View> G, X, Y, XG, YG;
+  VecPlan plan;
+  std::vector<long long> tau;     // channels of the product's parts, indexed like G
+  long long rows_per_batch = 0;   // sum over l of grid cells * (2l+1)
+  long long G01 = 1;              // grid cells per batch entry
+};
+
+size_t lin_bwd_bytes(const LinBwdShape &sh, long long cb, size_t *p_bytes, size_t *mix_bytes, size_t *wg_ws_bytes,
+                     size_t *wg_tmp_bytes) {
+  size_t pb = 0, mb = 0, wb = 0, tb = 0;
+  for (size_t k = 0; k < sh.G.size(); k++) {
+    const long long rows = cb * sh.G01 * (2 * sh.G[k].l + 1);
+    pb += (((size_t)rows * sh.tau[k] * sizeof(float2)) + 255) & ~(size_t)255;
+    mb = std::max(mb, mix_workspace_bytes(sh.G[k].n, (int)sh.tau[k]));
+    wb = std::max(wb, mix_wgrad_workspace_bytes(rows, (int)sh.tau[k], sh.G[k].n));
+    tb = std::max(tb, (size_t)sh.tau[k] * sh.G[k].n * sizeof(float2));
+  }
+  auto up = [](size_t v) { return (v + 255) & ~(size_t)255; };
+  if (p_bytes) *p_bytes = pb;
+  if (mix_bytes) *mix_bytes = up(mb);
+  if (wg_ws_bytes) *wg_ws_bytes = up(wb);
+  if (wg_tmp_bytes) *wg_tmp_bytes = up(tb);
+  return pb + up(mb) + up(wb) + up(tb);
+}
+
+// validation shared by the size query and the call; g: the gradient of the output (nr parts, n_out_l channels)
+int lin_bwd_shape(int ng, const gelib_part_desc *g, int nx, const gelib_part_desc *x, int ny, const gelib_part_desc *y,
+                  const gelib_part_desc *xg, const gelib_part_desc *yg, LinBwdShape &sh) {
+  int rc;
+  if ((rc = sort_parts(ng, g, kMaxOutParts, sh.G)) || (rc = sort_parts(nx, x, kMaxParts, sh.X)) ||
+      (rc = sort_parts(ny, y, kMaxParts, sh.Y)))
+    return rc;
+  if (xg && (rc = sort_parts(nx, xg, kMaxParts, sh.XG))) return rc;
+  if (yg && (rc = sort_parts(ny, yg, kMaxParts, sh.YG))) return rc;
+  for (size_t i = 0; i < sh.XG.size(); i++)
+    if (sh.XG[i].l != sh.X[i].l || sh.XG[i].n != sh.X[i].n) return GELIB_HIP_ERR_PARTS;
+  for (size_t i = 0; i < sh.YG.size(); i++)
+    if (sh.YG[i].l != sh.Y[i].l || sh.YG[i].n != sh.Y[i].n) return GELIB_HIP_ERR_PARTS;
+  if (sh.G.empty() || sh.X.empty() || sh.Y.empty()) return GELIB_HIP_ERR_UNSUPPORTED;
+  if ((rc = build_vec_plan(false, sh.G, sh.X, sh.Y, sh.plan, false))) return rc;
+  {
+    std::vector<const gelib_part_desc *> all;
+    for (auto *L : {&sh.G, &sh.X, &sh.Y, &sh.XG, &sh.YG})
+      for (auto &v : *L) all.push_back(v.d);
+    if ((rc = reconcile(all.data(), (int)all.size(), sh.plan.E))) return rc;
+  }
+  sh.tau = product_channels(sh.plan, sh.G.size());
+  sh.G01 = sh.plan.E[1] * sh.plan.E[2];
+  // what the matrix kernels need: every tensor with the full leading extents, gout packed so that its rows (cell, m) are
+  // one stride apart, even channel counts on both sides of every matrix
+  for (auto *L : {&sh.G, &sh.X, &sh.Y, &sh.XG, &sh.YG})
+    for (auto &v : *L)
+      for (int k = 0; k < 3; k++)
+        if (v.d->dims[k] != sh.plan.E[k]) return GELIB_HIP_ERR_UNSUPPORTED;
+  for (size_t k = 0; k < sh.G.size(); k++) {
+    const gelib_part_desc *d = sh.G[k].d;
+    const long long rows_cell = 2 * sh.G[k].l + 1;
+    if (d->strides[4] != 1 || (d->strides[3] & 1) || d->strides[3] < d->dims[4]) return GELIB_HIP_ERR_UNSUPPORTED;
+    if (d->dims[2] > 1 && d->strides[2] != rows_cell * d->strides[3]) return GELIB_HIP_ERR_UNSUPPORTED;
+    if (d->dims[1] > 1 && d->strides[1] != d->dims[2] * rows_cell * d->strides[3]) return GELIB_HIP_ERR_UNSUPPORTED;
+    if (d->dims[0] > 1 && d->strides[0] != d->dims[1] * d->dims[2] * rows_cell * d->strides[3]) return GELIB_HIP_ERR_UNSUPPORTED;
+    if (((uintptr_t)d->ptr & 15) || (sh.G[k].n & 1) || (sh.tau[k] & 1) || sh.tau[k] == 0 || sh.G[k].n == 0 ||
+        sh.tau[k] > 0x7fffffffLL)
+      return GELIB_HIP_ERR_UNSUPPORTED;
+  }
+  return GELIB_HIP_OK;
+}
+
+int linear_bwd_entry(const gelib_part_desc *xg, const gelib_part_desc *yg, void *const *wg, int ng,
+                     const gelib_part_desc *g, int nx, const gelib_part_desc *x, int ny, const gelib_part_desc *y,
+                     const void *const *w, int accumulate, void *workspace, uint64_t workspace_bytes, void *stream) {
+  t_last_path = kPathNone;
+  if (!xg && !yg && !wg) return GELIB_HIP_OK;
+  if (!w) return GELIB_HIP_ERR_NULL;
+  LinBwdShape sh;
+  int rc = lin_bwd_shape(ng, g, nx, x, ny, y, xg, yg, sh);
+  if (rc) return rc;
+  for (auto *L : {&sh.XG, &sh.YG})
+    for (auto &v : *L)
+      if ((rc = check_dest(v.d))) return rc;
+  for (auto *L : {&sh.G, &sh.X, &sh.Y, &sh.XG, &sh.YG})
+    for (auto &v : *L)
+      if ((rc = check_pointer(v.d))) return rc;
+  std::vector<const float2 *> W(sh.G.size());
+  std::vector<float2 *> WG(sh.G.size(), nullptr);
+  for (size_t k = 0; k < sh.G.size(); k++) {
+    const size_t orig = sh.G[k].d - g;   // position in the caller's order, which w and wg follow
+    W[k] = (const float2 *)w[orig];
+    if (wg) WG[k] = (float2 *)wg[orig];
+    if (!W[k] || (wg && !WG[k])) return GELIB_HIP_ERR_NULL;
+    const int64_t wd[5] = {sh.tau[k], 1, 1, 1, sh.G[k].n}, wst[5] = {sh.G[k].n, 0, 0, 0, 1};
+    if ((rc = check_range(W[k], wd, wst, 2 * sizeof(float)))) return rc;
+    if (wg && (rc = check_range(WG[k], wd, wst, 2 * sizeof(float)))) return rc;
+  }
+  const long long E0 = sh.plan.E[0];
+  if (E0 * sh.G01 == 0) return GELIB_HIP_OK;
+  if (!workspace || ((uintptr_t)workspace & 255)) return GELIB_HIP_ERR_WORKSPACE;
+  const int64_t sd[5] = {(int64_t)workspace_bytes, 1, 1, 1, 1}, sst[5] = {1, 0, 0, 0, 0};
+  if ((rc = check_range(workspace, sd, sst, 1))) return rc;
+  // the largest chunk of the batch whose product fits the workspace
+  long long cb = E0;
+  while (cb > 1 && lin_bwd_bytes(sh, cb, nullptr, nullptr, nullptr, nullptr) > workspace_bytes) cb = (cb + 1) / 2;
+  size_t pb, mb, wb, tb;
+  if (lin_bwd_bytes(sh, cb, &pb, &mb, &wb, &tb) > workspace_bytes) return GELIB_HIP_ERR_WORKSPACE;
+  char *base = (char *)workspace;
+  float *mix_ws = (float *)(base + pb), *wg_ws = (float *)(base + pb + mb);
+  float2 *wg_tmp = (float2 *)(base + pb + mb + wb);
+  hipStream_t s = (hipStream_t)stream;
+
+  auto chunk_of = [&](const gelib_part_desc &d, long long b0, long long cbn) {
+    gelib_part_desc c = d;
+    c.ptr = (char *)d.ptr + b0 * d.strides[0] * (long long)sizeof(float2);
+    c.dims[0] = cbn;
+    return c;
+  };
+  for (long long b0 = 0; b0 < E0; b0 += cb) {
+    const long long cbn = std::min(cb, E0 - b0);
+    std::vector<gelib_part_desc> P(sh.G.size()), gc(ng), xc(nx), yc(ny), xgc, ygc;
+    for (int i = 0; i < ng; i++) gc[i] = chunk_of(g[i], b0, cbn);
+    for (int i = 0; i < nx; i++) xc[i] = chunk_of(x[i], b0, cbn);
+    for (int i = 0; i < ny; i++) yc[i] = chunk_of(y[i], b0, cbn);
+    if (xg) for (int i = 0; i < nx; i++) xgc.push_back(chunk_of(xg[i], b0, cbn));
+    if (yg) for (int i = 0; i < ny; i++) ygc.push_back(chunk_of(yg[i], b0, cbn));
+    size_t off = 0;
+    for (size_t k = 0; k < sh.G.size(); k++) {   // the chunk's product parts, packed
+      const long long rows_cell = 2 * sh.G[k].l + 1, n = sh.tau[k];
+      gelib_part_desc &d = P[k];
+      d.ptr = base + off;
+      d.dims[0] = cbn, d.dims[1] = sh.plan.E[1], d.dims[2] = sh.plan.E[2], d.dims[3] = rows_cell, d.dims[4] = n;
+      d.strides[4] = 1, d.strides[3] = n, d.strides[2] = rows_cell * n, d.strides[1] = sh.plan.E[2] * rows_cell * n;
+      d.strides[0] = sh.G01 * rows_cell * n;
+      off += (((size_t)cb * sh.G01 * rows_cell * n * sizeof(float2)) + 255) & ~(size_t)255;
+    }
+    // 1. the chunk's product
+    if ((rc = vec_fwd_entry(false, (int)P.size(), P.data(), nx, xc.data(), ny, yc.data(), 0, stream))) return rc;
+    for (size_t k = 0; k < sh.G.size(); k++) {
+      const gelib_part_desc &go = gc[sh.G[k].d - g];
+      const long long rows = cbn * sh.G01 * (2 * sh.G[k].l + 1);
+      const int tau = (int)sh.tau[k], n_out = sh.G[k].n;
+      // 2. gradient of the matrix: first chunk straight into wg (or onto it), later chunks through the temporary
+      if (wg) {
+        const bool direct = b0 == 0 && !accumulate;
+        rc = launch_mix_wgrad(direct ? WG[k] : wg_tmp, (const float2 *)P[k].ptr, (const float2 *)go.ptr, rows, tau, n_out,
+                              tau, go.strides[3], wg_ws, wb, s);
+        if (rc) return rc == 11 ? GELIB_HIP_ERR_UNSUPPORTED : rc;
+        if (!direct && (rc = launch_add_into(WG[k], wg_tmp, (long long)tau * n_out, true, s))) return rc;
+      }
+      // 3. gradient of the product, over the product itself
+      if (xg || yg) {
+        rc = launch_mix((float2 *)P[k].ptr, (const float2 *)go.ptr, W[k], rows, n_out, tau, go.strides[3], tau, true, mix_ws,
+                        mb, s);
+        if (rc) return rc == 11 ? GELIB_HIP_ERR_UNSUPPORTED : rc;
+      }
+    }
+    // 4. the product's backward pass on it
+    if (xg || yg) {
+      rc = vec_bwd_entry(false, xg ? xgc.data() : nullptr, yg ? ygc.data() : nullptr, (int)P.size(), P.data(), nx, xc.data(),
+                         ny, yc.data(), accumulate, stream);
+      if (rc) return rc;
+    }
+  }
+  return GELIB_HIP_OK;
+}
+
 }  // namespace
 }  // namespace gelib_hip
 
@@ -990,6 +1163,20 @@ int gelib_hip_so3vec_cg_linear_fwd(int nr, const gelib_part_desc *r, int nx, con
                                    const gelib_part_desc *y, const void *const *w, int accumulate, void *workspace,
                                    uint64_t workspace_bytes, void *stream) {
   return linear_fwd_entry(nr, r, nx, x, ny, y, w, accumulate, workspace, workspace_bytes, stream);
+}
+int gelib_hip_so3vec_cg_linear_bwd(const gelib_part_desc *xg, const gelib_part_desc *yg, void *const *wg, int ng,
+                                   const gelib_part_desc *g, int nx, const gelib_part_desc *x, int ny,
+                                   const gelib_part_desc *y, const void *const *w, int accumulate, void *workspace,
+                                   uint64_t workspace_bytes, void *stream) {
+  return linear_bwd_entry(xg, yg, wg, ng, g, nx, x, ny, y, w, accumulate, workspace, workspace_bytes, stream);
+}
+uint64_t gelib_hip_so3vec_cg_linear_bwd_workspace_bytes(int ng, const gelib_part_desc *g, int nx, const gelib_part_desc *x,
+                                                        int ny, const gelib_part_desc *y, int64_t batch_chunk) {
+  LinBwdShape sh;
+  if (lin_bwd_shape(ng, g, nx, x, ny, y, nullptr, nullptr, sh)) return 0;
+  const long long cb = batch_chunk > 0 ? std::min<long long>(batch_chunk, sh.plan.E[0]) : sh.plan.E[0];
+  if (cb <= 0) return 0;
+  return (uint64_t)lin_bwd_bytes(sh, cb, nullptr, nullptr, nullptr, nullptr);
 }
 uint64_t gelib_hip_so3vec_cg_linear_workspace_bytes(int nr, const gelib_part_desc *r, int nx, const gelib_part_desc *x,
                                                     int ny, const gelib_part_desc *y) {

@@ -56,7 +56,7 @@ enum gelib_hip_status {
   GELIB_HIP_ERR_ARG = 12,          /* negative offset, negative stride or other malformed argument                   */
   GELIB_HIP_ERR_WORKSPACE = 13,    /* workspace missing, not 16-byte aligned or smaller than the size query says     */
   GELIB_HIP_ERR_TOO_LARGE = 14,    /* sizes beyond the stated maximum of gelib_hip_part_mix_channels_static          */
-  GELIB_HIP_ERR_UNSUPPORTED = 15   /* gelib_hip_so3vec_cg_linear_fwd: shapes outside what the fused kernel takes     */
+  GELIB_HIP_ERR_UNSUPPORTED = 15   /* gelib_hip_so3vec_cg_linear_fwd / _bwd: shapes outside what the call takes      */
 };
 
 #define GELIB_HIP_MAX_L 32          /* largest l of an operand part                     */
@@ -207,6 +207,34 @@ int gelib_hip_so3vec_cg_linear_fwd(int nr, const gelib_part_desc *r, int nx, con
  * descriptors are malformed or r does not have exactly the parts l = 0..4. */
 uint64_t gelib_hip_so3vec_cg_linear_workspace_bytes(int nr, const gelib_part_desc *r, int nx, const gelib_part_desc *x,
                                                     int ny, const gelib_part_desc *y);
+
+/*
+ * Backward pass of the call above in bounded memory: with out_l = P_l w_l, P = CGproduct(x, y), and g_l the gradient of
+ * out_l (ng parts, n_out_l channels each):
+ *     xg, yg (+)= the gradients of x and y          (Gvec::add_CGproduct_back0 / _back1, core/Gvec.hpp:323-345, applied
+ *                                                    to gP_l = g_l w_l^H, which torch's autograd forms in the reference),
+ *     wg[k]  (+)= sum over the rows of P_l^H g_l     (the gradient of the matmul of python/src/gelib/SO3vec.py:174-177
+ *                                                    with respect to the matrix; w[k] and wg[k] belong to g[k]).
+ * Any of xg, yg, wg may be NULL.  Neither P nor gP is ever held at full size (25 GB each at the headline type): the
+ * batch is taken in chunks whose product fits the workspace -- the forward kernels form a chunk's product there, the
+ * matrix-gradient kernel reads it, gP overwrites it in place and the backward kernels read that -- so the call moves the
+ * same bytes as the four separate calls and runs at their speed, in the memory of one chunk.  (One kernel that keeps the
+ * product on chip throughout would be no faster on this GPU: it needs two matrix products of 12.3 MFLOP per cell and
+ * three product-sized contractions on the vector unit, and for float32 the two units do not run at the same time.)
+ * workspace: 256-byte aligned device memory; gelib_hip_so3vec_cg_linear_bwd_workspace_bytes(..., batch_chunk) tells the
+ * bytes that let the call take batch_chunk batch entries at a time (<= 0: the whole batch at once); with less, the call
+ * takes smaller chunks, and GELIB_HIP_ERR_WORKSPACE when not even one batch entry fits.  Conditions
+ * (GELIB_HIP_ERR_UNSUPPORTED otherwise, nothing launched): every tensor has the full batch and grid extents, the parts of
+ * g are packed along (batch, grid, m) with 16-byte aligned rows, and the channel counts of the product's parts and of
+ * g's parts are even.  Operand shapes are not restricted to those of the fused forward kernel.  The sums of wg over the
+ * chunks are added in the order of the chunks: results do not depend on timing.
+ */
+int gelib_hip_so3vec_cg_linear_bwd(const gelib_part_desc *xg, const gelib_part_desc *yg, void *const *wg, int ng,
+                                   const gelib_part_desc *g, int nx, const gelib_part_desc *x, int ny,
+                                   const gelib_part_desc *y, const void *const *w, int accumulate, void *workspace,
+                                   uint64_t workspace_bytes, void *stream);
+uint64_t gelib_hip_so3vec_cg_linear_bwd_workspace_bytes(int ng, const gelib_part_desc *g, int nx, const gelib_part_desc *x,
+                                                        int ny, const gelib_part_desc *y, int64_t batch_chunk);
 
 /* ---- gather: sums of slices along the batch or a grid dimension ---------------------------------------------------------
  * A gather map is a list of (source, target) pairs with 0 <= source < n_in, 0 <= target < n_out (the arguments of

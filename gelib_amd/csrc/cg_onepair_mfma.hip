@@ -482,11 +482,20 @@ int device_tables(int l1, int l2, int lmin, int lt, int nl, const std::vector<in
             cfwd.push_back(c);
           }
     }
+    // both tables in one allocation (the forward one behind the backward one, 256-byte aligned), freed again when a
+    // copy fails
     Tables t{nullptr, step, nullptr, fstep};
-    GELIB_HIP_TRY(hipMalloc((void **)&t.coef, coef.size() * sizeof(float)));
-    GELIB_HIP_TRY(hipMemcpy(t.coef, coef.data(), coef.size() * sizeof(float), hipMemcpyHostToDevice));
-    GELIB_HIP_TRY(hipMalloc((void **)&t.coef_fwd, cfwd.size() * sizeof(float)));
-    GELIB_HIP_TRY(hipMemcpy(t.coef_fwd, cfwd.data(), cfwd.size() * sizeof(float), hipMemcpyHostToDevice));
+    const size_t bwd_bytes = (coef.size() * sizeof(float) + 255) & ~(size_t)255;
+    char *d = nullptr;
+    GELIB_HIP_TRY(hipMalloc((void **)&d, bwd_bytes + cfwd.size() * sizeof(float)));
+    hipError_t e = hipMemcpy(d, coef.data(), coef.size() * sizeof(float), hipMemcpyHostToDevice);
+    if (e == hipSuccess) e = hipMemcpy(d + bwd_bytes, cfwd.data(), cfwd.size() * sizeof(float), hipMemcpyHostToDevice);
+    if (e != hipSuccess) {
+      (void)hipFree(d);
+      return record_hip_error(e, "hipMemcpy(single-pair coefficient tables)");
+    }
+    t.coef = (float *)d;
+    t.coef_fwd = (float *)(d + bwd_bytes);
     it = g_tables.emplace(key, t).first;
   }
   *out = it->second;

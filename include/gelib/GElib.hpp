@@ -207,25 +207,23 @@ class SO3type : public GtypeBase {
   void set(const int ix, const int n) { parts[ix] = n; }
   bool operator==(const SO3type &y) const { return parts == y.parts; }
 
-  SO3type CGproduct(const SO3type &y, const int limit = null_ix) const {
+  // Type of the product: channels of part l = sum over the pairs (l1, l2) with |l1 - l2| <= l <= l1 + l2 of n1 n2
+  // (Diag: n1); a limit >= 0 keeps the parts up to it (core/Gtype.hpp:115-138).
+  SO3type CGproduct(const SO3type &y, const int limit = null_ix) const { return product_type(y, limit, false); }
+  SO3type DiagCGproduct(const SO3type &y, const int limit = null_ix) const { return product_type(y, limit, true); }
+
+ private:
+  SO3type product_type(const SO3type &y, const int limit, const bool diag) const {
     SO3type R;
-    for (auto &p : parts)
-      for (auto &q : y.parts)
-        SO3group::for_each_CGcomponent(p.first, q.first, [&](const int z, const int m) {
-          if (limit == null_ix || z <= limit) R.parts[z] += m * p.second * q.second;
-        });
-    return R;
-  }
-  SO3type DiagCGproduct(const SO3type &y, const int limit = null_ix) const {
-    SO3type R;
-    for (auto &p : parts)
-      for (auto &q : y.parts)
-        SO3group::for_each_CGcomponent(p.first, q.first, [&](const int z, const int m) {
-          if (limit == null_ix || z <= limit) R.parts[z] += m * p.second;
-        });
+    for (const auto &[l1, n1] : parts)
+      for (const auto &[l2, n2] : y.parts) {
+        const int top = limit == null_ix ? l1 + l2 : std::min(l1 + l2, limit);
+        for (int l = std::abs(l1 - l2); l <= top; l++) R.parts[l] += diag ? n1 : n1 * n2;
+      }
     return R;
   }
 
+ public:
   std::string str(const std::string indent = "") const {
     std::ostringstream oss;
     oss << indent << "(";

@@ -39,6 +39,8 @@ SHAPES = [
     (9, 0, 3, 3, 16, 4),
     (2, 6, 6, 6, 2, 4),          # operands above l = 4, product l up to 6
     (2, 5, 6, 1, 8, 2),
+    (2, 6, 6, 12, 2, 2),         # operands of l = 6 into l = 12: beyond the l range of the unrolled kernels' pair records
+    (3, 6, 5, 9, 4, 2),
     (5, 2, 3, 4, 32, 32),        # configuration 2's triple: the single-triple backward kernel, 32 channels of y
     (3, 3, 2, 1, 16, 64),        # ... 64
     (3, 4, 4, 8, 64, 16),        # ... 16

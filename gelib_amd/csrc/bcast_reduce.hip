@@ -24,13 +24,31 @@ struct ReduceArgs {
   int accumulate;
 };
 
-__device__ __forceinline__ long long tmp_cell(const ReduceArgs &a, int dc, int r) {
-  // destination cell -> coordinates; r -> coordinates along the summed dimensions (dimension 0 slowest)
+// Coordinates of the summed cells of one destination cell: the dimensions along which the destination broadcasts run
+// from 0 to E[k] - 1 (dimension 0 slowest), the others stay at the destination cell's own coordinate.
+struct SummedCell {
+  int c[3];   // coordinates in the temporary
+  int R[3];   // extent of the summed range per dimension (1 where the destination has the dimension itself)
+};
+
+__device__ __forceinline__ SummedCell summed_cell(const ReduceArgs &a, int dc, int r) {
+  SummedCell q;
   const int d2 = dc % a.D[2], d1 = (dc / a.D[2]) % a.D[1], d0 = dc / (a.D[2] * a.D[1]);
-  const int R2 = a.D[2] == 1 ? a.E[2] : 1, R1 = a.D[1] == 1 ? a.E[1] : 1;
-  const int r2 = r % R2, r1 = (r / R2) % R1, r0 = r / (R2 * R1);
-  const int c0 = a.D[0] == 1 ? r0 : d0, c1 = a.D[1] == 1 ? r1 : d1, c2 = a.D[2] == 1 ? r2 : d2;
-  return ((long long)c0 * a.E[1] + c1) * a.E[2] + c2;
+  q.R[0] = a.D[0] == 1 ? a.E[0] : 1, q.R[1] = a.D[1] == 1 ? a.E[1] : 1, q.R[2] = a.D[2] == 1 ? a.E[2] : 1;
+  const int r2 = r % q.R[2], r1 = (r / q.R[2]) % q.R[1], r0 = r / (q.R[2] * q.R[1]);
+  q.c[0] = a.D[0] == 1 ? r0 : d0, q.c[1] = a.D[1] == 1 ? r1 : d1, q.c[2] = a.D[2] == 1 ? r2 : d2;
+  return q;
+}
+__device__ __forceinline__ long long cell_index(const ReduceArgs &a, const SummedCell &q) {
+  return ((long long)q.c[0] * a.E[1] + q.c[1]) * a.E[2] + q.c[2];
+}
+// the next summed cell: the last summed dimension runs fastest
+__device__ __forceinline__ void next_cell(const ReduceArgs &a, SummedCell &q) {
+  if (q.R[2] > 1 && ++q.c[2] < a.E[2]) return;
+  if (q.R[2] > 1) q.c[2] = 0;
+  if (q.R[1] > 1 && ++q.c[1] < a.E[1]) return;
+  if (q.R[1] > 1) q.c[1] = 0;
+  if (q.R[0] > 1) ++q.c[0];
 }
 
 __device__ __forceinline__ float2 *dest_elem(const ReduceArgs &a, int dc, int e) {
@@ -46,11 +64,22 @@ __global__ void __launch_bounds__(256) bcast_stage1_kernel(ReduceArgs a, long lo
     const long long q = w / a.elems;
     const int p = (int)(q % a.P), dc = (int)(q / a.P);
     const int r0 = p * a.len, r1 = min(a.Rn, r0 + a.len);
+    // eight loads in flight at a time (a thread's loads would otherwise wait for each other); the order of the additions
+    // stays the order of the cells
     float2 acc = make_float2(0.f, 0.f);
-    for (int r = r0; r < r1; r++) {
-      const float2 v = a.tmp[tmp_cell(a, dc, r) * a.elems + e];
-      acc.x += v.x;
-      acc.y += v.y;
+    SummedCell sc = summed_cell(a, dc, r0);
+    for (int r = r0; r < r1; r += 8) {
+      float2 v[8];
+#pragma unroll
+      for (int u = 0; u < 8; u++) {
+        v[u] = r + u < r1 ? a.tmp[cell_index(a, sc) * a.elems + e] : make_float2(0.f, 0.f);
+        if (r + u < r1) next_cell(a, sc);
+      }
+#pragma unroll
+      for (int u = 0; u < 8; u++) {
+        acc.x += v[u].x;
+        acc.y += v[u].y;
+      }
     }
     if (a.P > 1) {
       a.part[w] = acc;
@@ -71,10 +100,15 @@ __global__ void __launch_bounds__(256) bcast_stage2_kernel(ReduceArgs a, long lo
     const int e = (int)(w % a.elems), dc = (int)(w / a.elems);
     float2 acc = make_float2(0.f, 0.f);
     const float2 *pp = a.part + (long long)dc * a.P * a.elems + e;
-    for (int p = 0; p < a.P; p++) {
-      const float2 v = pp[(long long)p * a.elems];
-      acc.x += v.x;
-      acc.y += v.y;
+    for (int p = 0; p < a.P; p += 8) {
+      float2 v[8];
+#pragma unroll
+      for (int u = 0; u < 8; u++) v[u] = p + u < a.P ? pp[(long long)(p + u) * a.elems] : make_float2(0.f, 0.f);
+#pragma unroll
+      for (int u = 0; u < 8; u++) {
+        acc.x += v[u].x;
+        acc.y += v[u].y;
+      }
     }
     float2 *dst = dest_elem(a, dc, e);
     if (a.accumulate) {
@@ -86,12 +120,15 @@ __global__ void __launch_bounds__(256) bcast_stage2_kernel(ReduceArgs a, long lo
   }
 }
 
-// ranges per destination cell: enough threads to fill the GPU, at least 16 cells per range
+// ranges per destination cell: enough threads to fill the GPU, at least 64 cells per range, and about as many ranges as
+// cells per range (a thread of the second stage adds the ranges one after the other, as one of the first adds cells)
 int choose_ranges(long long dcells, int elems, int Rn) {
-  const long long want_threads = 1 << 19;
+  const long long want_threads = 1 << 18;
   long long P = want_threads / std::max<long long>(1, dcells * elems);
-  P = std::min<long long>(P, Rn / 16);
-  P = std::min<long long>(P, 4096);
+  P = std::min<long long>(P, Rn / 64);
+  long long balanced = 1;
+  while (balanced * balanced < Rn) balanced *= 2;
+  P = std::min<long long>(P, balanced);
   return (int)std::max<long long>(1, P);
 }
 

@@ -159,7 +159,8 @@ def cpu_slice(torch, xs, ys, gs, rs, xgs, ygs, maxl, diag, nsample, single_core,
     def merge(gpu_parts, c32, c64, S):
         tot = {"components": 0, "outside_gate": 0.0, "cpu_f32_outside_gate_of_f64": 0.0, "by_rule_B": 0.0,
                "by_rule_C": 0.0, "rejected": 0, "max_err_over_rule_C_bound": 0.0, "max_gate_excess": 0.0,
-               "max_err_vs_f64": {"gpu": 0.0, "cpu_f32": 0.0}}
+               "outside_gate_complex": 0.0, "max_err_vs_f64": {"gpu": 0.0, "cpu_f32": 0.0}}
+        elements = 0
         for t, b, c, s in zip(gpu_parts, c32, c64, S):
             a = t[:nsample].cpu().numpy()
             rep = U.parity_counts(a, b, c, s)
@@ -168,12 +169,16 @@ def cpu_slice(torch, xs, ys, gs, rs, xgs, ygs, maxl, diag, nsample, single_core,
                 tot[k] += rep[k] * n
             tot["components"] += n
             tot["rejected"] += rep["rejected"]
+            # the gate read per complex element: |gpu - cpu| <= 1e-6 + 1e-5 |cpu| on the moduli
+            tot["outside_gate_complex"] += float((np.abs(a - b) > U.ATOL + U.RTOL * np.abs(b)).sum())
+            elements += a.size
             tot["max_err_over_rule_C_bound"] = max(tot["max_err_over_rule_C_bound"], rep["max_err_over_rule_C_bound"])
             tot["max_gate_excess"] = max(tot["max_gate_excess"], U.gate_excess(a, b))
             tot["max_err_vs_f64"]["gpu"] = max(tot["max_err_vs_f64"]["gpu"], U.max_abs_err(a, c))
             tot["max_err_vs_f64"]["cpu_f32"] = max(tot["max_err_vs_f64"]["cpu_f32"], U.max_abs_err(b, c))
         for k in ("outside_gate", "cpu_f32_outside_gate_of_f64", "by_rule_B", "by_rule_C"):
             tot[k] /= max(1, tot["components"])
+        tot["outside_gate_complex"] /= max(1, elements)
         return tot
 
     fwd = merge(rs, r, r64, Sr)
@@ -181,7 +186,8 @@ def cpu_slice(torch, xs, ys, gs, rs, xgs, ygs, maxl, diag, nsample, single_core,
     parity = {"ok": fwd["rejected"] == 0 and bwd["rejected"] == 0, "samples": nsample, "fwd": fwd, "bwd": bwd,
               "rules": "per real component: A |gpu-cpu| <= 1e-6 + 1e-5|cpu|; else B (cpu_f32 itself outside that gate "
                        "of float64 and |gpu-f64| <= |cpu-f64|); else C |gpu-f64| <= 1e-6 + 2*eps32*sum|terms|; "
-                       "outside_gate = fraction not passing A, rejected = components passing none"}
+                       "outside_gate = fraction not passing A, rejected = components passing none; "
+                       "outside_gate_complex = fraction of complex elements with |gpu-cpu| > 1e-6 + 1e-5|cpu| (moduli)"}
     return {"single_core_s": dt1, "all_cores_s": dt_all, "cores": nth, "parity": parity}
 
 

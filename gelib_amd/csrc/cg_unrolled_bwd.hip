@@ -15,6 +15,7 @@ int launch_unrolled_bwd_diag8_pad(const BwdArgs &a, int nblocks, size_t lds_byte
 int launch_unrolled_bwd_cg6_l6(const BwdArgs &a, int nblocks, size_t lds_bytes, hipStream_t s);
 int launch_unrolled_bwd_cg6_l6_pad(const BwdArgs &a, int nblocks, size_t lds_bytes, hipStream_t s);
 int launch_unrolled_bwd_cg6_hi(const BwdArgs &a, int nblocks, size_t lds_bytes, hipStream_t s);
+int launch_unrolled_bwd_cg6_hi_pad(const BwdArgs &a, int nblocks, size_t lds_bytes, hipStream_t s);
 int launch_unrolled_bwd_one(const BwdArgs &a, int nblocks, size_t lds_bytes, hipStream_t s);
 int launch_one_triple_bwd_k1_small(const BwdArgs &a, int nblocks, size_t lds_bytes, hipStream_t s);
 int launch_one_triple_bwd_k1_large(const BwdArgs &a, int nblocks, size_t lds_bytes, hipStream_t s);
@@ -43,11 +44,12 @@ size_t unrolled_bwd_lds_bytes(int bank_len, int xsize, int ysize, int cells_per_
 // Operands up to l = 4: every product (l up to 8), Diag or not, any channel counts.  Operands up to l = 6: CGproduct
 // capped at l = 6 (two instantiations, power-of-two channel counts and others, five minutes of compile time each; a
 // kernel for the uncapped product, l up to 12, is not built).
-// ... and the part above l = 6 of such a product on its own: llo = the smallest l present (power-of-two channels).
+// ... and the part above l = 6 of such a product on its own: llo = the smallest l present.
 bool unrolled_bwd_takes(bool diag, bool padded, int lcap, int lop, int llo) {
   if (lop <= kLT) return lcap <= 2 * kLT;
   if (lop > kLTMax || diag) return false;
-  return lcap <= kLTMax || (llo > kLTMax && lcap <= 2 * kLTMax && !padded);
+  (void)padded;
+  return lcap <= kLTMax || (llo > kLTMax && lcap <= 2 * kLTMax);
 }
 
 int unrolled_bwd_cap(int lcap, int lop, int llo) {
@@ -63,7 +65,8 @@ int unrolled_bwd_lo(int lcap, int lop, int llo) { return (lop > kLT && lcap > kL
 int launch_unrolled_bwd(const BwdArgs &a, bool diag, int lcap, int lop, int nblocks, size_t lds_bytes, hipStream_t s) {
   if (nblocks <= 0) return GELIB_HIP_OK;
   if (lop > kLT) {
-    if (lcap > kLTMax) return launch_unrolled_bwd_cg6_hi(a, nblocks, lds_bytes, s);
+    if (lcap > kLTMax)
+      return a.padded ? launch_unrolled_bwd_cg6_hi_pad(a, nblocks, lds_bytes, s) : launch_unrolled_bwd_cg6_hi(a, nblocks, lds_bytes, s);
     return a.padded ? launch_unrolled_bwd_cg6_l6_pad(a, nblocks, lds_bytes, s)
                     : launch_unrolled_bwd_cg6_l6(a, nblocks, lds_bytes, s);
   }

@@ -579,7 +579,8 @@ int unrolled_vec_bwd(const VecPlan &plan, const std::vector<const gelib_part_des
       lcap = std::max(lcap, t.l), llo = std::min(llo, t.l), lop = std::max(lop, std::max(t.l1, t.l2));
       padded = padded || !is_pow2(xs[t.xi].second) || !is_pow2(ys[t.yi].second);
     }
-    if (!plan.diag && !padded && g_bwd_l6_enable && g_bwd_l6_split && lop > kLT && lop <= kLTMax && llo <= kLTMax &&
+    (void)padded;
+    if (!plan.diag && g_bwd_l6_enable && g_bwd_l6_split && lop > kLT && lop <= kLTMax && llo <= kLTMax &&
         lcap > kLTMax && lcap <= 2 * kLTMax) {
       std::vector<VecTriple> ta, tb;
       std::vector<int> rla, rlb, map_a(rls.size(), -1), map_b(rls.size(), -1);

@@ -129,6 +129,8 @@ def test_pair_split_is_reproducible_and_respects_accumulate(cabi):
     (4, {2: 4, 5: 8, 6: 2}, {3: 4, 6: 4}, 9),                          # parts missing, capped between 6 and 12
     (2, {6: 16}, {6: 4}, -1),                                          # one pair, l = 0..12
     (5, {0: 2, 5: 2}, {1: 4, 6: 1}, 11),
+    (3, {l: 6 for l in range(7)}, {l: 6 for l in range(7)}, -1),       # channel counts that are not powers of two
+    (4, {2: 6, 5: 2}, {1: 12, 6: 5}, 9),
 ])
 def test_operands_above_l4_product_above_l6(cabi, case):
     """CGproduct of operands up to l = 6 that reaches above l = 6: the triples up to l = 6 on the unrolled kernels built

@@ -21,7 +21,7 @@ SYMBOLS = [
     "gelib_hip_part_mix_channels_static", "gelib_hip_part_mix_channels_wgrad", "gelib_hip_part_mix_workspace_bytes",
     "gelib_hip_so3vec_cg_linear_fwd", "gelib_hip_so3vec_cg_linear_workspace_bytes",
     "gelib_hip_so3vec_cg_linear_bwd", "gelib_hip_so3vec_cg_linear_bwd_workspace_bytes",
-    "gelib_hip_set_option",
+    "gelib_hip_set_option", "gelib_hip_set_stream_workspace",
     "gelib_hip_last_path",
     "gelib_hip_malloc", "gelib_hip_free", "gelib_hip_memcpy", "gelib_hip_memset", "gelib_hip_synchronize",
 ]
@@ -97,6 +97,7 @@ def lib():
         L.gelib_hip_part_mix_workspace_bytes.restype = ctypes.c_uint64
         L.gelib_hip_part_mix_workspace_bytes.argtypes = [ctypes.c_int, ctypes.c_int64, ctypes.c_int, ctypes.c_int]
         L.gelib_hip_set_option.argtypes = [ctypes.c_char_p, ctypes.c_int]
+        L.gelib_hip_set_stream_workspace.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_uint64]
         _lib = L
     return _lib
 
@@ -250,6 +251,20 @@ def so3vec_cg_linear_bwd(xgparts, ygparts, wgparts, gparts, xparts, yparts, wpar
         return False
     check(rc)
     return True
+
+
+def set_stream_workspace(buf, stream=None):
+    """Lends the library the uint8 tensor buf (None: takes the loan back) as its scratch on `stream` (torch's current
+    stream of buf's device by default).  The caller keeps buf alive while calls or graphs may use it."""
+    import torch
+    if stream is None:
+        stream = torch.cuda.current_stream(buf.device if buf is not None else None)
+    sp = ctypes.c_void_p(stream.cuda_stream)
+    if buf is None:
+        check(lib().gelib_hip_set_stream_workspace(sp, None, 0))
+        return
+    base = (buf.data_ptr() + 255) & ~255
+    check(lib().gelib_hip_set_stream_workspace(sp, ctypes.c_void_p(base), buf.numel() - (base - buf.data_ptr())))
 
 
 def so3part_spharm(r, x, accumulate=True):

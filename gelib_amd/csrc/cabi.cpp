@@ -45,19 +45,34 @@ struct ScratchBuf {
 constexpr int kScratchKinds = 2;
 std::mutex g_scratch_mutex[kScratchKinds];
 std::map<std::pair<int, hipStream_t>, ScratchBuf> g_scratch[kScratchKinds];
+// memory the caller has lent for a stream (gelib_hip_set_stream_workspace): kind k uses the k-th of kScratchKinds equal
+// slices.  It is the caller's to keep alive, so it also serves calls that are being recorded into a graph.
+std::mutex g_lent_mutex;
+std::map<std::pair<int, hipStream_t>, ScratchBuf> g_lent;
 }  // namespace
 
 std::mutex &stream_scratch_mutex(int kind) { return g_scratch_mutex[kind]; }
 
 int stream_scratch(int kind, hipStream_t s, size_t bytes, void **out) {
-  // A call that is being recorded into a graph gets none (*out = nullptr) and takes its scratch-free route: the graph
-  // would keep the buffer's address, and a later call that needs a larger buffer frees it.
   *out = nullptr;
+  int dev = 0;
+  GELIB_HIP_TRY(hipGetDevice(&dev));
+  {
+    std::lock_guard<std::mutex> lock(g_lent_mutex);
+    auto it = g_lent.find({dev, s});
+    if (it != g_lent.end()) {
+      const size_t slice = (it->second.bytes / kScratchKinds) & ~(size_t)255;
+      if (bytes <= slice) {
+        *out = it->second.ptr + (size_t)kind * slice;
+        return GELIB_HIP_OK;
+      }
+    }
+  }
+  // A call that is being recorded into a graph gets none of the library's own (*out = nullptr) and takes its
+  // scratch-free route: the graph would keep the buffer's address, and a later call that needs a larger buffer frees it.
   hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
   if (hipStreamIsCapturing(s, &cap) != hipSuccess) (void)hipGetLastError();
   if (cap != hipStreamCaptureStatusNone) return GELIB_HIP_OK;
-  int dev = 0;
-  GELIB_HIP_TRY(hipGetDevice(&dev));
   ScratchBuf &buf = g_scratch[kind][{dev, s}];
   if (buf.bytes < bytes) {
     if (buf.ptr) {
@@ -1394,6 +1409,30 @@ uint64_t gelib_hip_part_mix_workspace_bytes(int kind, int64_t rows, int n_in, in
   if (kind == 0) return mix_workspace_bytes(n_in, n_out);
   if (kind == 1) return mix_wgrad_workspace_bytes(rows, n_in, n_out);
   return 0;
+}
+
+int gelib_hip_set_stream_workspace(void *stream, void *ptr, uint64_t bytes) {
+  int dev = 0;
+  GELIB_HIP_TRY(hipGetDevice(&dev));
+  if (ptr && bytes) {
+    if ((uintptr_t)ptr & 255) return GELIB_HIP_ERR_WORKSPACE;
+    const int64_t sd[5] = {(int64_t)bytes, 1, 1, 1, 1}, sst[5] = {1, 0, 0, 0, 0};
+    int rc = check_range(ptr, sd, sst, 1);
+    if (rc) return rc;
+  }
+  // both scratch users finish putting their kernels on the stream before the buffer changes under them
+  std::lock_guard<std::mutex> l0(stream_scratch_mutex(0));
+  std::lock_guard<std::mutex> l1(stream_scratch_mutex(1));
+  std::lock_guard<std::mutex> lock(g_lent_mutex);
+  if (ptr && bytes) {
+    ScratchBuf b;
+    b.ptr = (char *)ptr;
+    b.bytes = (size_t)bytes;
+    g_lent[{dev, (hipStream_t)stream}] = b;
+  } else {
+    g_lent.erase({dev, (hipStream_t)stream});
+  }
+  return GELIB_HIP_OK;
 }
 
 int gelib_hip_malloc(void **ptr, uint64_t bytes) {

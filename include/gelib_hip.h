@@ -270,6 +270,19 @@ int gelib_hip_memset(void *ptr, int value, uint64_t bytes);
 int gelib_hip_synchronize(void);
 
 /*
+ * Lends the library `bytes` of device memory (256-byte aligned) for its scratch on `stream` of the current device, in
+ * place of the buffers it would allocate itself: the per-cell gradients of a destination that broadcasts (first half) and
+ * the partial sums of backward launches with few cells (second half).  No counterpart in the reference; it is for callers
+ * that record calls into a HIP graph (a recorded call takes no scratch of the library's own, see the top of this file,
+ * and falls back to slower routes: with lent memory it runs exactly as an eager call does) and for callers that want
+ * every allocation in their own hands.  The memory stays the caller's and must outlive every call and every graph that
+ * uses it; a call whose need exceeds its half takes the library's own scratch (eager) or the scratch-free route
+ * (recorded).  ptr = NULL or bytes = 0 takes the loan back.  Needs per call: 64 MiB at most for the first half
+ * ("bcast_scratch_kb"), 16 x cells x (size of x + size of y per cell) bytes at most for the second (fewer than 1024 cells).
+ */
+int gelib_hip_set_stream_workspace(void *stream, void *ptr, uint64_t bytes);
+
+/*
  * Tuning / introspection (no counterpart in the reference).
  * gelib_hip_set_option("force_generic", 1) routes every call through the shape-agnostic kernels;
  * "check_pointers" (default 1) switches the device-pointer validation of every call off (0) or on: with 1 an

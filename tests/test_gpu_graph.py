@@ -83,3 +83,67 @@ def test_replays_match_eager_calls(cabi):
     torch.cuda.synchronize()
     for a, b in zip(xg + yg, got[5:15]):
         assert torch.allclose(a.view(torch.float32), b, rtol=1e-4, atol=1e-3)
+
+
+def test_recorded_calls_use_lent_scratch(cabi):
+    """With memory lent for the stream (gelib_hip_set_stream_workspace), a recorded call takes the routes an eager call
+    takes -- the pairs of a cell dealt to several blocks in a launch with few cells, per-cell gradients and a fixed-order
+    sum for an operand shared by the batch -- and replays give the eager bits."""
+    B, n = 48, 16
+    cabi.set_option("unrolled_bwd_split", 1)
+    xs = [U.dev(U.seeded(10 + l, B, 2 * l + 1, n)) for l in range(5)]
+    x1 = [U.dev(U.seeded(40 + l, 1, 2 * l + 1, n)) for l in range(5)]
+    ys = [U.dev(U.seeded(20 + l, B, 2 * l + 1, n)) for l in range(5)]
+    taus = cabi.so3type_product({l: n for l in range(5)}, {l: n for l in range(5)}, 4)
+    gs = [U.dev(U.seeded(30 + l, B, 2 * l + 1, taus[l])) for l in range(5)]
+    xg, yg = [torch.empty_like(t) for t in xs], [torch.empty_like(t) for t in ys]
+    xg1, yg1 = [torch.empty_like(t) for t in x1], [torch.empty_like(t) for t in ys]
+    stream = torch.cuda.Stream()
+    lent = torch.empty(64 << 20, dtype=torch.uint8, device="cuda")
+    cabi.set_stream_workspace(lent, stream)
+    paths = []
+
+    def work():
+        cabi.so3vec_bwd(xg, yg, gs, xs, ys, accumulate=False)
+        paths.append(cabi.last_path())
+        cabi.so3vec_bwd(xg1, yg1, gs, x1, ys, accumulate=False)      # x shared by the batch
+        paths.append(cabi.last_path())
+
+    try:
+        with torch.cuda.stream(stream):
+            work()
+        torch.cuda.synchronize()
+        want = bits(xg + yg + xg1 + yg1)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            work()
+        torch.cuda.synchronize()
+        assert paths == [2, 2, 2, 2]          # the unrolled kernels, also for the shared operand, also while recording
+        for k in range(2):
+            for t in xg + yg + xg1 + yg1:
+                t.fill_(7.0)
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            assert all(torch.equal(a, b) for a, b in zip(bits(xg + yg + xg1 + yg1), want)), "replay %d" % k
+        # without the loan a recorded call takes the scratch-free routes and still agrees to rounding (an eager call on
+        # that route first: it uploads the per-triple tables of the shape-agnostic kernels, which a recorded call cannot)
+        cabi.set_stream_workspace(None, stream)
+        cabi.set_option("bcast_reduce", 0)
+        with torch.cuda.stream(stream):
+            cabi.so3vec_bwd(xg1, yg1, gs, x1, ys, accumulate=False)
+        torch.cuda.synchronize()
+        cabi.set_option("bcast_reduce", 1)
+        paths.clear()
+        graph2 = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph2, stream=stream):
+            work()
+        torch.cuda.synchronize()
+        assert paths == [2, 1]
+        graph2.replay()
+        torch.cuda.synchronize()
+        for a, b in zip(bits(xg + yg + xg1 + yg1), want):
+            assert torch.allclose(a, b, rtol=1e-4, atol=1e-3)
+    finally:
+        cabi.set_option("bcast_reduce", 1)
+        cabi.set_stream_workspace(None, stream)

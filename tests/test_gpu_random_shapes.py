@@ -58,8 +58,7 @@ def test_random_product(cabi, seed):
     B, bx, tx, ty, maxl, diag = draw(rng)
     xs = [U.seeded(seed * 10 + l, bx, 2 * l + 1, n) for l, n in sorted(tx.items())]
     ys = [U.seeded(seed * 10 + 50 + l, B, 2 * l + 1, n) for l, n in sorted(ty.items())]
-    bxs = [np.broadcast_to(a, (B,) + a.shape[1:]) for a in xs]
-    O = U.VecOracle(bxs, ys, maxl, diag, gseed=seed + 100)
+    O = U.VecOracle(xs, ys, maxl, diag, gseed=seed + 100)    # an x of batch 1 is shared by the batch, in the oracle too
     r32, gs = O.r32, O.gs
     tag = "seed %d: B %d bx %d %s x %s maxl %d diag %d" % (seed, B, bx, tx, ty, maxl, diag)
     dxs, dys = [U.dev(a) for a in xs], [U.dev(a) for a in ys]
@@ -73,10 +72,10 @@ def test_random_product(cabi, seed):
         O.check_fwd_onto([U.host(a) for a in drs], start, what)
     else:
         O.check_fwd([U.host(a) for a in drs], what)
-    # both gradients; a broadcast x gets none (its gradient is a sum over the batch, a different call)
+    # both gradients; that of an x shared by the batch is the sum over the batch (formed inside the library)
     dgs = [U.dev(a) for a in gs]
     dyg = [torch.full(a.shape, 2.0 + 1j, dtype=torch.complex64, device="cuda") for a in ys]
-    dxg = None if bx != B else [torch.full(a.shape, 2.0 + 1j, dtype=torch.complex64, device="cuda") for a in xs]
+    dxg = [torch.full(a.shape, 2.0 + 1j, dtype=torch.complex64, device="cuda") for a in xs]
     cabi.so3vec_bwd(dxg, dyg, dgs, dxs, dys, accumulate=False, diag=diag)
     torch.cuda.synchronize()
     path = cabi.last_path()

@@ -21,8 +21,6 @@ using namespace gelib_hip;
 
 namespace gelib_hip {
 
-int launch_add_into(float2 *dst, const float2 *src, long long n, bool accumulate, hipStream_t s);  // bcast_reduce.hip
-
 namespace {
 thread_local std::string t_last_error;
 thread_local int t_last_path = kPathNone;

@@ -57,7 +57,9 @@ int launch_zero_fill(const PartDev &d, const long long D[3], int M, int n, hipSt
 // use, grown when more is asked for, kept until the process ends.  The caller holds stream_scratch_mutex(kind) from
 // the call until the last kernel that uses the buffer is on the stream (kernels of one stream run in order, so the
 // next user of the buffer comes after them).  kind 0: per-cell gradients of a broadcast destination; 1: partial sums of
-// backward launches that deal the pairs of a cell to several blocks.
+// backward launches that deal the pairs of a cell to several blocks.  Memory that the caller has lent for the stream
+// (gelib_hip_set_stream_workspace) is used first, half of it per kind.  *out = nullptr (status OK) when the stream is
+// being recorded into a graph and nothing is lent: the caller then takes its scratch-free route.
 int stream_scratch(int kind, hipStream_t s, size_t bytes, void **out);
 std::mutex &stream_scratch_mutex(int kind);
 
@@ -66,6 +68,7 @@ std::mutex &stream_scratch_mutex(int kind);
 size_t bcast_partial_bytes(const long long E[3], const long long D[3], int rows, int n);
 int launch_bcast_reduce(const float2 *tmp, float2 *partial, const PartDev &d, const long long E[3], const long long D[3],
                         int rows, int n, bool accumulate, hipStream_t s);
+int launch_add_into(float2 *dst, const float2 *src, long long n, bool accumulate, hipStream_t s);   // dst[i] (+)= src[i]
 
 // ---- spherical harmonics (spharm.hip): xs = strides of x in floats over (batch, grid0, grid1, xyz, channel) ----
 int launch_spharm(const PartDev &r, const float *x, const long long xs[5], const long long D[3], int L, int n,

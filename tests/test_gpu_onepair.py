@@ -21,7 +21,11 @@ def cabi():
     c.lib()
     c.set_option("force_generic", 0)
     c.set_option("onepair", 1)
-    return c
+    # operands up to l = 6 with power-of-two channel counts would go to the unrolled kernels (two launches, l <= 6 and
+    # l = 7..12), which are faster there; this file is about the single-pair family
+    c.set_option("unrolled_bwd_l6_split", 0)
+    yield c
+    c.set_option("unrolled_bwd_l6_split", 1)
 
 
 def c128(L):

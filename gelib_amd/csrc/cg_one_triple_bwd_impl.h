@@ -165,18 +165,6 @@ __device__ __forceinline__ void one_triple_cell(const BwdArgs &a, PairPtr pr, co
   }
 }
 
-template <int L1, int L2, bool WX, bool WY, int K, bool SMALL>
-__device__ __forceinline__ void one_triple_any_l(int only_dl, const BwdArgs &a, PairPtr pr, const float2 *xs,
-                                                 const float2 *ys, float2 *ximg, float2 *yimg, long long cell, int lane) {
-  static_for<2 * cmin_(L1, L2) + 1>([&](auto dc) __attribute__((always_inline)) {
-    constexpr int D = decltype(dc)::value;
-    if constexpr (one_triple_small(L1, L2, cabs_(L1 - L2) + D, K) == SMALL) {
-      if (only_dl == D)  // uniform
-        one_triple_cell<L1, L2, D, WX, WY, K>(a, pr, xs, ys, ximg, yimg, cell, lane);
-    }
-  });
-}
-
 // One part between memory and a wave's LDS image of it (rows contiguous); the channel count is a power of two.
 // Done by ONE wave for itself: the wave's LDS operations execute in order, so no block barrier is involved.
 template <bool TO_LDS>
@@ -202,9 +190,12 @@ __device__ __forceinline__ void wave_copy_part(const FastPart P, int rows, float
 
 // A wave takes whole cells, a.cells_per_block / 4 of them one after the other, independently of the other waves of its
 // block (they only share the block's LDS allocation): it stages x and y of a cell in its own piece of LDS, goes through
-// the cell's runs, parks the two gradients in LDS and writes them out in whole rows.
-template <bool WX, bool WY, int K, bool SMALL>
-__global__ void __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(SMALL ? 4 : 1)))
+// the cell's runs, parks the two gradients in LDS and writes them out in whole rows.  One kernel per triple: each gets
+// the registers its own body needs (one kernel with a switch over the triples spills in the larger bodies, since what
+// is live around the switch comes on top of every body).
+template <int L1, int L2, int D, bool WX, bool WY, int K>
+__global__ void __launch_bounds__(kBlock)
+    __attribute__((amdgpu_waves_per_eu(one_triple_small(L1, L2, cabs_(L1 - L2) + D, K) ? 4 : 1)))
 one_triple_bwd_kernel(const BwdArgs a) {
   extern __shared__ float lds[];
   const int xsize = a.xsize, ysize = a.ysize, cpb = a.cells_per_block;
@@ -214,7 +205,7 @@ one_triple_bwd_kernel(const BwdArgs a) {
   float2 *ximg = ys + ysize;
   float2 *yimg = ximg + xsize;
   const PairPtr p = (PairPtr)a.pairs;
-  const int only_dl = a.only_dl, per_wave = cpb / kWaves;
+  const int per_wave = cpb / kWaves;
   const long long first = (long long)blockIdx.x * cpb + (long long)wave * per_wave;
   for (int t = 0; t < per_wave; t++) {
     const long long cell = first + t;
@@ -222,17 +213,7 @@ one_triple_bwd_kernel(const BwdArgs a) {
     if (WY) wave_copy_part<true>(a.x[0], a.xrows[0], xs, cell, lane, false);
     if (WX) wave_copy_part<true>(a.y[0], a.yrows[0], ys, cell, lane, false);
     __builtin_amdgcn_wave_barrier();
-    switch (p->l1 * (kLT + 1) + p->l2) {
-#define GELIB_CASE(A, B)                                                                       \
-  case A * (kLT + 1) + B:                                                                      \
-    one_triple_any_l<A, B, WX, WY, K, SMALL>(only_dl, a, p, xs, ys, ximg, yimg, cell, lane);   \
-    break;
-#define GELIB_ROW(A) GELIB_CASE(A, 0) GELIB_CASE(A, 1) GELIB_CASE(A, 2) GELIB_CASE(A, 3) GELIB_CASE(A, 4)
-      GELIB_ROW(0) GELIB_ROW(1) GELIB_ROW(2) GELIB_ROW(3) GELIB_ROW(4)
-#undef GELIB_ROW
-#undef GELIB_CASE
-      default: break;
-    }
+    one_triple_cell<L1, L2, D, WX, WY, K>(a, p, xs, ys, ximg, yimg, cell, lane);
     __builtin_amdgcn_wave_barrier();
     if (WX) wave_copy_part<false>(a.xg[0], a.xrows[0], ximg, cell, lane, a.accumulate != 0);
     if (WY) wave_copy_part<false>(a.yg[0], a.yrows[0], yimg, cell, lane, a.accumulate != 0);
@@ -240,13 +221,35 @@ one_triple_bwd_kernel(const BwdArgs a) {
   }
 }
 
+template <int N, int I = 0, typename F>
+void host_for(F &&f) {
+  if constexpr (I < N) {
+    f(std::integral_constant<int, I>{});
+    host_for<N, I + 1>(f);
+  }
+}
+
+// Launches the kernel of (l1, l2, l) if it belongs to the class SMALL of this translation unit.
 template <int K, bool SMALL>
-int launch_one_triple_k(const BwdArgs &a, int nblocks, size_t lds, hipStream_t s) {
-  static_assert(kLT == 4, "the case table above lists l1, l2 = 0..4");
+int launch_one_triple_k(const BwdArgs &a, int l1, int l2, int l, int nblocks, size_t lds, hipStream_t s) {
   const bool wx = a.want_x != 0, wy = a.want_y != 0;
-  if (wx && wy) hipLaunchKernelGGL((one_triple_bwd_kernel<true, true, K, SMALL>), dim3(nblocks), dim3(kBlock), lds, s, a);
-  else if (wx) hipLaunchKernelGGL((one_triple_bwd_kernel<true, false, K, SMALL>), dim3(nblocks), dim3(kBlock), lds, s, a);
-  else hipLaunchKernelGGL((one_triple_bwd_kernel<false, true, K, SMALL>), dim3(nblocks), dim3(kBlock), lds, s, a);
+  bool found = false;
+  host_for<kLT + 1>([&](auto ac) {
+    host_for<kLT + 1>([&](auto bc) {
+      constexpr int A = decltype(ac)::value, B = decltype(bc)::value;
+      host_for<2 * cmin_(A, B) + 1>([&](auto dc) {
+        constexpr int D = decltype(dc)::value;
+        if constexpr (one_triple_small(A, B, cabs_(A - B) + D, K) == SMALL) {
+          if (l1 != A || l2 != B || l != cabs_(A - B) + D) return;
+          found = true;
+          if (wx && wy) hipLaunchKernelGGL((one_triple_bwd_kernel<A, B, D, true, true, K>), dim3(nblocks), dim3(kBlock), lds, s, a);
+          else if (wx) hipLaunchKernelGGL((one_triple_bwd_kernel<A, B, D, true, false, K>), dim3(nblocks), dim3(kBlock), lds, s, a);
+          else hipLaunchKernelGGL((one_triple_bwd_kernel<A, B, D, false, true, K>), dim3(nblocks), dim3(kBlock), lds, s, a);
+        }
+      });
+    });
+  });
+  if (!found) return GELIB_HIP_ERR_UNSUPPORTED;
   GELIB_HIP_TRY(hipGetLastError());
   return GELIB_HIP_OK;
 }

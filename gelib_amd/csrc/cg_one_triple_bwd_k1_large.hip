@@ -4,8 +4,8 @@
 
 namespace gelib_hip {
 
-int launch_one_triple_bwd_k1_large(const BwdArgs &a, int nblocks, size_t lds_bytes, hipStream_t s) {
-  return launch_one_triple_k<1, false>(a, nblocks, lds_bytes, s);
+int launch_one_triple_bwd_k1_large(const BwdArgs &a, int l1, int l2, int l, int nblocks, size_t lds_bytes, hipStream_t s) {
+  return launch_one_triple_k<1, false>(a, l1, l2, l, nblocks, lds_bytes, s);
 }
 
 }  // namespace gelib_hip

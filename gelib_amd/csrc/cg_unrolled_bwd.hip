@@ -17,10 +17,10 @@ int launch_unrolled_bwd_cg6_l6_pad(const BwdArgs &a, int nblocks, size_t lds_byt
 int launch_unrolled_bwd_cg6_hi(const BwdArgs &a, int nblocks, size_t lds_bytes, hipStream_t s);
 int launch_unrolled_bwd_cg6_hi_pad(const BwdArgs &a, int nblocks, size_t lds_bytes, hipStream_t s);
 int launch_unrolled_bwd_one(const BwdArgs &a, int nblocks, size_t lds_bytes, hipStream_t s);
-int launch_one_triple_bwd_k1_small(const BwdArgs &a, int nblocks, size_t lds_bytes, hipStream_t s);
-int launch_one_triple_bwd_k1_large(const BwdArgs &a, int nblocks, size_t lds_bytes, hipStream_t s);
-int launch_one_triple_bwd_k2_small(const BwdArgs &a, int nblocks, size_t lds_bytes, hipStream_t s);
-int launch_one_triple_bwd_k2_large(const BwdArgs &a, int nblocks, size_t lds_bytes, hipStream_t s);
+int launch_one_triple_bwd_k1_small(const BwdArgs &a, int l1, int l2, int l, int nblocks, size_t lds_bytes, hipStream_t s);
+int launch_one_triple_bwd_k1_large(const BwdArgs &a, int l1, int l2, int l, int nblocks, size_t lds_bytes, hipStream_t s);
+int launch_one_triple_bwd_k2_small(const BwdArgs &a, int l1, int l2, int l, int nblocks, size_t lds_bytes, hipStream_t s);
+int launch_one_triple_bwd_k2_large(const BwdArgs &a, int l1, int l2, int l, int nblocks, size_t lds_bytes, hipStream_t s);
 
 // The kernel built for one triple with 16 k channels in the second operand (k = 1, 2) and at least 16 in the first.
 size_t one_triple_bwd_lds_bytes(int xsize, int ysize) {   // per wave: the operands of a cell and its two gradients
@@ -30,8 +30,8 @@ size_t one_triple_bwd_lds_bytes(int xsize, int ysize) {   // per wave: the opera
 int launch_one_triple_bwd(const BwdArgs &a, int k, int l1, int l2, int l, int nblocks, size_t lds_bytes, hipStream_t s) {
   if (nblocks <= 0) return GELIB_HIP_OK;
   const bool small = k * (4 * (2 * l2 + 1) + 2 * (2 * l + 1)) + 5 * (2 * l1 + 1) <= 120;
-  if (k == 1) return small ? launch_one_triple_bwd_k1_small(a, nblocks, lds_bytes, s) : launch_one_triple_bwd_k1_large(a, nblocks, lds_bytes, s);
-  if (k == 2) return small ? launch_one_triple_bwd_k2_small(a, nblocks, lds_bytes, s) : launch_one_triple_bwd_k2_large(a, nblocks, lds_bytes, s);
+  if (k == 1) return small ? launch_one_triple_bwd_k1_small(a, l1, l2, l, nblocks, lds_bytes, s) : launch_one_triple_bwd_k1_large(a, l1, l2, l, nblocks, lds_bytes, s);
+  if (k == 2) return small ? launch_one_triple_bwd_k2_small(a, l1, l2, l, nblocks, lds_bytes, s) : launch_one_triple_bwd_k2_large(a, l1, l2, l, nblocks, lds_bytes, s);
   return GELIB_HIP_ERR_ARG;
 }
 

@@ -519,6 +519,8 @@ bool split_at_l6(const VecPlan &plan, const std::vector<View> &R, VecPlan &A, Ve
   return true;
 }
 
+int g_pairwise = 1;  // vectors of several parts with l above 7: one launch of the single-pair kernels per pair
+
 // The kernel families in the order they are tried, then the shape-agnostic kernels.
 int fwd_dispatch(const VecPlan &plan, const std::vector<View> &R, const std::vector<View> &X, const std::vector<View> &Y,
                  int accumulate, hipStream_t s) {
@@ -568,11 +570,46 @@ int fwd_dispatch(const VecPlan &plan, const std::vector<View> &R, const std::vec
       t_last_path = kPathOnePair;
       return GELIB_HIP_OK;
     }
-    rc = staged_vec_fwd(plan, rd, xd, yd, accumulate != 0, s, &used);
-    if (rc) return rc;
-    if (used) {
-      t_last_path = kPathStaged;
-      return GELIB_HIP_OK;
+    {
+      // Vectors of several parts with l above 7: one launch of the matrix-core single-pair kernel per (x part, y part)
+      // pair (every pair writes channel blocks of its own); a pair that kernel does not take goes through this
+      // dispatch by itself.
+      int lop = 0;
+      for (auto &v : X) lop = std::max(lop, v.l);
+      for (auto &v : Y) lop = std::max(lop, v.l);
+      if (g_pairwise && !plan.diag && X.size() * Y.size() >= 2 && lop > 7) {
+        bool any = false;
+        for (int p = 0; p < (int)X.size(); p++)
+          for (int q = 0; q < (int)Y.size(); q++) {
+            VecPlan sub;
+            sub.diag = plan.diag;
+            for (int k = 0; k < 3; k++) sub.E[k] = plan.E[k];
+            for (auto t : plan.triples)
+              if (t.xi == p && t.yi == q) {
+                t.xi = t.yi = 0;
+                sub.triples.push_back(t);
+              }
+            if (sub.triples.empty()) continue;
+            rc = onepair_mfma_vec_fwd(sub, rd, {X[p].d}, {Y[q].d}, accumulate != 0, s, &used);
+            if (rc) return rc;
+            if (used) any = true;
+            else if (!any) goto whole;  // not even the first pair: the vector stays in one piece
+            else if ((rc = fwd_dispatch(sub, R, {X[p]}, {Y[q]}, accumulate, s))) return rc;
+          }
+        if (any) {
+          t_last_path = kPathOnePair;
+          return GELIB_HIP_OK;
+        }
+      }
+    }
+  whole:
+    {
+      rc = staged_vec_fwd(plan, rd, xd, yd, accumulate != 0, s, &used);
+      if (rc) return rc;
+      if (used) {
+        t_last_path = kPathStaged;
+        return GELIB_HIP_OK;
+      }
     }
   }
   t_last_path = kPathGeneric;
@@ -628,7 +665,6 @@ int vec_fwd_entry(bool diag, int nr, const gelib_part_desc *r, int nx, const gel
 // its share to the two gradient parts it touches (launches on one stream run one after the other, so the order of the
 // additions is fixed).  The any-l kernels would otherwise take such vectors in one pass that adds partial sums into LDS
 // with float atomics; g is read once either way.  Taken only when every pair is one the single-pair kernels accept.
-int g_pairwise = 1;
 int pairwise_onepair_bwd(const VecPlan &plan, const std::vector<View> &G, const std::vector<View> &X,
                          const std::vector<View> &Y, const std::vector<View> &XG, const std::vector<View> &YG,
                          const std::vector<const gelib_part_desc *> &gd, bool want_x, bool want_y, int accumulate,

@@ -1,5 +1,7 @@
-// Backward pass of a product of ONE x part with ONE y part of large l, 8 x 8 channels, on the matrix cores: both
-// gradients from one pass over g (the l1 = l2 = 10, all 21 l case; any l1 <= 15, l2 <= 15, at most 22 values of l).
+// Backward pass of a product of ONE x part with ONE y part of large l on the matrix cores: both gradients from one pass
+// over g (the l1 = l2 = 10, all 21 l case; any l1 <= 15, l2 <= 15, at most 22 values of l).  Described for 8 x 8
+// channels, one wave per cell; PairShape below says how the other channel counts map onto the same scheme (16 channels:
+// one tile instead of four; 128 or 256 channels: two or four waves per cell, 64 channels each).
 //
 // For one row number m = m1 + m2 the contraction over l,
 //     Q[m1, chan] = sum_l C_l[m1, m - m1] g_l[m, chan],
@@ -34,6 +36,7 @@
 // 32-byte pieces: 1.47 ms instead of the any-l kernel's 1.05.)
 #include <cstring>
 #include <map>
+#include <type_traits>
 #include <mutex>
 #include <vector>
 
@@ -67,6 +70,7 @@ typedef float v4f __attribute__((ext_vector_type(4)));
 typedef const __attribute__((address_space(1))) v4f *GlobalIn4;
 typedef __attribute__((address_space(1))) v4f *GlobalOut4;
 typedef const __attribute__((address_space(1))) float *GlobalIn1;
+typedef __attribute__((address_space(1))) float *GlobalOut1;
 typedef const __attribute__((address_space(4))) int *IntPtr;
 
 __device__ __forceinline__ float wave_shr1(float v) {  // lane k receives lane k - 1, lane 0 receives 0
@@ -75,19 +79,54 @@ __device__ __forceinline__ float wave_shr1(float v) {  // lane k receives lane k
 
 constexpr int kQueue = 6;  // steps whose operands are in flight or waiting in registers
 
-__global__ void __launch_bounds__(64) onepair_mfma_bwd_kernel(const OnePairMfmaArgs a) {
+// How the N1 x N2 channels (a, j) of a block, channel a N2 + j, meet the matrix tiles.  A wave takes 64 neighbouring
+// channels, four tiles of 32 floats (lane i loads floats 4 i .. 4 i + 3 of its piece of a row, one float per tile), or
+// all 16 channels, one tile (lane i loads float i).  Register v of the tiles of lane (i, h) then holds channel
+//     (CW / 4) (v / 4) + (CW / 8) h + jj,   jj = 0 .. JL - 1,
+// of the wave's CW channels (four tiles: jj = 2 (v % 4) + e / 2, real part in tile e even, imaginary part in tile e + 1;
+// one tile: jj = (v % 4) / 2, real part in v even, imaginary part in v + 1).  If the lane's JL channels are a whole row of
+// j (JL = N2), the two halves of the wave hold different a (a = 2 (v / 4) + h): a lane's x-gradient sums are complete,
+// the y-gradient is added over the halves.  Otherwise (2 JL = N2) the halves hold different j (j = JL h + jj,
+// a = v / 4): the y-gradient sums of the wave are complete, the x-gradient is added over the halves.  Several waves:
+// wave w has the channels a = w CW / N2 .. of x, and the y-gradient is added over the waves at the end.
+template <int N1, int N2>
+struct PairShape {
+  static constexpr int kChan = N1 * N2;
+  static constexpr int T = kChan >= 64 ? 4 : 1;
+  static constexpr int W = kChan >= 64 ? kChan / 64 : 1;
+  static constexpr int CW = 16 * T;
+  static constexpr int JL = T == 4 ? 8 : 2;
+  static constexpr bool kHalfIsA = JL == N2;
+  static constexpr int kSlots = kHalfIsA ? 2 : 1;  // images of the y-gradient a wave parks its rows in
+  static constexpr int kAWave = CW / N2;           // channels a of a wave
+  static_assert(kChan == 16 || kChan % 64 == 0, "16 channels, or whole waves of 64");
+  static_assert(W >= 1 && W <= 4, "at most four waves per cell");
+  static_assert(JL == N2 || 2 * JL == N2, "a lane holds a whole row of j or half of one");
+};
+
+template <int N1, int N2>
+__global__ void __launch_bounds__((64 * PairShape<N1, N2>::W)) onepair_mfma_bwd_kernel(const OnePairMfmaArgs a) {
+  using Sh = PairShape<N1, N2>;
+  constexpr int T = Sh::T, JL = Sh::JL, W = Sh::W;
+  constexpr bool kHalfIsA = Sh::kHalfIsA;
+  using GT = std::conditional_t<T == 4, v4f, float>;
   __shared__ unsigned long long gbase[kNLm + 1];  // address of row 0 of the cell's block in part dl; slot nl: a harmless row
   __shared__ unsigned growb[kNLm + 1];            // distance between rows in bytes
-  __shared__ float2 ys[(2 * kMaxLm + 1) * 8];
-  __shared__ float2 accy[2][(2 * kMaxLm + 1) * 8];
-  const int lane = threadIdx.x, i = lane & 31, h = lane >> 5;
+  __shared__ float2 ys[(2 * kMaxLm + 1) * N2];
+  __shared__ float2 accy_all[W * Sh::kSlots][(2 * kMaxLm + 1) * N2];
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63, i = lane & 31, h = lane >> 5;
+  float2(*accy)[(2 * kMaxLm + 1) * N2] = accy_all + wave * Sh::kSlots;
+  const int jbase = kHalfIsA ? 0 : JL * h;  // the lane's first channel j
+  // channel a of the sums q = 0..3 of the lane
+  auto a_of = [&](int q) __attribute__((always_inline)) { return wave * Sh::kAWave + (kHalfIsA ? 2 * q + h : q); };
   const int l1 = a.l1, l2 = a.l2, lmin = a.lmin, lt = a.lt, nl = a.nl;
   const long long cell = blockIdx.x;
   const int r1 = 2 * l1 + 1, r2 = 2 * l2 + 1;
 
   static_for<kNLm>([&](auto dc) __attribute__((always_inline)) {
     constexpr int dl = decltype(dc)::value;
-    if (lane == 0 && dl < nl) {
+    if (threadIdx.x == 0 && dl < nl) {
       const FastPart P = a.g[dl];
       const bool there = P.ptr != nullptr;
       // a triple that is not there reads the coefficient table (finite numbers) and meets coefficients that are zero
@@ -95,20 +134,20 @@ __global__ void __launch_bounds__(64) onepair_mfma_bwd_kernel(const OnePairMfmaA
       growb[dl] = there ? (unsigned)P.sm * 8u : 0u;
     }
   });
-  if (lane == 0) {
+  if (threadIdx.x == 0) {
     gbase[nl] = (unsigned long long)a.coef;
     growb[nl] = 0u;
   }
-  for (int e = lane; e < r2 * 8; e += 64) {
-    ys[e] = a.y.ptr[cell * a.y.sb + (long long)(e >> 3) * a.y.sm + (e & 7)];
-    accy[0][e] = make_float2(0.f, 0.f);
-    accy[1][e] = make_float2(0.f, 0.f);
+  for (int e = threadIdx.x; e < r2 * N2; e += 64 * W) {
+    ys[e] = a.y.ptr[cell * a.y.sb + (long long)(e / N2) * a.y.sm + (e % N2)];
+#pragma unroll
+    for (int k = 0; k < W * Sh::kSlots; k++) accy_all[k][e] = make_float2(0.f, 0.f);
   }
-  // the lane's row of x: m1 = i - l1, channels 2 b + h; a lane beyond the rows holds zeros (so do its coefficients)
+  // the lane's row of x: m1 = i - l1, its four channels a; a lane beyond the rows holds zeros (so do its coefficients)
   float2 xv[4];
 #pragma unroll
   for (int b = 0; b < 4; b++)
-    xv[b] = i < r1 ? a.x.ptr[cell * a.x.sb + (long long)i * a.x.sm + (2 * b + h)] : make_float2(0.f, 0.f);
+    xv[b] = i < r1 ? a.x.ptr[cell * a.x.sb + (long long)i * a.x.sm + a_of(b)] : make_float2(0.f, 0.f);
   __syncthreads();
 
   // The steps of all m form one sequence (two values of l per step, m ascending), padded with idle steps to a multiple
@@ -149,26 +188,30 @@ __global__ void __launch_bounds__(64) onepair_mfma_bwd_kernel(const OnePairMfmaA
       c.left = 1 << 30;
     }
   };
-  v4f G[kQueue];
+  GT G[kQueue];
   float C[kQueue];
   long long coef_at = lane;  // the lane's coefficient of the step that is fetched next
-  auto fetch = [&](const Cursor &c, v4f &g, float &cf) __attribute__((always_inline)) {
+  // the lane's piece of a row: 4 T bytes, 512 bytes on for every wave; the harmless row (the coefficient table) is
+  // read at the same offsets, which its idle steps at the end cover
+  const unsigned lane_off = (unsigned)wave * 512u + (unsigned)i * (4u * T);
+  auto fetch = [&](const Cursor &c, GT &g, float &cf) __attribute__((always_inline)) {
     int dl = c.dlb + h;
     dl = dl < nl ? dl : nl;
     const unsigned long long base = gbase[dl];
     const unsigned rowb = growb[dl];
-    const unsigned long long addr = base + (unsigned long long)((unsigned)(c.m + lmin + dl) * rowb) + (unsigned)i * 16u;
-    g = *(GlobalIn4)addr;
+    const unsigned long long addr = base + (unsigned long long)((unsigned)(c.m + lmin + dl) * rowb) + lane_off;
+    if constexpr (T == 4) g = *(GlobalIn4)addr;
+    else g = *(GlobalIn1)addr;
     cf = *((GlobalIn1)a.coef + coef_at);   // the table ends with a queue's worth of idle steps
     coef_at += 64;
   };
 
-  float2 ax[4], S[8];
+  float2 ax[4], S[JL];
 #pragma unroll
   for (int b = 0; b < 4; b++) ax[b] = make_float2(0.f, 0.f);
 #pragma unroll
-  for (int j = 0; j < 8; j++) S[j] = make_float2(0.f, 0.f);
-  f16v D[4];
+  for (int j = 0; j < JL; j++) S[j] = make_float2(0.f, 0.f);
+  f16v D[T];
 
   // the sums of one m are in D: both gradients, then every row of the y-gradient moves one lane up
   auto finish_m = [&](int m) __attribute__((always_inline)) {
@@ -178,10 +221,10 @@ __global__ void __launch_bounds__(64) onepair_mfma_bwd_kernel(const OnePairMfmaA
     const int mlane = (paired && m > 0 && (i - l1) <= mneg + l2) ? mneg : m;
     int m2 = mlane - (i - l1);
     m2 = m2 < -l2 ? -l2 : (m2 > l2 ? l2 : m2);
-    const float4 *yrow = reinterpret_cast<const float4 *>(ys + (m2 + l2) * 8);
-    float2 yv[8];
+    const float4 *yrow = reinterpret_cast<const float4 *>(ys + (m2 + l2) * N2 + jbase);
+    float2 yv[JL];
 #pragma unroll
-    for (int q = 0; q < 4; q++) {
+    for (int q = 0; q < JL / 2; q++) {
       const float4 t = yrow[q];
       yv[2 * q] = make_float2(t.x, t.y);
       yv[2 * q + 1] = make_float2(t.z, t.w);
@@ -189,35 +232,39 @@ __global__ void __launch_bounds__(64) onepair_mfma_bwd_kernel(const OnePairMfmaA
 #pragma unroll
     for (int b = 0; b < 4; b++)
 #pragma unroll
-      for (int vv = 0; vv < 4; vv++)
-#pragma unroll
-        for (int e2 = 0; e2 < 2; e2++) {
-          const float qr = D[2 * e2][4 * b + vv], qi = D[2 * e2 + 1][4 * b + vv];
-          const int j = 2 * vv + e2;
-          ax[b].x = fmaf(qr, yv[j].x, ax[b].x);
-          ax[b].x = fmaf(qi, yv[j].y, ax[b].x);
-          ax[b].y = fmaf(qi, yv[j].x, ax[b].y);
-          ax[b].y = fmaf(-qr, yv[j].y, ax[b].y);
-          S[j].x = fmaf(qr, xv[b].x, S[j].x);
-          S[j].x = fmaf(qi, xv[b].y, S[j].x);
-          S[j].y = fmaf(qi, xv[b].x, S[j].y);
-          S[j].y = fmaf(-qr, xv[b].y, S[j].y);
+      for (int j = 0; j < JL; j++) {
+        float qr, qi;
+        if constexpr (T == 4) {
+          qr = D[2 * (j & 1)][4 * b + (j >> 1)];
+          qi = D[2 * (j & 1) + 1][4 * b + (j >> 1)];
+        } else {
+          qr = D[0][4 * b + 2 * j];
+          qi = D[0][4 * b + 2 * j + 1];
         }
+        ax[b].x = fmaf(qr, yv[j].x, ax[b].x);
+        ax[b].x = fmaf(qi, yv[j].y, ax[b].x);
+        ax[b].y = fmaf(qi, yv[j].x, ax[b].y);
+        ax[b].y = fmaf(-qr, yv[j].y, ax[b].y);
+        S[j].x = fmaf(qr, xv[b].x, S[j].x);
+        S[j].x = fmaf(qi, xv[b].y, S[j].x);
+        S[j].y = fmaf(qi, xv[b].x, S[j].y);
+        S[j].y = fmaf(-qr, xv[b].y, S[j].y);
+      }
     if (!is_last(m)) {  // the row that leaves m1 = l1 is complete (paired: its terms with m > 0 are); after the last m the rows stay where they are
 #pragma unroll
-      for (int j = 0; j < 8; j++) {
+      for (int j = 0; j < JL; j++) {
         S[j].x = wave_shr1(S[j].x);
         S[j].y = wave_shr1(S[j].y);
       }
       const int mdone = m - l1;  // the row now in column r1
       if (i == r1 && mdone >= -l2 && mdone <= l2) {
-        float4 *dst = reinterpret_cast<float4 *>(accy[h] + (mdone + l2) * 8);
+        float4 *dst = reinterpret_cast<float4 *>(accy[kHalfIsA ? h : 0] + (mdone + l2) * N2 + jbase);
 #pragma unroll
-        for (int q = 0; q < 4; q++) dst[q] = make_float4(S[2 * q].x, S[2 * q].y, S[2 * q + 1].x, S[2 * q + 1].y);
+        for (int q = 0; q < JL / 2; q++) dst[q] = make_float4(S[2 * q].x, S[2 * q].y, S[2 * q + 1].x, S[2 * q + 1].y);
       }
       if (i == 0 || i >= r1) {  // zeros enter at m1 = -l1; nothing travels on beyond the last column
 #pragma unroll
-        for (int j = 0; j < 8; j++) S[j] = make_float2(0.f, 0.f);
+        for (int j = 0; j < JL; j++) S[j] = make_float2(0.f, 0.f);
       }
     }
   };
@@ -236,21 +283,21 @@ __global__ void __launch_bounds__(64) onepair_mfma_bwd_kernel(const OnePairMfmaA
   for (int q0 = 0; q0 < nsteps; q0 += kQueue) {
     static_for<kQueue>([&](auto kc) __attribute__((always_inline)) {
       constexpr int k = decltype(kc)::value;
-      const v4f g = G[k];
+      const GT g = G[k];
       const float c = C[k];
+      auto piece = [&](int e) __attribute__((always_inline)) {
+        if constexpr (T == 4) return g[e];
+        else return g;
+      };
       if (fresh) {  // uniform: the first step of an m starts from zero (a constant operand, no registers to clear)
         f16v zero;
 #pragma unroll
         for (int v = 0; v < 16; v++) zero[v] = 0.f;
-        D[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(g.x, c, zero, 0, 0, 0);
-        D[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(g.y, c, zero, 0, 0, 0);
-        D[2] = __builtin_amdgcn_mfma_f32_32x32x2f32(g.z, c, zero, 0, 0, 0);
-        D[3] = __builtin_amdgcn_mfma_f32_32x32x2f32(g.w, c, zero, 0, 0, 0);
+#pragma unroll
+        for (int e = 0; e < T; e++) D[e] = __builtin_amdgcn_mfma_f32_32x32x2f32(piece(e), c, zero, 0, 0, 0);
       } else {
-        D[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(g.x, c, D[0], 0, 0, 0);
-        D[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(g.y, c, D[1], 0, 0, 0);
-        D[2] = __builtin_amdgcn_mfma_f32_32x32x2f32(g.z, c, D[2], 0, 0, 0);
-        D[3] = __builtin_amdgcn_mfma_f32_32x32x2f32(g.w, c, D[3], 0, 0, 0);
+#pragma unroll
+        for (int e = 0; e < T; e++) D[e] = __builtin_amdgcn_mfma_f32_32x32x2f32(piece(e), c, D[e], 0, 0, 0);
       }
       fresh = ck.left == 1 && closes(ck.m);  // the next step starts new sums
       fetch(cf, G[k], C[k]);
@@ -265,9 +312,9 @@ __global__ void __launch_bounds__(64) onepair_mfma_bwd_kernel(const OnePairMfmaA
   {
     const int m2 = (paired ? 0 : lt) - (i - l1);
     if (i < r1 && m2 >= -l2 && m2 <= l2) {
-      float4 *dst = reinterpret_cast<float4 *>(accy[h] + (m2 + l2) * 8);
+      float4 *dst = reinterpret_cast<float4 *>(accy[kHalfIsA ? h : 0] + (m2 + l2) * N2 + jbase);
 #pragma unroll
-      for (int q = 0; q < 4; q++) {
+      for (int q = 0; q < JL / 2; q++) {
         const float4 o = dst[q];
         dst[q] = make_float4(o.x + S[2 * q].x, o.y + S[2 * q].y, o.z + S[2 * q + 1].x, o.w + S[2 * q + 1].y);
       }
@@ -276,18 +323,28 @@ __global__ void __launch_bounds__(64) onepair_mfma_bwd_kernel(const OnePairMfmaA
   __syncthreads();
 
   const bool accumulate = a.accumulate != 0;
+  if constexpr (!kHalfIsA) {  // the two halves of the wave hold the sums over different j
+#pragma unroll
+    for (int b = 0; b < 4; b++) {
+      ax[b].x += __shfl_xor(ax[b].x, 32);
+      ax[b].y += __shfl_xor(ax[b].y, 32);
+    }
+  }
   if (i < r1) {
 #pragma unroll
     for (int b = 0; b < 4; b++) {
-      float2 *p = a.xg.ptr + cell * a.xg.sb + (long long)i * a.xg.sm + (2 * b + h);
+      if (!kHalfIsA && (b >> 1) != h) continue;  // each half stores two of the four
+      float2 *p = a.xg.ptr + cell * a.xg.sb + (long long)i * a.xg.sm + a_of(b);
       float2 o = ax[b];
       if (accumulate) o.x += p->x, o.y += p->y;
       *p = o;
     }
   }
-  for (int e = lane; e < r2 * 8; e += 64) {
-    float2 *p = a.yg.ptr + cell * a.yg.sb + (long long)(e >> 3) * a.yg.sm + (e & 7);
-    float2 o = make_float2(accy[0][e].x + accy[1][e].x, accy[0][e].y + accy[1][e].y);
+  for (int e = threadIdx.x; e < r2 * N2; e += 64 * W) {
+    float2 *p = a.yg.ptr + cell * a.yg.sb + (long long)(e / N2) * a.yg.sm + (e % N2);
+    float2 o = accy_all[0][e];
+#pragma unroll
+    for (int k = 1; k < W * Sh::kSlots; k++) o.x += accy_all[k][e].x, o.y += accy_all[k][e].y;
     if (accumulate) o.x += p->x, o.y += p->y;
     *p = o;
   }
@@ -299,113 +356,141 @@ constexpr int kColsF = 24;                     // columns (values of l) the forw
 constexpr int kCellsF = 8;                     // cells (waves) per block of the forward kernel
 
 // Forward: g[] are the parts of the product (written), x and y the operands.  A block of eight waves takes eight cells
-// and shares one copy of the coefficient table in LDS (2 x 24 floats per step, 44 KB at l1 = l2 = 10), loaded by all of
-// its threads while the waves set up their cells.  Nothing is loaded from memory once the rows are being stored: loads
-// and stores return through one in-order counter, and a wait for a load issued behind stores waits for the stores to
-// be acknowledged (with the coefficients fetched from memory step by step the waves spent a third of their time so).
-// All parts have the same row length (a.rowb; the host sends other cases to the any-l kernels).
+// (four or two when a cell's 128 or 256 channels take two or four waves) and shares one copy of the coefficient table
+// in LDS (2 x 24 floats per step, 44 KB at l1 = l2 = 10), loaded by all of its threads while the waves set up their
+// cells.  Nothing is loaded from memory once the rows are being stored: loads and stores return through one in-order
+// counter, and a wait for a load issued behind stores waits for the stores to be acknowledged (with the coefficients
+// fetched from memory step by step the waves spent a third of their time so).
+// ONE_ROWB: all parts have the same row length a.rowb (true whenever the parts hold just this pair's block); otherwise
+// every register row carries its own.
+// Channels: a wave's columns are the floats of 64 neighbouring channels (column i of tile t = float 4 i + t: the lane
+// forms the products of channels 2 i and 2 i + 1 = (a, j) and (a, j + 1)), or of all 16 (one tile, column i = float i:
+// the lane forms the real or the imaginary part of channel i / 2).
+template <int N1, int N2, bool ONE_ROWB>
 __global__ void __launch_bounds__(64 * kCellsF) onepair_mfma_fwd_kernel(const OnePairMfmaArgs a) {
+  using Sh = PairShape<N1, N2>;
+  constexpr int T = Sh::T, W = Sh::W;
+  constexpr int XROW = N1 * 8, YROW = N2 * 8;  // bytes of a row of the operands in LDS
   extern __shared__ float4 smem4[];
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int cw = wave / W, ww = wave % W;  // the wave's cell within the block, its piece of the cell's channels
   const int lane = threadIdx.x & 63, i = lane & 31, h = lane >> 5;
   const int l1 = a.l1, l2 = a.l2, lmin = a.lmin, lt = a.lt, nl = a.nl;
   const int r1 = 2 * l1 + 1, r2 = 2 * l2 + 1;
   float *ctab = reinterpret_cast<float *>(smem4);
   const int tab4 = a.nsteps_fwd * (2 * kColsF / 4);  // float4s of the table
-  // per wave: x with one row of zeros behind it, y with one row of zeros on either side (the second m1 of an odd count
+  // per cell: x with one row of zeros behind it, y with one row of zeros on either side (the second m1 of an odd count
   // reads one row too far; its coefficient is zero, so the row must only be finite)
-  const int wave4 = (r1 + 1 + r2 + 2) * 4;  // float4s: a row is 8 complex = 4 float4
-  float2 *xs = reinterpret_cast<float2 *>(smem4 + tab4 + wave * wave4);
-  float2 *ys = xs + (r1 + 1) * 8 + 8;  // row 0 of y; the zero row sits in front of it
+  const int cell4 = ((r1 + 1) * N1 + (r2 + 2) * N2) / 2;  // float4s
+  float2 *xs = reinterpret_cast<float2 *>(smem4 + tab4 + cw * cell4);
+  float2 *ys = xs + (r1 + 1) * N1 + N2;  // row 0 of y; the zero row sits in front of it
   {
     const float4 *src = reinterpret_cast<const float4 *>(a.coef_fwd);
     for (int e = threadIdx.x; e < tab4; e += 64 * kCellsF) smem4[e] = src[e];
   }
-  long long cell = (long long)blockIdx.x * kCellsF + wave;
+  long long cell = (long long)blockIdx.x * (kCellsF / W) + cw;
   const bool live = cell < a.ncells;  // a wave beyond the last cell repeats it and stores nothing
   cell = live ? cell : a.ncells - 1;
-  for (int e = lane; e < r1 * 8; e += 64) xs[e] = a.x.ptr[cell * a.x.sb + (long long)(e >> 3) * a.x.sm + (e & 7)];
-  for (int e = lane; e < r2 * 8; e += 64) ys[e] = a.y.ptr[cell * a.y.sb + (long long)(e >> 3) * a.y.sm + (e & 7)];
-  if (lane < 8) {
-    xs[r1 * 8 + lane] = make_float2(0.f, 0.f);
-    ys[lane - 8] = make_float2(0.f, 0.f);
-    ys[r2 * 8 + lane] = make_float2(0.f, 0.f);
+  for (int e = ww * 64 + lane; e < r1 * N1; e += 64 * W) xs[e] = a.x.ptr[cell * a.x.sb + (long long)(e / N1) * a.x.sm + (e % N1)];
+  for (int e = ww * 64 + lane; e < r2 * N2; e += 64 * W) ys[e] = a.y.ptr[cell * a.y.sb + (long long)(e / N2) * a.y.sm + (e % N2)];
+  if (ww == 0) {
+    if (lane < N1) xs[r1 * N1 + lane] = make_float2(0.f, 0.f);
+    if (lane < N2) {
+      ys[lane - N2] = make_float2(0.f, 0.f);
+      ys[r2 * N2 + lane] = make_float2(0.f, 0.f);
+    }
   }
-  // Register v of a tile belongs to part l = lmin + 8 (v / 4) + 4 h + v % 4.  cur[v]: the lane's 16 bytes of row m of
+  // Register v of a tile belongs to part l = lmin + 8 (v / 4) + 4 h + v % 4.  cur[v]: the lane's 4 T bytes of row m of
   // that part for the m at hand (the rows of a part start at m = -l; before that the address is not used), advanced by
   // the row length after every m.  Bit v of `there`: the part exists and the wave has a cell.
   const long long rowb = a.rowb;
   unsigned long long cur[16];
+  unsigned rowbv[ONE_ROWB ? 1 : 16];
   unsigned there = 0;
   static_for<16>([&](auto vc) __attribute__((always_inline)) {
     constexpr int v = decltype(vc)::value;
     cur[v] = 0;
+    if constexpr (!ONE_ROWB) rowbv[v] = 0;
     static_for<2>([&](auto hc) __attribute__((always_inline)) {
       constexpr int dl = 8 * (v / 4) + 4 * decltype(hc)::value + (v % 4);
       if constexpr (dl < kNLm) {
         if (hc.value == h && dl < nl && live && a.g[dl].ptr != nullptr) {
           const FastPart P = a.g[dl];
+          const long long rb = ONE_ROWB ? rowb : (long long)P.sm * 8;
           cur[v] = (unsigned long long)(P.ptr + cell * P.sb + (a.offs[dl] + a.offs_add)) +
-                   (unsigned long long)((long long)(lmin + dl - lt) * rowb) + (unsigned)i * 16u;
+                   (unsigned long long)((long long)(lmin + dl - lt) * rb) + (unsigned)ww * 512u + (unsigned)i * (4u * T);
+          if constexpr (!ONE_ROWB) rowbv[v] = (unsigned)rb;
           there |= 1u << v;
         }
       }
     });
   });
   const int lbase = lmin + 4 * h;  // l of register v: lbase + 8 (v / 4) + v % 4
-  const char *xmine = reinterpret_cast<const char *>(xs + (i >> 2));   // row r: + r * 64 bytes
-  const char *ymine = reinterpret_cast<const char *>(ys) + (i & 3) * 16;  // row r: + r * 64: y[r, j], y[r, j + 1]
+  // the lane's channel(s): (a, j), and for a wave of 64 channels (a, j + 1) as well
+  const int chan = T == 4 ? ww * 64 + 2 * i : i >> 1;
+  const char *xmine = reinterpret_cast<const char *>(xs + chan / N2);  // row r: + r * XROW bytes
+  const char *ymine = reinterpret_cast<const char *>(ys + chan % N2);  // row r: + r * YROW
+  const bool imag = (i & 1) != 0;  // one tile: the lane's float is the imaginary part
   // the lane's coefficient of step s: 192 s bytes on; the columns beyond the table's read its last one, which is zero
   const char *cmine = reinterpret_cast<const char *>(ctab + h * kColsF + (i < kColsF ? i : kColsF - 1));
   __syncthreads();
 
   const bool accumulate = a.accumulate != 0;
-  f16v D[4];
+  f16v D[T];
   int at = 0;  // first step of the m at hand in the table
   for (int m = -lt; m <= lt; m++) {
     const int lo = (m - l2 > -l1) ? m - l2 : -l1, hi = (m + l2 < l1) ? m + l2 : l1;
     const int nst = (hi - lo + 2) >> 1;
     // step k: m1 = lo + 2 k + h, m2 = m - m1: the addresses of a step are those of step 0 plus constants (y runs
     // backwards: its base is the row of the last unrolled step, so that the constants are not negative)
-    const char *xm = xmine + (lo + h + l1) * 64;
-    const char *ym = ymine + (m - lo - h + l2 - 2 * (kStepsM - 1)) * 64;
+    const char *xm = xmine + (lo + h + l1) * XROW;
+    const char *ym = ymine + (m - lo - h + l2 - 2 * (kStepsM - 1)) * YROW;
     const char *cm = cmine + at * (2 * kColsF * 4);
     static_for<kStepsM>([&](auto kc) __attribute__((always_inline)) {
       constexpr int k = decltype(kc)::value;
       if (k < nst) {  // uniform
-        const float2 xv = *reinterpret_cast<const float2 *>(xm + k * 128);
-        const float4 yv = *reinterpret_cast<const float4 *>(ym + (kStepsM - 1 - k) * 128);
+        const float2 xv = *reinterpret_cast<const float2 *>(xm + k * 2 * XROW);
         const float c = *reinterpret_cast<const float *>(cm + k * (2 * kColsF * 4));
-        const float p0 = fmaf(-xv.y, yv.y, xv.x * yv.x), p1 = fmaf(xv.y, yv.x, xv.x * yv.y);
-        const float p2 = fmaf(-xv.y, yv.w, xv.x * yv.z), p3 = fmaf(xv.y, yv.z, xv.x * yv.w);
+        float p[T];
+        if constexpr (T == 4) {
+          const float4 yv = *reinterpret_cast<const float4 *>(ym + (kStepsM - 1 - k) * 2 * YROW);
+          p[0] = fmaf(-xv.y, yv.y, xv.x * yv.x), p[1] = fmaf(xv.y, yv.x, xv.x * yv.y);
+          p[2] = fmaf(-xv.y, yv.w, xv.x * yv.z), p[3] = fmaf(xv.y, yv.z, xv.x * yv.w);
+        } else {
+          const float2 yv = *reinterpret_cast<const float2 *>(ym + (kStepsM - 1 - k) * 2 * YROW);
+          p[0] = imag ? fmaf(xv.y, yv.x, xv.x * yv.y) : fmaf(-xv.y, yv.y, xv.x * yv.x);
+        }
         if constexpr (k == 0) {  // the first step of an m starts from zero (a constant operand, no registers to clear)
           f16v zero;
 #pragma unroll
           for (int v = 0; v < 16; v++) zero[v] = 0.f;
-          D[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(c, p0, zero, 0, 0, 0);
-          D[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(c, p1, zero, 0, 0, 0);
-          D[2] = __builtin_amdgcn_mfma_f32_32x32x2f32(c, p2, zero, 0, 0, 0);
-          D[3] = __builtin_amdgcn_mfma_f32_32x32x2f32(c, p3, zero, 0, 0, 0);
+#pragma unroll
+          for (int e = 0; e < T; e++) D[e] = __builtin_amdgcn_mfma_f32_32x32x2f32(c, p[e], zero, 0, 0, 0);
         } else {
-          D[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(c, p0, D[0], 0, 0, 0);
-          D[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(c, p1, D[1], 0, 0, 0);
-          D[2] = __builtin_amdgcn_mfma_f32_32x32x2f32(c, p2, D[2], 0, 0, 0);
-          D[3] = __builtin_amdgcn_mfma_f32_32x32x2f32(c, p3, D[3], 0, 0, 0);
+#pragma unroll
+          for (int e = 0; e < T; e++) D[e] = __builtin_amdgcn_mfma_f32_32x32x2f32(c, p[e], D[e], 0, 0, 0);
         }
       }
     });
-    // register v of the four tiles: floats 4 i .. 4 i + 3 of row m of its part
+    // register v of the tiles: the lane's floats of row m of its part
     const int mabs = m < 0 ? -m : m;
 #pragma unroll
     for (int v = 0; v < 16; v++) {
       if (((there >> v) & 1u) && lbase + (8 * (v / 4) + v % 4) >= mabs) {
-        GlobalOut4 p = (GlobalOut4)cur[v];
-        v4f o;
-        o.x = D[0][v], o.y = D[1][v], o.z = D[2][v], o.w = D[3][v];
-        if (accumulate) o += *p;
-        *p = o;
+        if constexpr (T == 4) {
+          GlobalOut4 q = (GlobalOut4)cur[v];
+          v4f o;
+          o.x = D[0][v], o.y = D[1][v], o.z = D[2][v], o.w = D[3][v];
+          if (accumulate) o += *q;
+          *q = o;
+        } else {
+          GlobalOut1 q = (GlobalOut1)cur[v];
+          float o = D[0][v];
+          if (accumulate) o += *q;
+          *q = o;
+        }
       }
-      cur[v] += rowb;
+      cur[v] += ONE_ROWB ? (unsigned long long)rowb : (unsigned long long)rowbv[v];
     }
     at += nst;
   }
@@ -502,10 +587,52 @@ int device_tables(int l1, int l2, int lmin, int lt, int nl, const std::vector<in
   return GELIB_HIP_OK;
 }
 
+// The channel counts the backward kernel is built for.
+#define GELIB_ONEPAIR_SHAPES(X) X(8, 8) X(4, 4) X(8, 16) X(16, 16) X(16, 8) X(4, 16) X(8, 2)
+bool bwd_shape_built(int n1, int n2) {
+#define GELIB_X(A, B) if (n1 == A && n2 == B) return true;
+  GELIB_ONEPAIR_SHAPES(GELIB_X)
+#undef GELIB_X
+  return false;
+}
+void launch_bwd_shape(int n1, int n2, const OnePairMfmaArgs &a, hipStream_t s) {
+#define GELIB_X(A, B)                                                                                                   \
+  if (n1 == A && n2 == B)                                                                                               \
+    hipLaunchKernelGGL((onepair_mfma_bwd_kernel<A, B>), dim3((unsigned)a.ncells), dim3(64 * PairShape<A, B>::W), 0, s, a);
+  GELIB_ONEPAIR_SHAPES(GELIB_X)
+#undef GELIB_X
+}
+
+template <int N1, int N2, bool ONE_ROWB>
+int launch_fwd_one(const OnePairMfmaArgs &a, unsigned nblocks, size_t lds, hipStream_t s) {
+  static std::mutex attr_mutex;
+  static std::map<int, bool> attr_set;  // device -> the kernel may use 80 KB of LDS
+  int dev = 0;
+  GELIB_HIP_TRY(hipGetDevice(&dev));
+  {
+    std::lock_guard<std::mutex> lock(attr_mutex);
+    if (!attr_set[dev]) {
+      GELIB_HIP_TRY(hipFuncSetAttribute((const void *)onepair_mfma_fwd_kernel<N1, N2, ONE_ROWB>,
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)(80 * 1024)));
+      attr_set[dev] = true;
+    }
+  }
+  hipLaunchKernelGGL((onepair_mfma_fwd_kernel<N1, N2, ONE_ROWB>), dim3(nblocks), dim3(64 * kCellsF), lds, s, a);
+  return GELIB_HIP_OK;
+}
+int launch_fwd_shape(int n1, int n2, bool one_rowb, const OnePairMfmaArgs &a, unsigned nblocks, size_t lds, hipStream_t s) {
+#define GELIB_X(A, B)                                                                     \
+  if (n1 == A && n2 == B)                                                                 \
+    return one_rowb ? launch_fwd_one<A, B, true>(a, nblocks, lds, s) : launch_fwd_one<A, B, false>(a, nblocks, lds, s);
+  GELIB_ONEPAIR_SHAPES(GELIB_X)
+#undef GELIB_X
+  return GELIB_HIP_ERR_ARG;
+}
+
 }  // namespace
 
-// Both gradients of a non-Diag product of one x part with one y part, 8 x 8 channels, l1, l2 <= 15.  *used = 1 if
-// the launch was made; anything else is left to the other kernels.
+// Both gradients of a non-Diag product of one x part with one y part, l1, l2 <= 15, for the channel counts listed in
+// GELIB_ONEPAIR_SHAPES.  *used = 1 if the launch was made; anything else is left to the other kernels.
 int onepair_mfma_vec_bwd(const VecPlan &plan, const std::vector<const gelib_part_desc *> &g,
                          const std::vector<const gelib_part_desc *> &x, const std::vector<const gelib_part_desc *> &y,
                          const std::vector<const gelib_part_desc *> &xg, const std::vector<const gelib_part_desc *> &yg,
@@ -520,7 +647,7 @@ int onepair_mfma_vec_bwd(const VecPlan &plan, const std::vector<const gelib_part
       !lists_to_fast(yg, plan.E, true, &fyg, nullptr))
     return GELIB_HIP_OK;
   const int l1 = lx[0].first, l2 = ly[0].first, n1 = lx[0].second, n2 = ly[0].second;
-  if (n1 != 8 || n2 != 8 || l1 > kMaxLm || l2 > kMaxLm) return GELIB_HIP_OK;
+  if (!bwd_shape_built(n1, n2) || l1 > kMaxLm || l2 > kMaxLm) return GELIB_HIP_OK;
   const int lmin = std::abs(l1 - l2);
   int lmax = -1;
   for (auto &t : plan.triples) lmax = std::max(lmax, t.l);
@@ -538,8 +665,10 @@ int onepair_mfma_vec_bwd(const VecPlan &plan, const std::vector<const gelib_part
     a.g[dl] = fg[t.ri];
     a.offs[dl] = t.offs;
     present[dl] = 1;
-    // the lane's 16 bytes of a row must be 16-byte aligned: block offset, row and cell strides even
-    if (((t.offs) & 1) || (fg[t.ri].sm & 1) || (fg[t.ri].sb & 1) || ((uintptr_t)fg[t.ri].ptr & 15)) return GELIB_HIP_OK;
+    // 64 channels per wave: the lane's 16 bytes of a row must be 16-byte aligned (block offset, row and cell strides
+    // even); with 16 channels a lane loads single floats
+    if (n1 * n2 >= 64 && (((t.offs) & 1) || (fg[t.ri].sm & 1) || (fg[t.ri].sb & 1) || ((uintptr_t)fg[t.ri].ptr & 15)))
+      return GELIB_HIP_OK;
     if ((long long)fg[t.ri].sm * 8 * (2 * t.l + 1) >= (1LL << 32)) return GELIB_HIP_OK;  // row offsets are 32 bits
   }
   const long long ncells = plan.E[0] * plan.E[1] * plan.E[2];
@@ -559,13 +688,13 @@ int onepair_mfma_vec_bwd(const VecPlan &plan, const std::vector<const gelib_part
   a.lt = lt;
   a.nl = nl;
   a.accumulate = accumulate ? 1 : 0;
-  hipLaunchKernelGGL(onepair_mfma_bwd_kernel, dim3((unsigned)ncells), dim3(64), 0, s, a);
+  launch_bwd_shape(n1, n2, a, s);
   GELIB_HIP_TRY(hipGetLastError());
   *used = 1;
   return GELIB_HIP_OK;
 }
 
-// The product itself for the same shapes (non-Diag, 8 x 8 channels, l1, l2 <= 15, 4 to 22 values of l).
+// The product itself for the same shapes (non-Diag, l1, l2 <= 15, 4 to 22 values of l).
 int onepair_mfma_vec_fwd(const VecPlan &plan, const std::vector<const gelib_part_desc *> &r,
                          const std::vector<const gelib_part_desc *> &x, const std::vector<const gelib_part_desc *> &y,
                          bool accumulate, hipStream_t s, int *used) {
@@ -577,7 +706,7 @@ int onepair_mfma_vec_fwd(const VecPlan &plan, const std::vector<const gelib_part
       !lists_to_fast(r, plan.E, true, &fr, &lr))
     return GELIB_HIP_OK;
   const int l1 = lx[0].first, l2 = ly[0].first, n1 = lx[0].second, n2 = ly[0].second;
-  if (n1 != 8 || n2 != 8 || l1 > kMaxLm || l2 > kMaxLm) return GELIB_HIP_OK;
+  if (!bwd_shape_built(n1, n2) || l1 > kMaxLm || l2 > kMaxLm) return GELIB_HIP_OK;
   const int lmin = std::abs(l1 - l2);
   int lmax = -1;
   for (auto &t : plan.triples) lmax = std::max(lmax, t.l);
@@ -589,16 +718,19 @@ int onepair_mfma_vec_fwd(const VecPlan &plan, const std::vector<const gelib_part
   a.x = fx[0];
   a.y = fy[0];
   std::vector<int> present(nl, 0);
+  bool one_rowb = true;
   for (auto &t : plan.triples) {
     const int dl = t.l - lmin;
     a.g[dl] = fr[t.ri];
     a.offs[dl] = t.offs;
     present[dl] = 1;
-    // a lane stores 16 bytes at a time: block offset, row and cell strides even, base aligned
-    if (((t.offs) & 1) || (fr[t.ri].sm & 1) || (fr[t.ri].sb & 1) || ((uintptr_t)fr[t.ri].ptr & 15)) return GELIB_HIP_OK;
-    // one row length for every part (true whenever the parts hold just this pair's block)
+    // 64 channels per wave: a lane stores 16 bytes at a time (block offset, row and cell strides even, base aligned);
+    // with 16 channels it stores single floats
+    if (n1 * n2 >= 64 && (((t.offs) & 1) || (fr[t.ri].sm & 1) || (fr[t.ri].sb & 1) || ((uintptr_t)fr[t.ri].ptr & 15)))
+      return GELIB_HIP_OK;
+    if ((long long)fr[t.ri].sm * 8 >= (1LL << 32)) return GELIB_HIP_OK;  // row lengths are 32 bits
     if (a.rowb == 0) a.rowb = (long long)fr[t.ri].sm * 8;
-    if (a.rowb != (long long)fr[t.ri].sm * 8) return GELIB_HIP_OK;
+    if (a.rowb != (long long)fr[t.ri].sm * 8) one_rowb = false;
   }
   const long long ncells = plan.E[0] * plan.E[1] * plan.E[2];
   if (ncells > 0x7fffffffLL) return GELIB_HIP_OK;
@@ -615,22 +747,14 @@ int onepair_mfma_vec_fwd(const VecPlan &plan, const std::vector<const gelib_part
   a.lt = lt;
   a.nl = nl;
   a.accumulate = accumulate ? 1 : 0;
-  // LDS of a block: the table and eight cells' operands (with their rows of zeros); two blocks per compute unit fit
+  // LDS of a block: the table and its cells' operands (with their rows of zeros); two blocks per compute unit fit
   // up to 80 KB each, beyond that the any-l kernels take the pair
-  const size_t lds = (size_t)t.nsteps_fwd * 2 * kColsF * 4 + (size_t)kCellsF * (2 * l1 + 1 + 2 * l2 + 1 + 3) * 64;
+  const int cells_per_block = n1 * n2 >= 64 ? kCellsF * 64 / (n1 * n2) : kCellsF;
+  const size_t lds = (size_t)t.nsteps_fwd * 2 * kColsF * 4 +
+                     (size_t)cells_per_block * ((size_t)(2 * l1 + 2) * n1 + (size_t)(2 * l2 + 3) * n2) * 8;
   if (lds > 80 * 1024) return GELIB_HIP_OK;
-  {
-    static std::mutex attr_mutex;
-    static std::map<int, size_t> attr_set;  // device -> largest size asked for so far
-    int dev = 0;
-    GELIB_HIP_TRY(hipGetDevice(&dev));
-    std::lock_guard<std::mutex> lock(attr_mutex);
-    if (attr_set[dev] < lds) {
-      GELIB_HIP_TRY(hipFuncSetAttribute((const void *)onepair_mfma_fwd_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)(80 * 1024)));
-      attr_set[dev] = 80 * 1024;
-    }
-  }
-  hipLaunchKernelGGL(onepair_mfma_fwd_kernel, dim3((unsigned)((ncells + kCellsF - 1) / kCellsF)), dim3(64 * kCellsF), lds, s, a);
+  rc = launch_fwd_shape(n1, n2, one_rowb, a, (unsigned)((ncells + cells_per_block - 1) / cells_per_block), lds, s);
+  if (rc) return rc;
   GELIB_HIP_TRY(hipGetLastError());
   *used = 1;
   return GELIB_HIP_OK;

@@ -43,6 +43,18 @@ constexpr int steps_below(int l1, int l2, int ltop, int m) {
   for (int k = -ltop; k < m; k++) s += steps_of(l1, l2, k);
   return s;
 }
+// Step records: the coefficients of a step, one for every l of the pair that has a row m = m1 + m2 (l >= |m|, from lmin
+// up), the steps one after the other in the order the kernel takes them.  Position of the first coefficient of step k
+// of row number m:
+constexpr int rec_pos(int l1, int l2, int lmin, int ltop, int m, int k) {
+  int pos = 0;
+  for (int mm = -ltop; mm <= m; mm++) {
+    const int ma = mm < 0 ? -mm : mm;
+    const int nv = ltop - (lmin > ma ? lmin : ma) + 1;  // coefficients per step of this row number
+    pos += (mm < m ? steps_of(l1, l2, mm) : k) * nv;
+  }
+  return pos;
+}
 
 // All g, x, y pointers that the arithmetic loops dereference are typed as global memory, so the loads are
 // global_load (vmcnt only) rather than flat_load (which also ties up the LDS counter).
@@ -154,11 +166,13 @@ __device__ __forceinline__ void pair_bwd(const GParts<LCAP> &gp, PairPtr pr, Coe
     gsm[dl] = present ? G.sm : 0;
     cl[dl] = present ? Cs + p.cg[DL0 + dl] : Zc;
   });
-  constexpr int RECW = pow2ceil_(NLP);                 // floats per record
-  constexpr int kGroup = 16;                           // floats per load
-  constexpr int PER = kGroup / RECW;                   // steps per group
-  constexpr int NSTEPS = steps_below(L1, L2, LTOP, LTOP + 1);
-  constexpr int NGROUPS = (NSTEPS * RECW + kGroup - 1) / kGroup;
+  // Step records are fetched with scalar loads, kGroup floats at a time into one of two sets of scalar registers: the
+  // next group is on its way while the steps of this one run.  Scalar loads return in any order, so every wait for
+  // one is a wait for all: the fewer groups, the fewer waits (16 floats per group: 3.7 ms on the l <= 6 launch of
+  // L=6, 8 channels, 16384 cells; 32 floats: 2.9 ms).
+  constexpr int kGroup = 32;
+  constexpr int NREC = rec_pos(L1, L2, LMIN, LTOP, LTOP, steps_of(L1, L2, LTOP));  // floats of all steps
+  constexpr int NGROUPS = (NREC + kGroup - 1) / kGroup;
   const CoeffPtr recs = Cs - p.cg_base + (REC ? p.rec_off : 0);   // Cs is the bank plus cg_base
   float cb[2][kGroup];
   auto load_group = [&](auto gc, float(&dst)[kGroup]) __attribute__((always_inline)) {
@@ -208,21 +222,28 @@ __device__ __forceinline__ void pair_bwd(const GParts<LCAP> &gp, PairPtr pr, Coe
       constexpr int m1 = M1LO + decltype(kc)::value;
       constexpr int m2 = m - m1;
       float qr = 0.f, qi = 0.f;
-      constexpr int step = steps_below(L1, L2, LTOP, m) + decltype(kc)::value;
-      constexpr int grp = step / PER, slot = step % PER;
+      constexpr int kk = decltype(kc)::value;
+      constexpr int DLV = (LMIN > MABS ? LMIN : MABS) - LMIN;       // the first dl with a row m
+      constexpr int P0 = rec_pos(L1, L2, LMIN, LTOP, m, kk);         // the step's first coefficient
+      // the step before this one (none: -1)
+      constexpr int PPREV = (mi == 0 && kk == 0) ? -kGroup
+                            : (kk > 0 ? rec_pos(L1, L2, LMIN, LTOP, m, kk - 1)
+                                      : rec_pos(L1, L2, LMIN, LTOP, m - 1, steps_of(L1, L2, m - 1) - 1));
+      constexpr int grp = P0 / kGroup;
       static_for<NLP>([&](auto dl_c) __attribute__((always_inline)) {
         constexpr int dl = decltype(dl_c)::value;
         if constexpr (LMIN + dl >= MABS) {
           float c;
-          if constexpr (REC) c = cb[grp & 1][slot * RECW + dl];
+          if constexpr (REC) c = cb[((P0 + dl - DLV) / kGroup) & 1][(P0 + dl - DLV) % kGroup];
           else c = cl[dl][(m1 + L1) * (2 * L2 + 1) + (m2 + L2)];
           qr = fmaf(c, gl[dl].x, qr);
           qi = fmaf(c, gl[dl].y, qi);
         }
       });
-      if constexpr (REC && slot == 0 && grp + 1 < NGROUPS) {
-        // the next group is requested only after this one has been waited for: scalar loads return in any order, so
-        // a wait for one of them is a wait for all that are in flight
+      if constexpr (REC && grp != (PPREV < 0 ? -1 : PPREV / kGroup) && grp + 1 < NGROUPS) {
+        // The first step that starts in a group requests the next one, into the registers of the group before (whose
+        // last coefficient an earlier step has used: a step has at most 13 coefficients, a group 32), and only after
+        // its own coefficients have been waited for.
         __builtin_amdgcn_sched_barrier(0);
         load_group(std::integral_constant<int, grp + 1>{}, cb[(grp + 1) & 1]);
         __builtin_amdgcn_sched_barrier(0);

@@ -111,11 +111,12 @@ int ilog2(int v) {
 
 namespace {
 
-// Step records for the backward kernels: for every pair, one record per (m1,m2) step in the order the kernel runs
-// them (row number m = m1 + m2 rising from -ltop, m1 rising inside a row), holding C_l[m1,m2] for
-// l = max(|l1-l2|, lo) .. ltop = min(l1+l2, cap) -- zero where the part is absent or l < |m| -- padded to a power of two floats.
-// cap is the largest l the kernel that will run has code for (unrolled_bwd_cap).  A pair's records start on a 64-byte
-// boundary of the device allocation and are padded to whole 64-byte groups, the unit the kernel loads.
+// Step records for the backward kernels: for every pair, the coefficients of its (m1,m2) steps in the order the kernel
+// runs them (row number m = m1 + m2 rising from -ltop, m1 rising inside a row): C_l[m1,m2] for the l from
+// max(|l1-l2|, lo, |m|) to ltop = min(l1+l2, cap), zero where the part is absent (rec_pos in cg_unrolled_bwd_impl.h is
+// the same count on the device side).  cap is the largest l the kernel that will run has code for (unrolled_bwd_cap).
+// A pair's records start on a 64-byte boundary of the device allocation and are padded to whole groups of 32 floats,
+// the unit the kernel loads.
 void append_step_records(bool diag, int cap, int lo, size_t pair_bytes, std::vector<PairRec> *pairs, std::vector<float> *bank) {
   (void)diag;
   for (auto &p : *pairs) p.rec_off = -1;
@@ -126,20 +127,19 @@ void append_step_records(bool diag, int cap, int lo, size_t pair_bytes, std::vec
     const int dl0 = lmin - std::abs(p.l1 - p.l2);   // the pair's tables are indexed from |l1 - l2|
     if (lmin > ltop) continue;
     const int nl = ltop - lmin + 1, w2 = 2 * p.l2 + 1;
-    int recw = 1;
-    while (recw < nl) recw *= 2;
     p.rec_off = (int)bank->size();
+    // a step holds one coefficient for every l of the pair with a row m (l >= |m|), zero where the triple is absent
     for (int m = -ltop; m <= ltop; m++)
       for (int m1 = std::max(-p.l1, m - p.l2); m1 <= std::min(p.l1, m + p.l2); m1++) {
         const int m2 = m - m1;
-        for (int dl = 0; dl < recw; dl++) {
+        for (int dl = std::max(lmin, std::abs(m)) - lmin; dl < nl; dl++) {
           float c = 0.f;
-          if (dl < nl && dl0 + dl < kMaxDl && p.ri[dl0 + dl] >= 0 && lmin + dl >= std::abs(m))
+          if (dl0 + dl < kMaxDl && p.ri[dl0 + dl] >= 0)
             c = (*bank)[p.cg_base + p.cg[dl0 + dl] + (m1 + p.l1) * w2 + (m2 + p.l2)];
           bank->push_back(c);
         }
       }
-    while (bank->size() % 16) bank->push_back(0.f);
+    while (bank->size() % 32) bank->push_back(0.f);  // the kernel fetches whole groups of 32 floats
   }
 }
 

@@ -18,6 +18,12 @@
 // those loads in flight across the control flow between units, so it lost to the plain form.)
 #pragma once
 
+// 1: every kernel for whole pairs reads its coefficients as step records (below), not only those for operands above
+// kLT.  Measured on L=4, 16 channels, 32768 cells: backward 4.65 -> 4.4 ms capped at l = 4, 8.1 -> 7.3 ms uncapped.
+#ifndef GELIB_BWD_RECORDS_ALL
+#define GELIB_BWD_RECORDS_ALL 1
+#endif
+
 #include "cg_lane_sums.h"
 #include "cg_unrolled_dev.h"
 
@@ -440,7 +446,7 @@ unrolled_bwd_kernel(const BwdArgs a) {
         pair_bwd_one<A, B, LCAP, DIAG, WX, WY, PAD>(only_dl, gp, p, C, Zc, zrows, xs, ys, xacc, yacc, xsize, ysize,   \
                                                     cell0, offs_add, q);                                      \
       else                                                                                                    \
-        pair_bwd<A, B, LCAP, DIAG, WX, WY, PAD, (LT > kLT), -1, LLO>(gp, p, C, Zc, zrows, xs, ys, xacc, yacc, xsize,  \
+        pair_bwd<A, B, LCAP, DIAG, WX, WY, PAD, (LT > kLT || GELIB_BWD_RECORDS_ALL), -1, LLO>(gp, p, C, Zc, zrows, xs, ys, xacc, yacc, xsize,  \
                                                                        ysize, cell0, offs_add, q);            \
     }                                                                                                         \
     break;

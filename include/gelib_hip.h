@@ -301,8 +301,9 @@ int gelib_hip_set_stream_workspace(void *stream, void *ptr, uint64_t bytes);
  * "staged_bwd_lds_target", "staged_bwd_threads" (256, 512, 1024), "staged_bwd_stripes" (0 never, otherwise wherever they
  * apply), "staged_bwd_atomic" (1/0: allow the single-pass backward kernels that add with LDS float atomics; off by
  * default, so that results do not depend on timing), "staged_bwd_pairs" (1/0: the pair-wise one of those),
- * "pairwise_bwd" (one launch of the single-pair kernels per pair of parts: 0 never, 1 for operand l above 7, 2 wherever
- * every pair qualifies), "onepair_mfma" (1/0: the matrix-core form of the single-pair kernel), "onepair_mfma_fwd" (1/0:
+ * "pairwise_bwd" (one launch of the single-pair kernels per pair of parts, backward and -- for operand l above 7 --
+ * forward: 0 never, 1 for operand l above 7, 2 backward wherever every pair qualifies), "onepair_mfma" (1/0: the
+ * matrix-core form of the single-pair kernel, built for 4 x 4, 8 x 2, 8 x 8, 4 x 16, 8 x 16, 16 x 8 and 16 x 16 channels), "onepair_mfma_fwd" (1/0:
  * its forward kernel), "onepair_mfma_paired" (1/0: row numbers taken in pairs when l1 = l2), "unrolled_bwd_one" (1/0: the
  * backward kernel built for calls with one triple), "diag6_sets" (1/0: the Diag backward kernel with compile-time sets of
  * l2 per wave), "diag6_l8" (0: Diag products above l = 6 are always split at l = 6; 1: operands up to l = 4 run forward in

@@ -65,7 +65,8 @@ MFMA_SHAPES = {(8, 8), (4, 4), (8, 16), (16, 16), (16, 8), (4, 16), (8, 2)}
 @pytest.mark.parametrize("mfma", [1, 0])
 @pytest.mark.parametrize("B,l1,n1,l2,n2,maxl,diag", CASES)
 def test_onepair_bwd(cabi, B, l1, n1, l2, n2, maxl, diag, mfma):
-    """Both forms of the family: with the matrix-core kernel allowed (it takes the 8 x 8 cases) and without it."""
+    """Both forms of the family: with the matrix-core kernel allowed (it takes the channel counts in MFMA_SHAPES) and
+    without it."""
     if not mfma and ((n1, n2) != (8, 8) or diag):
         pytest.skip("the same kernel either way" if n1 * n2 <= 64 else "more than 64 channel slots: only the matrix-core kernel takes it")
     cabi.set_option("onepair_mfma", mfma)

@@ -156,6 +156,14 @@ __device__ __forceinline__ void pair_bwd(const GParts<LCAP> &gp, PairPtr pr, Coe
 #pragma unroll
     for (int m2 = 0; m2 <= 2 * L2; m2++) yv[m2] = yp[m2 * N2];
   }
+  if (PAD && !valid) {
+    // A lane beyond the real channels works on channel (0, 0) with operands of zero: whatever it reads of g (finite
+    // wherever that channel's own lane sees finite values), it adds zeros to the sums it shares.
+#pragma unroll
+    for (int m1 = 0; m1 <= 2 * L1; m1++) xv[m1] = make_float2(0.f, 0.f);
+#pragma unroll
+    for (int m2 = 0; m2 <= 2 * L2; m2++) yv[m2] = make_float2(0.f, 0.f);
+  }
 #pragma unroll
   for (int m1 = 0; m1 <= 2 * L1; m1++) ax[m1] = make_float2(0.f, 0.f);
 #pragma unroll
@@ -195,7 +203,7 @@ __device__ __forceinline__ void pair_bwd(const GParts<LCAP> &gp, PairPtr pr, Coe
       constexpr int L = LMIN + dl;
       if constexpr (L >= cabs_(m)) {
         const v2f t = gptr[dl][(m + L) * gsm[dl]];
-        dst[dl] = (PAD && !valid) ? make_float2(0.f, 0.f) : make_float2(t.x, t.y);
+        dst[dl] = make_float2(t.x, t.y);
       }
     });
   };

@@ -52,6 +52,10 @@ struct PairRec {
   int log2_u;        // log2 of the lane slots per cell: n1p*n2p (Diag: n1p) with n1p, n2p the channel counts rounded up
                      // to powers of two; -1 when that exceeds 2^20
   int lg_n2p;        // log2 of n2p
+  int rpc;           // runs of 64 lane slots per cell when a cell has 64 slots or more (else 0): n1p*n2p / 64, or
+                     // n1*n2p / 64 (Diag: n1 / 64) when that is whole -- the channels of the first operand need no
+                     // rounding up as long as a cell's slots fill whole runs
+  unsigned rpc_magic;  // ceil(2^32 / rpc) for rpc > 1 (run / rpc = the high half of run * rpc_magic), else 0
   int rec_off;       // offset (floats) in the bank of the pair's step records (kernel for operands up to l = kLTMax), or -1
   int cost_rank;     // position of the pair when the pairs are sorted by falling cost (backward launches that deal the
                      // pairs of a cell to several blocks take every S-th of that order)

@@ -87,11 +87,17 @@ struct LanePos {
   bool live;
 };
 
-__device__ __forceinline__ LanePos lane_pos(int run, int lane, int log2_u, int ncell) {
-  const int flat = (run << 6) + lane;
+// rpc > 0: a cell has rpc runs of 64 slots (not necessarily a power of two of them); otherwise 2^log2_u < 64 slots.
+__device__ __forceinline__ LanePos lane_pos(int run, int lane, int log2_u, int rpc, unsigned rpc_magic, int ncell) {
   LanePos q;
-  q.cell_local = flat >> log2_u;
-  q.u = flat & ((1 << log2_u) - 1);
+  if (rpc > 0) {  // uniform
+    q.cell_local = rpc > 1 ? (int)__umulhi((unsigned)run, rpc_magic) : run;
+    q.u = ((run - q.cell_local * rpc) << 6) + lane;
+  } else {
+    const int flat = (run << 6) + lane;
+    q.cell_local = flat >> log2_u;
+    q.u = flat & ((1 << log2_u) - 1);
+  }
   q.live = q.cell_local < ncell;
   if (!q.live) q.cell_local = ncell - 1;  // dead lanes read valid memory and never store
   return q;
@@ -430,7 +436,7 @@ unrolled_bwd_kernel(const BwdArgs a) {
   const PairPtr pairs = (PairPtr)a.pairs;
   const int npairs = a.npairs, offs_add = a.offs_add, only_dl = a.only_dl;
   (void)only_dl;
-  auto runs_of = [&](int k) { return ((cpb << pairs[k].log2_u) + kWave - 1) >> 6; };
+  auto runs_of = [&](int k) { return pairs[k].rpc > 0 ? cpb * pairs[k].rpc : ((cpb << pairs[k].log2_u) + kWave - 1) >> 6; };
   GParts<LCAP> gp;
   static_for<LCAP + 1>([&](auto l) __attribute__((always_inline)) { gp.G[l.value] = a.g[l.value]; });
   const CoeffPtr Zc = (CoeffPtr)(a.bank + a.zero_off);    // a table of zeros and ...
@@ -445,7 +451,7 @@ unrolled_bwd_kernel(const BwdArgs a) {
     const int first = (wave - dealt) & (kWaves - 1);
     dealt += nruns;
     for (int run = first; run < nruns; run += kWaves) {
-      const LanePos q = lane_pos(run, lane, p->log2_u, ncell);
+      const LanePos q = lane_pos(run, lane, p->log2_u, p->rpc, p->rpc_magic, ncell);
       switch (p->l1 * (kLTMax + 1) + p->l2) {
 #define GELIB_CASE(A, B)                                                                                      \
   case A * (kLTMax + 1) + B:                                                                                  \

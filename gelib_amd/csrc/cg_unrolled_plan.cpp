@@ -194,6 +194,13 @@ int get_plan(bool diag, const std::vector<VecTriple> &triples, const std::vector
         const int lgu = diag ? lg1 : lg1 + lg2;
         rec.lg_n2p = lg2;
         rec.log2_u = lgu <= 20 ? lgu : -1;
+        rec.rpc = 0;
+        rec.rpc_magic = 0;
+        if (lgu >= 6 && lgu <= 20) {
+          const long long pow2_slots = 1LL << lgu, tight = (long long)rec.n1 * (diag ? 1 : (1LL << lg2));
+          rec.rpc = (int)((tight % 64 == 0 ? tight : pow2_slots) / 64);
+          if (rec.rpc > 1) rec.rpc_magic = (unsigned)(((1ULL << 32) + rec.rpc - 1) / rec.rpc);
+        }
         if (!is_pow2(rec.n1) || (!diag && !is_pow2(rec.n2))) plan.padded = true;
       }
       rec.xoff = xoff[t.xi];
@@ -416,7 +423,7 @@ int run_bwd(bool diag, const std::vector<VecTriple> &triples, const std::vector<
   const size_t lds_target = lop > kLT ? 52 * 1024 : (size_t)g_bwd_lds_target;
   auto runs_at = [&](int c) {
     long long runs = 0;
-    for (auto &p : plan->pairs) runs += (((long long)c << p.log2_u) + kWave - 1) / kWave;
+    for (auto &p : plan->pairs) runs += p.rpc > 0 ? (long long)c * p.rpc : (((long long)c << p.log2_u) + kWave - 1) / kWave;
     return runs;
   };
   // few runs per cell (few pairs, few channels): more cells per block, so that the staging of the operands, the two

@@ -175,6 +175,10 @@ def test_parts_in_any_order(cabi):
     (33, {l: 12 for l in range(5)}, {l: 12 for l in range(5)}, 4),
     (70, {1: 1, 3: 3}, {2: 5}, 4),                           # 5 and 15 lane slots per cell: many cells per run
     (3, {2: 24}, {3: 40}, -1),                               # 24 x 40 channels: several runs per cell, n2 padded to 64
+    # the first operand's channels are not rounded up where a cell's lane slots still fill whole runs of 64
+    (5, {0: 3, 2: 3}, {1: 64, 2: 32}, -1),                   # 3 x 64 slots: three runs; 3 x 32: rounded up to 4 x 32
+    (4, {1: 20, 3: 12}, {0: 24, 2: 16}, 4),                  # 20 x 32, 12 x 32, 20 x 16, 12 x 16 slots
+    (2, {0: 192, 1: 192}, {0: 192, 1: 192}, -1),             # Diag: 192 channels, three runs per cell (CGproduct: 192 x 256)
 ])
 @pytest.mark.parametrize("diag", [False, True])
 def test_channel_counts_that_are_not_powers_of_two(cabi, case, diag):

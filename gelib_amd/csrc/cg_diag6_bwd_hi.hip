@@ -1,0 +1,9 @@
+// Instantiation of the lane-per-channel Diag backward kernel for the part of a product above l = 6: operand parts up to
+// l = 6, gradient parts l = 7..12, adding onto what the launch for l <= 6 (cg_diag6_bwd.hip) wrote.
+#include "cg_diag6_impl.h"
+
+namespace gelib_hip {
+
+int launch_diag6_bwd_hi(const Diag6Args &a, hipStream_t s) { return launch_diag6_bwd_variant<2 * kL6, false, kL6, kL6 + 1>(a, s); }
+
+}  // namespace gelib_hip

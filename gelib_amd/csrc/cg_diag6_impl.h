@@ -108,12 +108,13 @@ __device__ __forceinline__ void load_rows(float2 (&v)[2 * L + 1], const FastPart
   }
 }
 
-template <int L1, int L2, int LCAP, bool PACKED>
+// LLO: the launch takes only the l from LLO up (the part of a product above l = 6 is a launch of its own).
+template <int L1, int L2, int LCAP, bool PACKED, int LLO = 0>
 __device__ __forceinline__ void fwd_pair(const Diag6Args &a, const float2 (&xv)[2 * L1 + 1],
                                          const float2 (&yv)[2 * L2 + 1], const WavePos q) {
-  constexpr int LMIN = iabs(L1 - L2);
+  constexpr int LMIN = imax(iabs(L1 - L2), LLO);
   constexpr int LTOP = imin(L1 + L2, LCAP);
-  if constexpr (LMIN <= LCAP) {
+  if constexpr (LMIN <= LTOP) {
     constexpr int NL = LTOP - LMIN + 1;
     const OffsPtr offs = (OffsPtr)a.offs + (L1 * kNP + L2) * kNR;
     const CoeffPtr C = (CoeffPtr)a.bank;
@@ -203,7 +204,7 @@ __device__ __forceinline__ void read_rows(float2 (&v)[2 * L + 1], const float2 *
 // leave room for three blocks per compute unit instead of five, and the store stream needs the waves (measured on
 // L = 6, 64 channels, 131072 cells: no image 18.2 - 20.2 ms, y alone 16.6 - 17.4 ms, both 29.7 ms).
 // LOP: the largest l of an operand part the kernel has code for.
-template <int LCAP, bool PACKED, int LOP>
+template <int LCAP, bool PACKED, int LOP, int LLO = 0>
 __global__ void __launch_bounds__(256) diag6_fwd_kernel(const Diag6Args a) {
   __shared__ float2 yimg[(LOP + 1) * (LOP + 1) * 64];
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
@@ -213,29 +214,33 @@ __global__ void __launch_bounds__(256) diag6_fwd_kernel(const Diag6Args a) {
   __syncthreads();
   static_for<LOP + 1>([&](auto l1c) __attribute__((always_inline)) {
     constexpr int L1 = decltype(l1c)::value;
-    if (a.x[L1].ptr != nullptr) {
-      float2 xv[2 * L1 + 1];
-      load_rows<L1, PACKED>(xv, a.x[L1], q, a.xbc != 0);
-      static_for<LOP + 1>([&](auto l2c) __attribute__((always_inline)) {
-        constexpr int L2 = decltype(l2c)::value;
-        if (((L1 * kNP + L2) & 3) == wave && a.y[L2].ptr != nullptr) {
-          float2 yv[2 * L2 + 1];
-          read_rows<L2>(yv, yimg, lane);
-          fwd_pair<L1, L2, LCAP, PACKED>(a, xv, yv, q);
-        }
-      });
+    if constexpr (L1 + LOP >= LLO) {  // some pair of this l1 reaches an l the launch takes
+      if (a.x[L1].ptr != nullptr) {
+        float2 xv[2 * L1 + 1];
+        load_rows<L1, PACKED>(xv, a.x[L1], q, a.xbc != 0);
+        static_for<LOP + 1>([&](auto l2c) __attribute__((always_inline)) {
+          constexpr int L2 = decltype(l2c)::value;
+          if constexpr (L1 + L2 >= LLO) {
+            if (((L1 * kNP + L2) & 3) == wave && a.y[L2].ptr != nullptr) {
+              float2 yv[2 * L2 + 1];
+              read_rows<L2>(yv, yimg, lane);
+              fwd_pair<L1, L2, LCAP, PACKED, LLO>(a, xv, yv, q);
+            }
+          }
+        });
+      }
     }
   });
 }
 
 // One pair of the backward pass: every l of the pair together, one row number m = m1 + m2 at a time.
-template <int L1, int L2, int LCAP, bool PACKED>
+template <int L1, int L2, int LCAP, bool PACKED, int LLO = 0>
 __device__ __forceinline__ void bwd_pair(const Diag6Args &a, const float2 (&xv)[2 * L1 + 1],
                                          const float2 (&yv)[2 * L2 + 1], float2 (&ax)[2 * L1 + 1], float2 *yimg,
                                          const WavePos q) {
-  constexpr int LMIN = iabs(L1 - L2);
+  constexpr int LMIN = imax(iabs(L1 - L2), LLO);
   constexpr int LTOP = imin(L1 + L2, LCAP);
-  if constexpr (LMIN <= LCAP) {
+  if constexpr (LMIN <= LTOP) {
     constexpr int NL = LTOP - LMIN + 1;
     constexpr int ROWS = (LTOP + 1) * (LTOP + 1) - LMIN * LMIN;
     constexpr int kBudget = PACKED ? kRowBudgetPacked : kRowBudget;
@@ -359,7 +364,7 @@ __device__ __forceinline__ void store_rows(const float2 *v, int vstride, const F
 // Three waves per SIMD (168 registers) is what the LDS of a block lets a compute unit hold; both forms fit by
 // themselves (the packed one with a smaller row budget).  Forcing the limit with amdgpu_waves_per_eu instead changed the
 // schedule for the worse (twice as many waits).
-template <int LCAP, bool PACKED, int LOP>
+template <int LCAP, bool PACKED, int LOP, int LLO = 0>
 __global__ void __launch_bounds__(256) diag6_bwd_kernel(const Diag6Args a) {
   constexpr int kXRows = 2 * LOP + 1;
   constexpr int kYRows = (LOP + 1) * (LOP + 1);
@@ -374,6 +379,7 @@ __global__ void __launch_bounds__(256) diag6_bwd_kernel(const Diag6Args a) {
   __syncthreads();
   static_for<LOP + 1>([&](auto l1c) __attribute__((always_inline)) {
     constexpr int L1 = decltype(l1c)::value;
+    if constexpr (L1 + LOP < LLO) return;  // no pair of this l1 reaches an l the launch takes
     if (a.x[L1].ptr != nullptr) {  // the same for the whole block
       // x is needed for the y-gradient only and y for the x-gradient only; an operand whose gradient is not wanted is
       // never read (a part-level call for one gradient does not even have it) and enters as zeros
@@ -388,15 +394,17 @@ __global__ void __launch_bounds__(256) diag6_bwd_kernel(const Diag6Args a) {
       for (int m1 = 0; m1 <= 2 * L1; m1++) ax[m1] = make_float2(0.f, 0.f);
       static_for<LOP + 1>([&](auto l2c) __attribute__((always_inline)) {
         constexpr int L2 = LOP - decltype(l2c)::value;  // descending, so that neighbours in l2 run at the same time
-        if (a.owner[L2] == wave && a.y[L2].ptr != nullptr) {
-          float2 yv[2 * L2 + 1];
-          if (wx) {
-            load_rows<L2, PACKED>(yv, a.y[L2], q, a.ybc != 0);
-          } else {
+        if constexpr (L1 + L2 >= LLO) {
+          if (a.owner[L2] == wave && a.y[L2].ptr != nullptr) {
+            float2 yv[2 * L2 + 1];
+            if (wx) {
+              load_rows<L2, PACKED>(yv, a.y[L2], q, a.ybc != 0);
+            } else {
 #pragma unroll
-            for (int m2 = 0; m2 <= 2 * L2; m2++) yv[m2] = make_float2(0.f, 0.f);
+              for (int m2 = 0; m2 <= 2 * L2; m2++) yv[m2] = make_float2(0.f, 0.f);
+            }
+            bwd_pair<L1, L2, LCAP, PACKED, LLO>(a, xv, yv, ax, yimg, q);
           }
-          bwd_pair<L1, L2, LCAP, PACKED>(a, xv, yv, ax, yimg, q);
         }
       });
       if (!wx) return;  // continues with the next l1 (this is the body of a per-l1 lambda); uniform for the block
@@ -435,8 +443,10 @@ __global__ void __launch_bounds__(256) diag6_bwd_kernel(const Diag6Args a) {
   static_for<LOP + 1>([&](auto l2c) __attribute__((always_inline)) {
     constexpr int L2 = decltype(l2c)::value;
     const FastPart YG = a.yg[L2];
-    if (wy && a.owner[L2] == wave && YG.ptr != nullptr)
-      store_rows<L2, PACKED>(yimg + (L2 * L2) * 64 + lane, 64, YG, q, accumulate, a.ybc != 0, a.lg_npad);
+    if constexpr (L2 + LOP >= LLO) {
+      if (wy && a.owner[L2] == wave && YG.ptr != nullptr)
+        store_rows<L2, PACKED>(yimg + (L2 * L2) * 64 + lane, 64, YG, q, accumulate, a.ybc != 0, a.lg_npad);
+    }
   });
 }
 
@@ -541,16 +551,16 @@ int launch_diag6_bwd_sets_variant(const Diag6Args &a, hipStream_t s) {
   return GELIB_HIP_OK;
 }
 
-template <int LCAP, bool PACKED, int LOP = kL6>
+template <int LCAP, bool PACKED, int LOP = kL6, int LLO = 0>
 int launch_diag6_fwd_variant(const Diag6Args &a, hipStream_t s) {
-  hipLaunchKernelGGL((diag6_fwd_kernel<LCAP, PACKED, LOP>), dim3((unsigned)a.nwaves), dim3(256), 0, s, a);
+  hipLaunchKernelGGL((diag6_fwd_kernel<LCAP, PACKED, LOP, LLO>), dim3((unsigned)a.nwaves), dim3(256), 0, s, a);
   GELIB_HIP_TRY(hipGetLastError());
   return GELIB_HIP_OK;
 }
 
-template <int LCAP, bool PACKED, int LOP = kL6>
+template <int LCAP, bool PACKED, int LOP = kL6, int LLO = 0>
 int launch_diag6_bwd_variant(const Diag6Args &a, hipStream_t s) {
-  hipLaunchKernelGGL((diag6_bwd_kernel<LCAP, PACKED, LOP>), dim3((unsigned)a.nwaves), dim3(256), 0, s, a);
+  hipLaunchKernelGGL((diag6_bwd_kernel<LCAP, PACKED, LOP, LLO>), dim3((unsigned)a.nwaves), dim3(256), 0, s, a);
   GELIB_HIP_TRY(hipGetLastError());
   return GELIB_HIP_OK;
 }

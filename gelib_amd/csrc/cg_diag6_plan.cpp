@@ -20,6 +20,7 @@ std::map<std::pair<int, std::vector<int>>, int *> g_offs;  // (device, offsets) 
 int g_enable = 1;
 int g_l8_enable = 1;    // the kernels for products up to l = 8 of operands up to l = 4: 1 forward, 2 backward too
 int g_sets_enable = 1;  // backward: the kernel with the waves' sets of l2 fixed at compile time, where it applies
+int g_hi_enable = 1;    // the kernels for the part l = 7..12 of a product by itself
 int g_one_channel = 1;  // CGproduct with a one-channel operand runs here as the Diag product with the channel repeated
 
 int device_bank(const float **out) {
@@ -61,7 +62,7 @@ int device_offs(const std::vector<int> &h, const int **out) {
 int make_args(const VecPlan &plan, const std::vector<const gelib_part_desc *> &r,
               const std::vector<const gelib_part_desc *> &x, const std::vector<const gelib_part_desc *> &y,
               const std::vector<const gelib_part_desc *> *xg, const std::vector<const gelib_part_desc *> *yg,
-              bool r_is_dest, Diag6Args *a, int *lcap, bool *ok) {
+              bool r_is_dest, Diag6Args *a, int *lcap, bool *ok, int *llo = nullptr) {
   *ok = false;
   if (!g_enable) return GELIB_HIP_OK;
   std::vector<FastPart> fx, fy, fr, fxg, fyg;
@@ -133,10 +134,13 @@ int make_args(const VecPlan &plan, const std::vector<const gelib_part_desc *> &r
   }
   std::vector<int> offs((size_t)kNP * kNP * kNR, -1);
   *lcap = 0;
+  int lowest = 1 << 30;
   for (auto &t : plan.triples) {
     offs[((size_t)t.l1 * kNP + t.l2) * kNR + t.l] = t.offs;
     *lcap = std::max(*lcap, t.l);
+    lowest = std::min(lowest, t.l);
   }
+  if (llo) *llo = lowest;
   int rc = device_offs(offs, &a->offs);
   if (rc) return rc;
   if ((rc = device_bank(&a->bank))) return rc;
@@ -186,15 +190,18 @@ int diag6_vec_fwd(const VecPlan &plan, const std::vector<const gelib_part_desc *
                   bool accumulate, hipStream_t s, int *used) {
   *used = 0;
   Diag6Args a;
-  int lcap = 0;
+  int lcap = 0, llo = 0;
   bool ok = false;
-  int rc = make_args(plan, r, x, y, nullptr, nullptr, true, &a, &lcap, &ok);
+  int rc = make_args(plan, r, x, y, nullptr, nullptr, true, &a, &lcap, &ok, &llo);
   if (rc || !ok) return rc;
-  // kernels are built for products capped at l = 6, and for products up to l = 8 of operands up to l = 4
-  const bool l8 = lcap > kL6;
+  // kernels are built for products capped at l = 6, for products up to l = 8 of operands up to l = 4, and for the part
+  // l = 7..12 of a product by itself
+  const bool hi = llo > kL6 && g_hi_enable;
+  const bool l8 = lcap > kL6 && !hi;
   if (l8 && !(lcap <= 8 && operands_up_to(a, 4) && g_l8_enable)) return GELIB_HIP_OK;
   a.accumulate = accumulate ? 1 : 0;
-  if (l8) rc = a.lg_npad < 6 ? launch_diag6_fwd_l8_packed(a, s) : launch_diag6_fwd_l8(a, s);
+  if (hi) rc = a.lg_npad < 6 ? launch_diag6_fwd_hi_packed(a, s) : launch_diag6_fwd_hi(a, s);
+  else if (l8) rc = a.lg_npad < 6 ? launch_diag6_fwd_l8_packed(a, s) : launch_diag6_fwd_l8(a, s);
   else rc = a.lg_npad < 6 ? launch_diag6_fwd_l6_packed(a, s) : launch_diag6_fwd_l6(a, s);
   if (rc) return rc;
   *used = 1;
@@ -208,21 +215,23 @@ int diag6_vec_bwd(const VecPlan &plan, const std::vector<const gelib_part_desc *
   *used = 0;
   if (xg.empty() && yg.empty()) return GELIB_HIP_OK;
   Diag6Args a;
-  int lcap = 0;
+  int lcap = 0, llo = 0;
   bool ok = false;
-  int rc = make_args(plan, g, x, y, xg.empty() ? nullptr : &xg, yg.empty() ? nullptr : &yg, false, &a, &lcap, &ok);
+  int rc = make_args(plan, g, x, y, xg.empty() ? nullptr : &xg, yg.empty() ? nullptr : &yg, false, &a, &lcap, &ok, &llo);
   if (rc || !ok) return rc;
   // (backward, the one-launch kernel for products up to l = 8 is used on request only, diag6_l8 = 2: the wave that owns
   // y[4] then has the terms of l = 5..8 on top of the largest share, and L=4, 64 channels, 131072 cells takes 16.4 ms
   // against 14.4 ms for the split at l = 6)
-  const bool l8 = lcap > kL6;
+  const bool hi = llo > kL6 && g_hi_enable;
+  const bool l8 = lcap > kL6 && !hi;
   if (l8 && !(lcap <= 8 && operands_up_to(a, 4) && g_l8_enable >= 2)) return GELIB_HIP_OK;
   a.accumulate = accumulate ? 1 : 0;
   a.want_x = xg.empty() ? 0 : 1;
   a.want_y = yg.empty() ? 0 : 1;
   bool all_y = true;
   for (int l = 0; l < kNP; l++) all_y = all_y && a.y[l].ptr != nullptr;
-  if (l8) rc = a.lg_npad < 6 ? launch_diag6_bwd_l8_packed(a, s) : launch_diag6_bwd_l8(a, s);
+  if (hi) rc = a.lg_npad < 6 ? launch_diag6_bwd_hi_packed(a, s) : launch_diag6_bwd_hi(a, s);
+  else if (l8) rc = a.lg_npad < 6 ? launch_diag6_bwd_l8_packed(a, s) : launch_diag6_bwd_l8(a, s);
   else if (a.lg_npad < 6) rc = launch_diag6_bwd_l6_packed(a, s);
   else if (all_y && g_sets_enable) rc = launch_diag6_bwd_l6_sets(a, s);
   else rc = launch_diag6_bwd_l6(a, s);
@@ -257,6 +266,10 @@ int diag6_part(int kind, const long long E[3], const gelib_part_desc *r, const g
 int diag6_set_option(const char *name, int value) {
   if (!std::strcmp(name, "diag6")) {
     g_enable = value;
+    return GELIB_HIP_OK;
+  }
+  if (!std::strcmp(name, "diag6_hi")) {
+    g_hi_enable = value;
     return GELIB_HIP_OK;
   }
   if (!std::strcmp(name, "diag6_l8")) {

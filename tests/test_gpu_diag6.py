@@ -122,18 +122,22 @@ def test_diag6_declines_what_it_cannot_do(cabi):
 @pytest.mark.parametrize("l8", [1, 2, 0])
 @pytest.mark.parametrize("B,tau,maxl", [(5, {l: 64 for l in range(5)}, -1), (3, {l: 16 for l in range(7)}, -1),
                                         (4, {2: 40, 6: 40}, 9), (6, {l: 16 for l in range(5)}, -1),
-                                        (3, {1: 96, 4: 96}, 7), (70, {3: 5, 4: 5}, -1)])
+                                        (3, {1: 96, 4: 96}, 7), (70, {3: 5, 4: 5}, -1),
+                                        (2, {l: 64 for l in range(7)}, -1), (3, {3: 70, 5: 70, 6: 70}, -1)])
 def test_diag_product_above_l6(cabi, B, tau, maxl, l8):
     """A Diag product whose l reaches above 6.  Operands up to l = 4 (product up to l = 8): one launch of the
     lane-per-channel kernels built for that case (forward with l8 = 1, backward too with l8 = 2).  Otherwise, or with those
     kernels switched off: the triples
-    up to l = 6 run on the lane-per-channel kernels, the rest on the other families, the gradients of the second part
-    added on top of the first."""
+    up to l = 6 run on the lane-per-channel kernels, the rest (l = 7..12) on a second launch of that family built for those
+    l (l8 = 0 here also switches that launch off) or on the other families, the gradients of the
+    second part added on top of the first."""
     cabi.set_option("diag6_l8", l8)
+    cabi.set_option("diag6_hi", 1 if l8 else 0)
     try:
         _above_l6(cabi, B, tau, maxl)
     finally:
         cabi.set_option("diag6_l8", 1)
+        cabi.set_option("diag6_hi", 1)
 
 
 def _above_l6(cabi, B, tau, maxl):

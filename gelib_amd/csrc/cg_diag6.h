@@ -61,6 +61,9 @@ struct Diag6Args {
 int launch_diag6_fwd_l6(const Diag6Args &a, hipStream_t s);  // product l up to 6
 int launch_diag6_bwd_l6(const Diag6Args &a, hipStream_t s);
 int launch_diag6_bwd_l6_sets(const Diag6Args &a, hipStream_t s);  // every part of y present: fixed sets of l2 per wave
+// operand parts up to l = 4, product up to l = 6 (backward)
+int launch_diag6_bwd_l6_lop4(const Diag6Args &a, hipStream_t s);
+int launch_diag6_bwd_l6_lop4_packed(const Diag6Args &a, hipStream_t s);
 // product parts l = 7..12 only
 int launch_diag6_fwd_hi(const Diag6Args &a, hipStream_t s);
 int launch_diag6_bwd_hi(const Diag6Args &a, hipStream_t s);

@@ -20,6 +20,7 @@ std::map<std::pair<int, std::vector<int>>, int *> g_offs;  // (device, offsets) 
 int g_enable = 1;
 int g_l8_enable = 1;    // the kernels for products up to l = 8 of operands up to l = 4: 1 forward, 2 backward too
 int g_sets_enable = 1;  // backward: the kernel with the waves' sets of l2 fixed at compile time, where it applies
+int g_lop4_enable = 1;  // backward: the kernels built for operands up to l = 4 (smaller images in LDS)
 int g_hi_enable = 1;    // the kernels for the part l = 7..12 of a product by itself
 int g_one_channel = 1;  // CGproduct with a one-channel operand runs here as the Diag product with the channel repeated
 
@@ -232,6 +233,7 @@ int diag6_vec_bwd(const VecPlan &plan, const std::vector<const gelib_part_desc *
   for (int l = 0; l < kNP; l++) all_y = all_y && a.y[l].ptr != nullptr;
   if (hi) rc = a.lg_npad < 6 ? launch_diag6_bwd_hi_packed(a, s) : launch_diag6_bwd_hi(a, s);
   else if (l8) rc = a.lg_npad < 6 ? launch_diag6_bwd_l8_packed(a, s) : launch_diag6_bwd_l8(a, s);
+  else if (g_lop4_enable && operands_up_to(a, 4)) rc = a.lg_npad < 6 ? launch_diag6_bwd_l6_lop4_packed(a, s) : launch_diag6_bwd_l6_lop4(a, s);
   else if (a.lg_npad < 6) rc = launch_diag6_bwd_l6_packed(a, s);
   else if (all_y && g_sets_enable) rc = launch_diag6_bwd_l6_sets(a, s);
   else rc = launch_diag6_bwd_l6(a, s);
@@ -266,6 +268,10 @@ int diag6_part(int kind, const long long E[3], const gelib_part_desc *r, const g
 int diag6_set_option(const char *name, int value) {
   if (!std::strcmp(name, "diag6")) {
     g_enable = value;
+    return GELIB_HIP_OK;
+  }
+  if (!std::strcmp(name, "diag6_lop4")) {
+    g_lop4_enable = value;
     return GELIB_HIP_OK;
   }
   if (!std::strcmp(name, "diag6_hi")) {

@@ -308,7 +308,8 @@ int gelib_hip_set_stream_workspace(void *stream, void *ptr, uint64_t bytes);
  * backward kernel built for calls with one triple), "diag6_sets" (1/0: the Diag backward kernel with compile-time sets of
  * l2 per wave), "diag6_l8" (0: Diag products above l = 6 are always split at l = 6; 1: operands up to l = 4 run forward in
  * one launch of the kernels built for products up to l = 8; 2: backward too), "diag6_hi" (1/0: the part l = 7..12 of a
- * split Diag product runs on the lane-per-channel kernels built for it), "fwd_narrow_decline" (1/0: products with
+ * split Diag product runs on the lane-per-channel kernels built for it), "diag6_lop4" (1/0: Diag backward kernels built
+ * for operands up to l = 4), "fwd_narrow_decline" (1/0: products with
  * at most four channel pairs per block go forward on the any-l kernels).  Unknown names return
  * GELIB_HIP_ERR_ARG.  Options are process-wide.
  * gelib_hip_last_path() tells which kernel family the last call of this thread used

@@ -309,7 +309,13 @@ int gelib_hip_set_stream_workspace(void *stream, void *ptr, uint64_t bytes);
  * l2 per wave), "diag6_l8" (0: Diag products above l = 6 are always split at l = 6; 1: operands up to l = 4 run forward in
  * one launch of the kernels built for products up to l = 8; 2: backward too), "diag6_hi" (1/0: the part l = 7..12 of a
  * split Diag product runs on the lane-per-channel kernels built for it), "diag6_lop4" (1/0: Diag backward kernels built
- * for operands up to l = 4), "fwd_narrow_decline" (1/0: products with
+ * for operands up to l = 4), "diag6_one_channel" (1/0: a CGproduct in which every part of exactly one operand has one
+ * channel runs on the lane-per-channel Diag kernels), "unrolled_bwd_one_wide" (1/0: the wave-per-cell backward kernel
+ * for calls with one triple and 16 or 32 channels in the second operand) and "unrolled_bwd_one_wide_cells" (cells from
+ * which it is used, 4096), "unrolled_bwd_split" (1/0: launches with few cells deal a cell's pairs to several blocks),
+ * "unrolled_bwd_split_below" (blocks below which they do, 1024) and "unrolled_bwd_split_max" (blocks per cell at most,
+ * 16), "unrolled_bwd_l6_split" (1/0: a product above l = 6 of operands above l = 4 goes backward in two launches of the
+ * unrolled kernels, l <= 6 and l = 7..12), "fwd_narrow_decline" (1/0: products with
  * at most four channel pairs per block go forward on the any-l kernels).  Unknown names return
  * GELIB_HIP_ERR_ARG.  Options are process-wide.
  * gelib_hip_last_path() tells which kernel family the last call of this thread used

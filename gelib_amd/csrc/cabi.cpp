@@ -483,14 +483,16 @@ PartOp triple_op(const VecPlan &plan, const VecTriple &t, const std::vector<View
 bool split_at_l6(const VecPlan &plan, const std::vector<View> &R, VecPlan &A, VecPlan &B, std::vector<View> &RA,
                  std::vector<View> &RB);
 bool split_diag(const VecPlan &plan, const std::vector<View> &R, const std::vector<View> &X, const std::vector<View> &Y,
-                VecPlan &A, VecPlan &B, std::vector<View> &RA, std::vector<View> &RB) {
+                VecPlan &A, VecPlan &B, std::vector<View> &RA, std::vector<View> &RB, bool forward = false) {
   if (!plan.diag) {
     auto all_one = [](const std::vector<View> &v) {
       for (auto &p : v)
         if (p.n != 1) return false;
       return true;
     };
-    if (all_one(X) == all_one(Y)) return false;   // exactly one narrow side
+    const bool nx = all_one(X), ny = all_one(Y);
+    // exactly one narrow side; forward also one channel on both sides (the Diag product of one channel)
+    if (nx == ny && !(forward && nx)) return false;
   }
   return split_at_l6(plan, R, A, B, RA, RB);
 }
@@ -644,7 +646,7 @@ int vec_fwd_entry(bool diag, int nr, const gelib_part_desc *r, int nx, const gel
   if (!g_force_generic) {
     VecPlan A, B;
     std::vector<View> RA, RB;
-    if (split_diag(plan, R, X, Y, A, B, RA, RB)) {
+    if (split_diag(plan, R, X, Y, A, B, RA, RB, true)) {
       std::vector<const gelib_part_desc *> rd, xd, yd;
       for (auto &v : RA) rd.push_back(v.d);
       for (auto &v : X) xd.push_back(v.d);

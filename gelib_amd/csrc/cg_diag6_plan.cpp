@@ -87,7 +87,13 @@ int make_args(const VecPlan &plan, const std::vector<const gelib_part_desc *> &r
     };
     ybc = all_one(ly);
     xbc = all_one(lx);
-    if (xbc == ybc) return GELIB_HIP_OK;   // exactly one narrow side (one channel on both sides stays where it was)
+    if (xbc && ybc && !xg && !yg) {
+      // one channel on both sides, forward: block channel 0 * 1 + 0 -- the Diag product of one channel, a cell per lane
+      // (the gradients of such a product stay with the unrolled kernels, which are faster there)
+      xbc = ybc = false;
+    } else if (xbc == ybc) {
+      return GELIB_HIP_OK;   // otherwise exactly one narrow side
+    }
   }
   const int n = (xbc ? ly : lx)[0].second;
   if (n < 1 || n > kMaxChannels) return GELIB_HIP_OK;

@@ -243,3 +243,30 @@ def test_one_channel_operand_with_many_channels_on_the_other_side(cabi):
     torch.cuda.synchronize()
     O.check_fwd([U.host(a) for a in drs], "n 96")
     O.check_bwd([U.host(a) for a in dxg], [U.host(a) for a in dyg], "n 96")
+
+
+@pytest.mark.parametrize("B,ls,maxl", [(70, range(5), 4), (33, range(7), -1), (5, (1, 3, 6), 9), (130, range(3), -1)])
+def test_cgproduct_of_one_channel_vectors_goes_forward_on_the_diag_kernels(cabi, B, ls, maxl):
+    """One channel in every part of both operands (products of spherical harmonics, say): block channel 0 * 1 + 0, the
+    Diag product of one channel.  Forward it runs on the lane-per-channel kernels, a cell per lane (split at l = 6 when
+    the product reaches higher); the gradients stay with the other families."""
+    xs = [U.seeded(900 + l, B, 2 * l + 1, 1) for l in ls]
+    ys = [U.seeded(950 + l, B, 2 * l + 1, 1) for l in ls]
+    O = U.VecOracle(xs, ys, maxl, False, gseed=990)
+    dxs, dys, dgs = [U.dev(a) for a in xs], [U.dev(a) for a in ys], [U.dev(a) for a in O.gs]
+    drs = [torch.full(p.shape, 7.0 + 1j, dtype=torch.complex64, device="cuda") for p in O.r32]
+    cabi.so3vec_fwd(drs, dxs, dys, accumulate=False)
+    assert cabi.last_path() == DIAG6
+    torch.cuda.synchronize()
+    O.check_fwd([U.host(a) for a in drs], "one channel on both sides, forward")
+    start = [U.seeded(970 + k, *p.shape) for k, p in enumerate(O.r32)]
+    drs2 = [U.dev(a) for a in start]
+    cabi.so3vec_fwd(drs2, dxs, dys, accumulate=True)
+    torch.cuda.synchronize()
+    O.check_fwd_onto([U.host(a) for a in drs2], start, "one channel on both sides, forward onto")
+    dxg = [torch.full(a.shape, 3.0 - 2j, dtype=torch.complex64, device="cuda") for a in xs]
+    dyg = [torch.full(a.shape, 3.0 - 2j, dtype=torch.complex64, device="cuda") for a in ys]
+    cabi.so3vec_bwd(dxg, dyg, dgs, dxs, dys, accumulate=False)
+    assert cabi.last_path() != DIAG6
+    torch.cuda.synchronize()
+    O.check_bwd([U.host(a) for a in dxg], [U.host(a) for a in dyg], "one channel on both sides, backward")

@@ -61,9 +61,11 @@ struct Diag6Args {
 int launch_diag6_fwd_l6(const Diag6Args &a, hipStream_t s);  // product l up to 6
 int launch_diag6_bwd_l6(const Diag6Args &a, hipStream_t s);
 int launch_diag6_bwd_l6_sets(const Diag6Args &a, hipStream_t s);  // every part of y present: fixed sets of l2 per wave
-// operand parts up to l = 4, product up to l = 6 (backward)
-int launch_diag6_bwd_l6_lop4(const Diag6Args &a, hipStream_t s);
-int launch_diag6_bwd_l6_lop4_packed(const Diag6Args &a, hipStream_t s);
+// operand parts up to l = 2, product up to l = 4: a wave per cell and channel group, no barriers
+int launch_diag6_small_fwd(const Diag6Args &a, hipStream_t s);
+int launch_diag6_small_bwd(const Diag6Args &a, hipStream_t s);
+int launch_diag6_small4_bwd(const Diag6Args &a, hipStream_t s);     // backward, operand parts up to l = 4, gradient parts up to l = 6
+int launch_diag6_small4_hi_bwd(const Diag6Args &a, hipStream_t s);  // ... gradient parts l = 7, 8 only
 // product parts l = 7..12 only
 int launch_diag6_fwd_hi(const Diag6Args &a, hipStream_t s);
 int launch_diag6_bwd_hi(const Diag6Args &a, hipStream_t s);

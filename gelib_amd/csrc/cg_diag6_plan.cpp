@@ -20,7 +20,8 @@ std::map<std::pair<int, std::vector<int>>, int *> g_offs;  // (device, offsets) 
 int g_enable = 1;
 int g_l8_enable = 1;    // the kernels for products up to l = 8 of operands up to l = 4: 1 forward, 2 backward too
 int g_sets_enable = 1;  // backward: the kernel with the waves' sets of l2 fixed at compile time, where it applies
-int g_lop4_enable = 1;  // backward: the kernels built for operands up to l = 4 (smaller images in LDS)
+int g_small_enable = 1;  // operands up to l = 2, and backward up to l = 4: the kernels that give a wave, not a block, a cell and
+                         // channel group
 int g_hi_enable = 1;    // the kernels for the part l = 7..12 of a product by itself
 int g_one_channel = 1;  // CGproduct with a one-channel operand runs here as the Diag product with the channel repeated
 
@@ -207,7 +208,8 @@ int diag6_vec_fwd(const VecPlan &plan, const std::vector<const gelib_part_desc *
   const bool l8 = lcap > kL6 && !hi;
   if (l8 && !(lcap <= 8 && operands_up_to(a, 4) && g_l8_enable)) return GELIB_HIP_OK;
   a.accumulate = accumulate ? 1 : 0;
-  if (hi) rc = a.lg_npad < 6 ? launch_diag6_fwd_hi_packed(a, s) : launch_diag6_fwd_hi(a, s);
+  if (g_small_enable && lcap <= 4 && operands_up_to(a, 2)) rc = launch_diag6_small_fwd(a, s);
+  else if (hi) rc = a.lg_npad < 6 ? launch_diag6_fwd_hi_packed(a, s) : launch_diag6_fwd_hi(a, s);
   else if (l8) rc = a.lg_npad < 6 ? launch_diag6_fwd_l8_packed(a, s) : launch_diag6_fwd_l8(a, s);
   else rc = a.lg_npad < 6 ? launch_diag6_fwd_l6_packed(a, s) : launch_diag6_fwd_l6(a, s);
   if (rc) return rc;
@@ -237,9 +239,11 @@ int diag6_vec_bwd(const VecPlan &plan, const std::vector<const gelib_part_desc *
   a.want_y = yg.empty() ? 0 : 1;
   bool all_y = true;
   for (int l = 0; l < kNP; l++) all_y = all_y && a.y[l].ptr != nullptr;
-  if (hi) rc = a.lg_npad < 6 ? launch_diag6_bwd_hi_packed(a, s) : launch_diag6_bwd_hi(a, s);
+  if (g_small_enable && lcap <= 4 && operands_up_to(a, 2)) rc = launch_diag6_small_bwd(a, s);
+  else if (g_small_enable && hi && lcap <= 8 && operands_up_to(a, 4)) rc = launch_diag6_small4_hi_bwd(a, s);
+  else if (g_small_enable && lcap <= 6 && operands_up_to(a, 4)) rc = launch_diag6_small4_bwd(a, s);
+  else if (hi) rc = a.lg_npad < 6 ? launch_diag6_bwd_hi_packed(a, s) : launch_diag6_bwd_hi(a, s);
   else if (l8) rc = a.lg_npad < 6 ? launch_diag6_bwd_l8_packed(a, s) : launch_diag6_bwd_l8(a, s);
-  else if (g_lop4_enable && operands_up_to(a, 4)) rc = a.lg_npad < 6 ? launch_diag6_bwd_l6_lop4_packed(a, s) : launch_diag6_bwd_l6_lop4(a, s);
   else if (a.lg_npad < 6) rc = launch_diag6_bwd_l6_packed(a, s);
   else if (all_y && g_sets_enable) rc = launch_diag6_bwd_l6_sets(a, s);
   else rc = launch_diag6_bwd_l6(a, s);
@@ -276,8 +280,8 @@ int diag6_set_option(const char *name, int value) {
     g_enable = value;
     return GELIB_HIP_OK;
   }
-  if (!std::strcmp(name, "diag6_lop4")) {
-    g_lop4_enable = value;
+  if (!std::strcmp(name, "diag6_small")) {
+    g_small_enable = value;
     return GELIB_HIP_OK;
   }
   if (!std::strcmp(name, "diag6_hi")) {

@@ -308,8 +308,8 @@ int gelib_hip_set_stream_workspace(void *stream, void *ptr, uint64_t bytes);
  * backward kernel built for calls with one triple), "diag6_sets" (1/0: the Diag backward kernel with compile-time sets of
  * l2 per wave), "diag6_l8" (0: Diag products above l = 6 are always split at l = 6; 1: operands up to l = 4 run forward in
  * one launch of the kernels built for products up to l = 8; 2: backward too), "diag6_hi" (1/0: the part l = 7..12 of a
- * split Diag product runs on the lane-per-channel kernels built for it), "diag6_lop4" (1/0: Diag backward kernels built
- * for operands up to l = 4), "diag6_one_channel" (1/0: a CGproduct in which every part of exactly one operand has one
+ * split Diag product runs on the lane-per-channel kernels built for it), "diag6_small" (1/0: Diag kernels that give a wave, not a
+ * block, a cell and channel group: operands up to l = 2, backward up to l = 4), "diag6_one_channel" (1/0: a CGproduct in which every part of exactly one operand has one
  * channel runs on the lane-per-channel Diag kernels), "unrolled_bwd_one_wide" (1/0: the wave-per-cell backward kernel
  * for calls with one triple and 16 or 32 channels in the second operand) and "unrolled_bwd_one_wide_cells" (cells from
  * which it is used, 4096), "unrolled_bwd_split" (1/0: launches with few cells deal a cell's pairs to several blocks),

@@ -42,6 +42,12 @@ CASES = [
     (5, {1: 32, 6: 32}, {6: 32}, 5),                                   # exactly half a wave per cell
     (3, {1: 64, 4: 64}, {l: 64 for l in range(7)}, 6),                 # every part of y, parts of x missing
     (2, {l: 64 for l in range(7)}, {l: 64 for l in range(7)}, 3),      # every part of y, product capped low
+    # operands up to l = 2 (and backward up to l = 4): a wave, not a block, per cell and channel group
+    (70, {0: 5, 1: 5}, {0: 5, 1: 5}, -1),                              # eight cells per wave, three lanes of each idle
+    (9, {l: 96 for l in range(3)}, {l: 96 for l in range(3)}, -1),     # two channel groups, product up to l = 4
+    (33, {1: 64}, {0: 64, 2: 64}, 2),                                  # parts missing, capped
+    (6, {l: 64 for l in range(5)}, {l: 64 for l in range(5)}, 4),      # operands up to l = 4, one cell per wave
+    (7, {2: 40, 4: 40}, {1: 40, 3: 40}, 6),                            # ... parts missing, product up to l = 6
 ]
 
 
@@ -176,6 +182,8 @@ ONE_CHANNEL = [
     (70, 5, [3, 4], [2], 6, "x"),                # eight cells per wave, three lanes of each idle
     (5, 64, range(7), range(7), 6, "y"),         # every part of y: the kernel with fixed sets of l2 per wave
     (3, 16, range(5), range(5), -1, "y"),        # product up to l = 8: split at l = 6 (or the l <= 8 kernels forward)
+    (37, 16, range(3), range(2), -1, "y"),       # wide parts up to l = 2: the kernels that give a wave a cell
+    (9, 64, range(3), range(3), 4, "x"),
 ]
 
 
